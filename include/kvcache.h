@@ -1,0 +1,232 @@
+/*
+ * kvcache.h -- C ABI of libkvcache, the MI355X (gfx950) paged KV-cache
+ * data-movement library: slot-mapped K/V write, block copy, and block
+ * gather/scatter between the HBM pool and a pinned host pool.
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes only; `stream` arguments are hipStream_t passed
+ *     as void* (NULL = the null stream);
+ *   - returns KVC_OK (0) or a negative kvc_status; never throws; the text of the
+ *     last failure on the calling thread is kvc_last_error_string();
+ *   - asynchronous on the given stream(s) unless the name ends in _sync;
+ *   - never allocates or frees device memory; the caller owns every buffer;
+ *   - every offset is computed in 64 bits (one layer of a 65536-block Llama-3-8B
+ *     pool already holds 2^31 elements);
+ *   - block ids / slots outside [0, capacity) are skipped by the kernels
+ *     (the reference leaves them undefined), host-resident id lists are
+ *     rejected with KVC_ERR_OUT_OF_RANGE before anything is launched.
+ *
+ * Pool layout (runtime/worker/llm_worker/model_worker.py:221-228):
+ *   kv_caches[L, num_blocks, 2, block_size, H, D], contiguous; kv_caches[l] is
+ *   the per-layer "NHD" paged cache handed to attention.
+ * Host pool layout (runtime/worker/llm_worker/kv_worker.py:123-127):
+ *   host[num_host_blocks, L, 2*block_size*H*D], C order, pinned.
+ */
+#ifndef KVCACHE_H_
+#define KVCACHE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KVC_ABI_VERSION 1
+
+typedef enum kvc_status {
+  KVC_OK = 0,
+  KVC_ERR_INVALID_ARG = -1,   /* null pointer, negative size, bad stride ...   */
+  KVC_ERR_UNSUPPORTED = -2,   /* elem_bytes / index width not supported        */
+  KVC_ERR_OUT_OF_RANGE = -3,  /* a host-resident block id is outside its pool  */
+  KVC_ERR_STAGING = -4,       /* staging buffer too small for the request      */
+  KVC_ERR_HIP = -5            /* a HIP runtime call failed (see error string)  */
+} kvc_status;
+
+/* how kvc_swap_out / kvc_swap_in move the bytes over PCIe */
+typedef enum kvc_swap_mode {
+  KVC_SWAP_STAGED = 0, /* gather/scatter kernel <-> device staging ring, large
+                          hipMemcpyAsync extents on the copy stream, overlapped */
+  KVC_SWAP_DIRECT = 1  /* one kernel that loads/stores the pinned host pool
+                          through its device mapping (no staging traffic)       */
+} kvc_swap_mode;
+
+int kvc_abi_version(void);
+const char* kvc_last_error_string(void);
+
+/* Launch-shape knobs for measurement sweeps; process-wide, not thread-safe
+ * against concurrent launches. No counterpart in the reference. Keys:
+ * "copy_unroll" (1,2,4,8,16), "copy_nt" (0/1), "copy_max_wgs" (0 = one
+ * workgroup per chunk), "write_vpt" (0 = by size, 1, 2, 4), "write_nt" (0/1),
+ * "direct_max_wgs". Unknown key: KVC_ERR_INVALID_ARG. */
+int kvc_set_tuning(const char* key, int value);
+
+/* ---------------------------------------------------------------------------
+ * K/V write, slot-mapped.
+ * Replaces fill_key_cache / fill_key_cache_kernel
+ *   (runtime/worker/llm_worker/ops/cache_ops.py:39-59,
+ *    runtime/worker/llm_worker/ops/triton/cache_kernels.py:39-58).
+ * For token i: s = slot_mapping[i]; the row of row_elems elements at
+ *   key + i*key_token_stride is copied to
+ *   key_cache + (s / block_size)*cache_block_stride + (s % block_size)*cache_slot_stride,
+ * likewise value -> value_cache. All strides are in ELEMENTS of elem_bytes.
+ * The reference's packed caches [num_slots, H, D] are
+ *   cache_block_stride = block_size*H*D, cache_slot_stride = H*D;
+ * one layer of the interleaved pool [nb, 2, bs, H, D] is
+ *   value_cache = key_cache + bs*H*D, cache_block_stride = 2*bs*H*D.
+ * slot_mapping lives on the device, slot_bytes is 4 (int32) or 8 (int64).
+ * A slot < 0 or >= num_cache_blocks*block_size is skipped.
+ * ------------------------------------------------------------------------- */
+int kvc_reshape_and_cache(const void* key, const void* value,
+                          void* key_cache, void* value_cache,
+                          const void* slot_mapping, int slot_bytes,
+                          int64_t num_tokens, int64_t row_elems,
+                          int64_t key_token_stride, int64_t value_token_stride,
+                          int64_t block_size, int64_t cache_block_stride,
+                          int64_t cache_slot_stride, int64_t num_cache_blocks,
+                          int elem_bytes, void* stream);
+
+/* Same write for num_layers layers in ONE launch: layer l reads
+ * key + l*key_layer_stride (value likewise) and writes the caches at
+ * + l*cache_layer_stride; every layer uses the same slot_mapping, as the
+ * reference's block tables are shared by all layers
+ * (runtime/worker/llm_worker/model_worker.py:399-423 builds them once per step).
+ * No counterpart launch exists in the reference, which writes one layer per
+ * attention call (runtime/worker/llm_worker/models/layers/attention.py:76-85). */
+int kvc_reshape_and_cache_layers(const void* key, const void* value,
+                                 void* key_cache, void* value_cache,
+                                 const void* slot_mapping, int slot_bytes,
+                                 int64_t num_tokens, int64_t row_elems,
+                                 int64_t key_token_stride, int64_t value_token_stride,
+                                 int64_t block_size, int64_t cache_block_stride,
+                                 int64_t cache_slot_stride, int64_t num_cache_blocks,
+                                 int64_t num_layers, int64_t key_layer_stride,
+                                 int64_t value_layer_stride, int64_t cache_layer_stride,
+                                 int elem_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * K/V write, page-table addressed (the reference's live write).
+ * Replaces the flashinfer.append_paged_kv_cache call at
+ *   runtime/worker/llm_worker/models/layers/attention.py:76-85
+ * (flashinfer-python 0.3.1.post1, "NHD" single-tensor cache
+ *  [num_pages, 2, page_size, H, D], runtime/worker/llm_worker/model_worker.py:65-66).
+ * For token i: b = batch_indices[i], p = positions[i],
+ *   page = kv_indices[kv_indptr[b] + p / page_size], e = p % page_size,
+ *   paged_kv_cache[page, 0, e] = append_key[i], paged_kv_cache[page, 1, e] = append_value[i].
+ * Index arrays are int32 on the device. kv_last_page_len is accepted for
+ * signature parity and not read (flashinfer does not read it either).
+ * page_stride is the distance between pages in elements (2*page_size*H*D when
+ * contiguous). b outside [0, batch_size), a page-table index outside
+ * [0, num_kv_indices) or a page outside [0, num_pages) skips the token.
+ * The _layers form adds the layer loop exactly as kvc_reshape_and_cache_layers.
+ * ------------------------------------------------------------------------- */
+int kvc_append_paged_kv_cache(const void* append_key, const void* append_value,
+                              const int32_t* batch_indices, const int32_t* positions,
+                              void* paged_kv_cache,
+                              const int32_t* kv_indices, const int32_t* kv_indptr,
+                              const int32_t* kv_last_page_len,
+                              int64_t nnz, int64_t batch_size, int64_t num_kv_indices,
+                              int64_t num_kv_heads, int64_t head_dim, int64_t page_size,
+                              int64_t key_token_stride, int64_t value_token_stride,
+                              int64_t page_stride, int64_t num_pages,
+                              int elem_bytes, void* stream);
+
+int kvc_append_paged_kv_cache_layers(const void* append_key, const void* append_value,
+                                     const int32_t* batch_indices, const int32_t* positions,
+                                     void* paged_kv_cache,
+                                     const int32_t* kv_indices, const int32_t* kv_indptr,
+                                     const int32_t* kv_last_page_len,
+                                     int64_t nnz, int64_t batch_size, int64_t num_kv_indices,
+                                     int64_t num_kv_heads, int64_t head_dim, int64_t page_size,
+                                     int64_t key_token_stride, int64_t value_token_stride,
+                                     int64_t page_stride, int64_t num_pages,
+                                     int64_t num_layers, int64_t key_layer_stride,
+                                     int64_t value_layer_stride, int64_t cache_layer_stride,
+                                     int elem_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Index preparation for the paged write.
+ * Replace the flashinfer.get_seq_lens / flashinfer.get_batch_indices_positions
+ * calls at runtime/worker/llm_worker/model_worker.py:425-433.
+ *   seq_lens[b] = max(kv_indptr[b+1]-kv_indptr[b]-1, 0)*page_size + kv_last_page_len[b]
+ *   for j in [append_indptr[b], append_indptr[b+1]):
+ *     batch_indices[j] = b
+ *     positions[j]     = seq_lens[b] - (append_indptr[b+1]-append_indptr[b]) + (j - append_indptr[b])
+ * Entries of the outputs at j >= append_indptr[batch_size] (up to nnz) are left
+ * untouched. All arrays int32 on the device.
+ * ------------------------------------------------------------------------- */
+int kvc_get_seq_lens(const int32_t* kv_indptr, const int32_t* kv_last_page_len,
+                     int64_t batch_size, int64_t page_size, int32_t* seq_lens,
+                     void* stream);
+
+int kvc_get_batch_indices_positions(const int32_t* append_indptr, const int32_t* seq_lens,
+                                    int64_t batch_size, int64_t nnz,
+                                    int32_t* batch_indices, int32_t* positions,
+                                    void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Block copy inside the pool (prefix-sharing copy-on-write).
+ * Replaces copy_blocks / copy_blocks_kernel
+ *   (runtime/worker/llm_worker/ops/cache_ops.py:8-36,
+ *    runtime/worker/llm_worker/ops/triton/cache_kernels.py:5-36).
+ * block_maps is the device array [src0, dst0, src1, dst1, ...] of int64 that the
+ * reference wrapper builds; for every layer l and pair j
+ *   kv_caches[l, dst_j, :] = kv_caches[l, src_j, :]   (block_bytes bytes each).
+ * layer_stride_bytes = num_blocks*block_bytes for the contiguous pool.
+ * Defined when the dsts are distinct and no dst is also a src (the reference
+ * gives no ordering between pairs); src == dst is a no-op.
+ * ------------------------------------------------------------------------- */
+int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pairs,
+                    int64_t num_layers, int64_t layer_stride_bytes,
+                    int64_t block_bytes, int64_t num_blocks, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Swap between the HBM pool and the pinned host pool.
+ * Replace the per-(layer, block) memcpy loops
+ *   _save_layer_kv_blocks_to_host  (runtime/worker/llm_worker/kv_worker.py:213-227)
+ *   _load_layer_kv_blocks_from_host (runtime/worker/llm_worker/kv_worker.py:197-211)
+ * and their layer loops (kv_worker.py:249-295).
+ *   swap_out: host[dst_ids[i], l, :] = pool[l, src_ids[i], :]
+ *   swap_in : pool[l, dst_ids[i], :] = host[src_ids[i], l, :]
+ * for i in [0, n) and l in [layer_begin, layer_end) -- the layer range keeps the
+ * reference's layer-pipelined protocol expressible (one call per finished layer
+ * or one call for all).
+ * src_ids / dst_ids are HOST arrays of int64 (they arrive as BlockMapping
+ * entries over gRPC, proto/worker.proto:78-85) and are range-checked here.
+ * host_pool must be pinned memory that the device can address (kvc_host_alloc_pinned).
+ * staging is a device buffer of staging_bytes >= kvc_swap_staging_bytes(...):
+ * its head holds the device copy of the id lists, the rest is the two-slot
+ * ring used by KVC_SWAP_STAGED. Kernels run on kernel_stream, PCIe copies on
+ * copy_stream (may equal kernel_stream: then nothing overlaps). On return all
+ * work is enqueued and kernel_stream has been made to wait for copy_stream's
+ * part, so synchronising kernel_stream alone completes the swap.
+ * ------------------------------------------------------------------------- */
+int64_t kvc_swap_staging_bytes(int64_t n, int64_t num_layers_in_range,
+                               int64_t block_bytes, int mode, int64_t chunk_blocks);
+
+int kvc_swap_out(const void* pool, void* host_pool,
+                 const int64_t* src_ids, const int64_t* dst_ids, int64_t n,
+                 int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                 int64_t num_gpu_blocks, int64_t num_host_blocks,
+                 int64_t layer_begin, int64_t layer_end,
+                 void* staging, int64_t staging_bytes, int mode,
+                 void* kernel_stream, void* copy_stream);
+
+int kvc_swap_in(void* pool, const void* host_pool,
+                const int64_t* src_ids, const int64_t* dst_ids, int64_t n,
+                int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                int64_t num_gpu_blocks, int64_t num_host_blocks,
+                int64_t layer_begin, int64_t layer_end,
+                void* staging, int64_t staging_bytes, int mode,
+                void* kernel_stream, void* copy_stream);
+
+/* Pinned, device-addressable host memory for the host pool; replaces
+ * pycuda.driver.pagelocked_empty (runtime/worker/llm_worker/kv_worker.py:123-127).
+ * Returns NULL on failure. */
+void* kvc_host_alloc_pinned(size_t bytes);
+int kvc_host_free_pinned(void* ptr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVCACHE_H_ */

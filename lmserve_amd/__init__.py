@@ -1,0 +1,28 @@
+"""MI355X-native paged KV-cache data movement behind LMServe's operator surface.
+
+    cache_ops   copy_blocks, fill_key_cache, reshape_and_cache(_layers)
+    paged       append_paged_kv_cache(_layers), get_seq_lens, get_batch_indices_positions
+    kv_worker   KVWorker (GPU <-> pinned host swap), Device, BlockMapping
+    index_prep  host-side block-table / slot-mapping construction
+
+Every operator runs a hand-written HIP kernel from libkvcache.so through the
+C ABI of include/kvcache.h; nothing here computes on the CPU.
+"""
+from . import _lib
+from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_block_maps,
+                        reshape_and_cache, reshape_and_cache_layers)
+from .index_prep import InferInput, KVIndexInputs, make_kv_index_inputs, to_device
+from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
+                        flatten_block_mappings)
+from .paged import (append_paged_kv_cache, append_paged_kv_cache_layers,
+                    get_batch_indices_positions, get_seq_lens)
+
+__all__ = [
+    "copy_blocks", "fill_key_cache", "reshape_and_cache", "reshape_and_cache_layers",
+    "flatten_block_maps", "check_block_maps",
+    "append_paged_kv_cache", "append_paged_kv_cache_layers", "get_seq_lens",
+    "get_batch_indices_positions",
+    "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",
+    "flatten_block_mappings",
+    "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device",
+]

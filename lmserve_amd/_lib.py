@@ -1,0 +1,100 @@
+"""ctypes binding of libkvcache.so (the C ABI in include/kvcache.h).
+
+There is no fallback: if the library is missing, `lib()` raises. Every
+operator in this package goes through the handles defined here.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from typing import Optional
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libkvcache.so")
+
+KVC_OK = 0
+KVC_ERR_INVALID_ARG = -1
+KVC_ERR_UNSUPPORTED = -2
+KVC_ERR_OUT_OF_RANGE = -3
+KVC_ERR_STAGING = -4
+KVC_ERR_HIP = -5
+
+KVC_SWAP_STAGED = 0
+KVC_SWAP_DIRECT = 1
+
+_I64 = c_int64
+_P = c_void_p
+
+# name -> (restype, argtypes); mirrors include/kvcache.h declaration by declaration
+SIGNATURES = {
+    "kvc_abi_version": (c_int, []),
+    "kvc_last_error_string": (c_char_p, []),
+    "kvc_set_tuning": (c_int, [c_char_p, c_int]),
+    "kvc_reshape_and_cache": (c_int, [_P, _P, _P, _P, _P, c_int, _I64, _I64, _I64, _I64, _I64,
+                                      _I64, _I64, _I64, c_int, _P]),
+    "kvc_reshape_and_cache_layers": (c_int, [_P, _P, _P, _P, _P, c_int, _I64, _I64, _I64, _I64,
+                                             _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                             c_int, _P]),
+    "kvc_append_paged_kv_cache": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64,
+                                          _I64, _I64, _I64, _I64, _I64, _I64, c_int, _P]),
+    "kvc_append_paged_kv_cache_layers": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64,
+                                                 _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                                 _I64, _I64, _I64, c_int, _P]),
+    "kvc_get_seq_lens": (c_int, [_P, _P, _I64, _I64, _P, _P]),
+    "kvc_get_batch_indices_positions": (c_int, [_P, _P, _I64, _I64, _P, _P, _P]),
+    "kvc_copy_blocks": (c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _P]),
+    "kvc_swap_staging_bytes": (_I64, [_I64, _I64, _I64, c_int, _I64]),
+    "kvc_swap_out": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
+                             _I64, c_int, _P, _P]),
+    "kvc_swap_in": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
+                            _I64, c_int, _P, _P]),
+    "kvc_host_alloc_pinned": (_P, [c_size_t]),
+    "kvc_host_free_pinned": (c_int, [_P]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+class KVCacheLibraryError(RuntimeError):
+    """libkvcache.so is missing, or a HIP runtime call inside it failed."""
+
+
+def lib() -> ctypes.CDLL:
+    """Load libkvcache.so once and type its entry points."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise KVCacheLibraryError(
+            f"{LIB_PATH} is not built; run `python -m lmserve_amd.build` (needs hipcc). "
+            "There is no CPU fallback for the KV-cache operators.")
+    handle = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(handle, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = handle
+    return handle
+
+
+def last_error() -> str:
+    return lib().kvc_last_error_string().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    """Turn a kvc_status into the Python exception the reference surface uses."""
+    if rc == KVC_OK:
+        return
+    msg = last_error()
+    if rc == KVC_ERR_UNSUPPORTED:
+        raise TypeError(msg)
+    if rc in (KVC_ERR_INVALID_ARG, KVC_ERR_STAGING):
+        raise ValueError(msg)
+    if rc == KVC_ERR_OUT_OF_RANGE:
+        raise IndexError(msg)
+    raise KVCacheLibraryError(msg)
+
+
+def set_tuning(key: str, value: int) -> None:
+    check(lib().kvc_set_tuning(key.encode(), int(value)))

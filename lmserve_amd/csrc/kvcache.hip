@@ -1,0 +1,942 @@
+// libkvcache: paged KV-cache data movement for MI355X (gfx950, CDNA4).
+//
+// Three kernels carry the whole path; all are HBM-bound byte movers, so the
+// design is about coalescing and bytes in flight, not arithmetic:
+//
+//   write_rows_kernel   one 16-byte vector per lane, lanes of a wavefront cover
+//                       consecutive vectors of a token row: the source side is a
+//                       dense stream, the cache side is one contiguous row per
+//                       (token, K|V, layer). blockIdx.y = (layer, K|V) so every
+//                       base pointer is wave-uniform.
+//   copy_tiles_kernel   a "tile" is one block of one layer (block_bytes
+//                       contiguous on both sides). A workgroup owns a chunk of
+//                       256 lanes x UNROLL x 16 bytes, issues all its loads
+//                       before its first store, and walks chunks grid-stride.
+//                       The same kernel serves copy_blocks (pool -> pool), the
+//                       swap gather/scatter (pool <-> staging ring in host
+//                       layout) and the direct swap (pool <-> mapped host pool).
+//   index kernels       seq_lens and (batch_indices, positions) for the paged
+//                       write; a few KiB of int32.
+//
+// The C ABI is declared in include/kvcache.h.
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "kvcache.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// error plumbing
+// ---------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define KVC_HIP(call)                                                          \
+  do {                                                                         \
+    hipError_t e_ = (call);                                                    \
+    if (e_ != hipSuccess)                                                      \
+      return fail(KVC_ERR_HIP, "%s failed: %s (%s:%d)", #call,                 \
+                  hipGetErrorString(e_), __FILE__, __LINE__);                  \
+  } while (0)
+
+// ---------------------------------------------------------------------------
+// tuning knobs (kvc_set_tuning); defaults are the measured best on MI355X
+// ---------------------------------------------------------------------------
+struct Tuning {
+  int copy_unroll = 4;      // 16-byte vectors in flight per lane in copy_tiles
+  int copy_nt = 1;          // non-temporal loads/stores in copy_tiles
+  int copy_max_wgs = 0;     // 0 = one workgroup per chunk, else grid cap
+  int write_vpt = 0;        // vectors per lane in write_rows, 0 = by size
+  int write_nt = 0;         // non-temporal stores in write_rows
+  int direct_max_wgs = 512; // grid cap of the direct (PCIe-bound) swap kernel
+};
+Tuning g_tune;
+
+constexpr int kThreads = 256;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int BYTES> struct VecOf;
+template <> struct VecOf<16> { using type = u32x4; };
+template <> struct VecOf<8> { using type = u32x2; };
+template <> struct VecOf<4> { using type = uint32_t; };
+template <> struct VecOf<2> { using type = uint16_t; };
+template <> struct VecOf<1> { using type = uint8_t; };
+
+template <bool NT, typename V>
+__device__ __forceinline__ V ld(const V* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <bool NT, typename V>
+__device__ __forceinline__ void st(V* p, V v) {
+  if constexpr (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
+// ---------------------------------------------------------------------------
+// write_rows_kernel
+// ---------------------------------------------------------------------------
+struct WriteArgs {
+  const char* key;
+  const char* value;
+  char* key_cache;
+  char* value_cache;
+  // slot-mapped addressing
+  const void* slot_mapping;
+  int slot_bytes;
+  // page-table addressing (used when batch_indices != nullptr)
+  const int32_t* batch_indices;
+  const int32_t* positions;
+  const int32_t* kv_indices;
+  const int32_t* kv_indptr;
+  int64_t batch_size;
+  int64_t num_kv_indices;
+  // geometry; every stride in BYTES
+  uint32_t num_tokens;     // tokens of this launch (host splits huge T)
+  uint32_t vecs_per_row;
+  int vpr_shift;           // log2(vecs_per_row) or -1
+  int64_t key_token_stride, value_token_stride;
+  int64_t key_layer_stride, value_layer_stride;
+  int64_t block_size;
+  int bs_shift;            // log2(block_size) or -1
+  int64_t cache_block_stride, cache_slot_stride, cache_layer_stride;
+  int64_t num_cache_blocks;
+};
+
+template <int VEC, int VPT, bool PAGED, bool NT>
+__global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
+  using V = typename VecOf<VEC>::type;
+  const uint32_t layer = blockIdx.y >> 1;
+  const uint32_t is_v = blockIdx.y & 1u;
+  const char* src_base = (is_v ? a.value + (int64_t)layer * a.value_layer_stride
+                               : a.key + (int64_t)layer * a.key_layer_stride);
+  char* dst_base = (is_v ? a.value_cache : a.key_cache) + (int64_t)layer * a.cache_layer_stride;
+  const int64_t tok_stride = is_v ? a.value_token_stride : a.key_token_stride;
+  const uint32_t total = a.num_tokens * a.vecs_per_row;  // host guarantees < 2^31
+
+  V data[VPT];
+  char* dst[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const uint32_t g = (blockIdx.x * VPT + j) * kThreads + threadIdx.x;
+    dst[j] = nullptr;
+    if (g >= total) continue;
+    uint32_t t, vec;
+    if (a.vpr_shift >= 0) {
+      t = g >> a.vpr_shift;
+      vec = g & (a.vecs_per_row - 1u);
+    } else {
+      t = g / a.vecs_per_row;
+      vec = g - t * a.vecs_per_row;
+    }
+    int64_t blk, off;
+    if constexpr (PAGED) {
+      const int64_t b = a.batch_indices[t];
+      const int64_t p = a.positions[t];
+      if (b < 0 || b >= a.batch_size || p < 0) continue;
+      int64_t pg, e;
+      if (a.bs_shift >= 0) {
+        pg = p >> a.bs_shift;
+        e = p & (a.block_size - 1);
+      } else {
+        pg = p / a.block_size;
+        e = p - pg * a.block_size;
+      }
+      const int64_t it = (int64_t)a.kv_indptr[b] + pg;
+      if (it < 0 || it >= a.num_kv_indices) continue;
+      blk = a.kv_indices[it];
+      off = e;
+    } else {
+      const int64_t s = (a.slot_bytes == 8)
+                            ? reinterpret_cast<const int64_t*>(a.slot_mapping)[t]
+                            : (int64_t) reinterpret_cast<const int32_t*>(a.slot_mapping)[t];
+      if (s < 0) continue;
+      if (a.bs_shift >= 0) {
+        blk = s >> a.bs_shift;
+        off = s & (a.block_size - 1);
+      } else {
+        blk = s / a.block_size;
+        off = s - blk * a.block_size;
+      }
+    }
+    if (blk < 0 || blk >= a.num_cache_blocks) continue;
+    data[j] = *reinterpret_cast<const V*>(src_base + (int64_t)t * tok_stride + (int64_t)vec * VEC);
+    dst[j] = dst_base + blk * a.cache_block_stride + off * a.cache_slot_stride + (int64_t)vec * VEC;
+  }
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    if (dst[j]) st<NT>(reinterpret_cast<V*>(dst[j]), data[j]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// copy_tiles_kernel
+// ---------------------------------------------------------------------------
+struct TileArgs {
+  const char* src_base;
+  char* dst_base;
+  const int64_t* src_ids;  // device; nullptr = identity (i)
+  const int64_t* dst_ids;  // device; nullptr = identity (i)
+  int id_stride;           // 1, or 2 for the interleaved [src,dst,...] pair list
+  int64_t src_layer_stride, src_block_stride;
+  int64_t dst_layer_stride, dst_block_stride;
+  int64_t num_src_blocks, num_dst_blocks;  // bounds for the id lists
+  int64_t tile_bytes;
+  uint32_t chunks_per_tile;
+  uint32_t num_layers;
+  uint64_t total_chunks;   // n * num_layers * chunks_per_tile
+};
+
+template <int VEC, int UNROLL, bool NT>
+__global__ __launch_bounds__(kThreads) void copy_tiles_kernel(TileArgs a) {
+  using V = typename VecOf<VEC>::type;
+  constexpr int64_t kChunk = (int64_t)kThreads * UNROLL * VEC;
+  for (uint64_t w = blockIdx.x; w < a.total_chunks; w += gridDim.x) {
+    // chunk fastest, then layer, then block: neighbouring workgroups stream
+    // neighbouring addresses of one tile
+    uint32_t chunk, layer;
+    int64_t i;
+    if (a.total_chunks <= 0xffffffffull) {  // 32-bit divisions when they suffice
+      const uint32_t w32 = (uint32_t)w;
+      const uint32_t tile = w32 / a.chunks_per_tile;
+      chunk = w32 - tile * a.chunks_per_tile;
+      const uint32_t blk = tile / a.num_layers;
+      layer = tile - blk * a.num_layers;
+      i = blk;
+    } else {
+      chunk = (uint32_t)(w % a.chunks_per_tile);
+      const uint64_t tile = w / a.chunks_per_tile;
+      layer = (uint32_t)(tile % a.num_layers);
+      i = (int64_t)(tile / a.num_layers);
+    }
+    const int64_t sid = a.src_ids ? a.src_ids[i * a.id_stride] : i;
+    const int64_t did = a.dst_ids ? a.dst_ids[i * a.id_stride] : i;
+    if (sid < 0 || sid >= a.num_src_blocks || did < 0 || did >= a.num_dst_blocks) continue;
+    const char* src = a.src_base + layer * a.src_layer_stride + sid * a.src_block_stride;
+    char* dst = a.dst_base + layer * a.dst_layer_stride + did * a.dst_block_stride;
+    if (src == dst) continue;
+    const int64_t base = chunk * kChunk + (int64_t)threadIdx.x * VEC;
+    V data[UNROLL];
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+      const int64_t off = base + (int64_t)j * kThreads * VEC;
+      if (off < a.tile_bytes) data[j] = ld<NT>(reinterpret_cast<const V*>(src + off));
+    }
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+      const int64_t off = base + (int64_t)j * kThreads * VEC;
+      if (off < a.tile_bytes) st<NT>(reinterpret_cast<V*>(dst + off), data[j]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// index kernels
+// ---------------------------------------------------------------------------
+__global__ void seq_lens_kernel(const int32_t* kv_indptr, const int32_t* last_page_len,
+                                int64_t batch_size, int32_t page_size, int32_t* seq_lens) {
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch_size) return;
+  int32_t pages = kv_indptr[b + 1] - kv_indptr[b] - 1;
+  if (pages < 0) pages = 0;
+  seq_lens[b] = pages * page_size + last_page_len[b];
+}
+
+__global__ void batch_indices_positions_kernel(const int32_t* append_indptr,
+                                               const int32_t* seq_lens, int64_t nnz,
+                                               int32_t* batch_indices, int32_t* positions) {
+  const int32_t b = blockIdx.x;
+  const int32_t begin = append_indptr[b];
+  const int32_t end = append_indptr[b + 1];
+  const int32_t first_pos = seq_lens[b] - (end - begin);
+  for (int32_t j = begin + (int32_t)threadIdx.x; j < end; j += blockDim.x) {
+    if (j < 0 || j >= nnz) continue;
+    batch_indices[j] = b;
+    positions[j] = first_pos + (j - begin);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host helpers
+// ---------------------------------------------------------------------------
+inline int log2_exact(int64_t x) {
+  if (x <= 0 || (x & (x - 1))) return -1;
+  int s = 0;
+  while ((int64_t(1) << s) < x) ++s;
+  return s;
+}
+
+// widest vector (bytes) that divides every value given (addresses and strides)
+inline int common_vec(std::initializer_list<uint64_t> vals) {
+  uint64_t acc = 16;
+  for (uint64_t v : vals) {
+    while (acc > 1 && (v % acc)) acc >>= 1;
+  }
+  return (int)acc;
+}
+
+template <int VEC, int VPT, bool PAGED>
+void launch_write_nt(const WriteArgs& a, dim3 grid, hipStream_t s, bool nt) {
+  if (nt) hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, true>), grid, dim3(kThreads), 0, s, a);
+  else hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, false>), grid, dim3(kThreads), 0, s, a);
+}
+
+template <int VEC, bool PAGED>
+void launch_write_vpt(const WriteArgs& a, int vpt, uint32_t layers2, hipStream_t s, bool nt) {
+  const uint64_t total = (uint64_t)a.num_tokens * a.vecs_per_row;
+  auto grid = [&](int v) {
+    return dim3((unsigned)((total + (uint64_t)kThreads * v - 1) / ((uint64_t)kThreads * v)), layers2, 1);
+  };
+  switch (vpt) {
+    case 1: launch_write_nt<VEC, 1, PAGED>(a, grid(1), s, nt); break;
+    case 2: launch_write_nt<VEC, 2, PAGED>(a, grid(2), s, nt); break;
+    default: launch_write_nt<VEC, 4, PAGED>(a, grid(4), s, nt); break;
+  }
+}
+
+template <bool PAGED>
+void launch_write(const WriteArgs& a, int vec, int vpt, uint32_t layers2, hipStream_t s, bool nt) {
+  switch (vec) {
+    case 16: launch_write_vpt<16, PAGED>(a, vpt, layers2, s, nt); break;
+    case 8: launch_write_vpt<8, PAGED>(a, vpt, layers2, s, nt); break;
+    case 4: launch_write_vpt<4, PAGED>(a, vpt, layers2, s, nt); break;
+    case 2: launch_write_vpt<2, PAGED>(a, vpt, layers2, s, nt); break;
+    default: launch_write_vpt<1, PAGED>(a, vpt, layers2, s, nt); break;
+  }
+}
+
+struct WriteGeom {
+  int64_t num_tokens, row_elems;
+  int64_t key_token_stride, value_token_stride;       // elements
+  int64_t block_size, cache_block_stride, cache_slot_stride, num_cache_blocks;
+  int64_t num_layers, key_layer_stride, value_layer_stride, cache_layer_stride;
+  int elem_bytes;
+};
+
+int check_write_geom(const char* fn, const void* key, const void* value, const void* kc,
+                     const void* vc, const WriteGeom& g) {
+  if (g.elem_bytes != 1 && g.elem_bytes != 2 && g.elem_bytes != 4 && g.elem_bytes != 8)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: elem_bytes=%d (need 1, 2, 4 or 8)", fn, g.elem_bytes);
+  if (g.num_tokens < 0 || g.row_elems < 0 || g.num_layers < 0)
+    return fail(KVC_ERR_INVALID_ARG, "%s: negative size (tokens=%lld row_elems=%lld layers=%lld)", fn,
+                (long long)g.num_tokens, (long long)g.row_elems, (long long)g.num_layers);
+  if (g.block_size <= 0 || g.num_cache_blocks < 0)
+    return fail(KVC_ERR_INVALID_ARG, "%s: block_size=%lld num_cache_blocks=%lld", fn,
+                (long long)g.block_size, (long long)g.num_cache_blocks);
+  if (g.num_tokens == 0 || g.row_elems == 0 || g.num_layers == 0) return KVC_OK;
+  if (!key || !value || !kc || !vc)
+    return fail(KVC_ERR_INVALID_ARG, "%s: null key/value/cache pointer", fn);
+  if (g.key_token_stride < g.row_elems || g.value_token_stride < g.row_elems)
+    return fail(KVC_ERR_INVALID_ARG, "%s: token stride smaller than the row (%lld/%lld < %lld)", fn,
+                (long long)g.key_token_stride, (long long)g.value_token_stride, (long long)g.row_elems);
+  if (g.cache_slot_stride < g.row_elems || g.cache_block_stride < 0 || g.cache_layer_stride < 0 ||
+      g.key_layer_stride < 0 || g.value_layer_stride < 0)
+    return fail(KVC_ERR_INVALID_ARG, "%s: bad cache/layer stride", fn);
+  if (g.num_layers * 2 > 65535)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: num_layers=%lld exceeds 32767", fn, (long long)g.num_layers);
+  if (g.row_elems * g.elem_bytes > (int64_t(1) << 30))
+    return fail(KVC_ERR_UNSUPPORTED, "%s: row of %lld bytes is beyond 1 GiB", fn,
+                (long long)(g.row_elems * g.elem_bytes));
+  return KVC_OK;
+}
+
+// shared driver of the four write entry points
+int run_write(const char* fn, const void* key, const void* value, void* kc, void* vc,
+              const void* slot_mapping, int slot_bytes, const int32_t* batch_indices,
+              const int32_t* positions, const int32_t* kv_indices, const int32_t* kv_indptr,
+              int64_t batch_size, int64_t num_kv_indices, const WriteGeom& g, void* stream) {
+  int rc = check_write_geom(fn, key, value, kc, vc, g);
+  if (rc != KVC_OK) return rc;
+  if (g.num_tokens == 0 || g.row_elems == 0 || g.num_layers == 0) return KVC_OK;
+  const bool paged = batch_indices != nullptr;
+  if (paged) {
+    if (!positions || !kv_indices || !kv_indptr)
+      return fail(KVC_ERR_INVALID_ARG, "%s: null index array", fn);
+    if (batch_size < 0 || num_kv_indices < 0)
+      return fail(KVC_ERR_INVALID_ARG, "%s: negative batch_size/num_kv_indices", fn);
+  } else {
+    if (!slot_mapping) return fail(KVC_ERR_INVALID_ARG, "%s: null slot_mapping", fn);
+    if (slot_bytes != 4 && slot_bytes != 8)
+      return fail(KVC_ERR_UNSUPPORTED, "%s: slot_bytes=%d (need 4 or 8)", fn, slot_bytes);
+  }
+  const int64_t E = g.elem_bytes;
+  const int vec = common_vec({(uint64_t)(uintptr_t)key, (uint64_t)(uintptr_t)value,
+                              (uint64_t)(uintptr_t)kc, (uint64_t)(uintptr_t)vc,
+                              (uint64_t)(g.row_elems * E), (uint64_t)(g.key_token_stride * E),
+                              (uint64_t)(g.value_token_stride * E),
+                              (uint64_t)(g.key_layer_stride * E), (uint64_t)(g.value_layer_stride * E),
+                              (uint64_t)(g.cache_block_stride * E), (uint64_t)(g.cache_slot_stride * E),
+                              (uint64_t)(g.cache_layer_stride * E)});
+  WriteArgs a{};
+  a.key_cache = (char*)kc;
+  a.value_cache = (char*)vc;
+  a.slot_bytes = slot_bytes;
+  a.batch_indices = batch_indices;
+  a.positions = positions;
+  a.kv_indices = kv_indices;
+  a.kv_indptr = kv_indptr;
+  a.batch_size = batch_size;
+  a.num_kv_indices = num_kv_indices;
+  a.vecs_per_row = (uint32_t)(g.row_elems * E / vec);
+  a.vpr_shift = log2_exact(a.vecs_per_row);
+  a.key_token_stride = g.key_token_stride * E;
+  a.value_token_stride = g.value_token_stride * E;
+  a.key_layer_stride = g.key_layer_stride * E;
+  a.value_layer_stride = g.value_layer_stride * E;
+  a.block_size = g.block_size;
+  a.bs_shift = log2_exact(g.block_size);
+  a.cache_block_stride = g.cache_block_stride * E;
+  a.cache_slot_stride = g.cache_slot_stride * E;
+  a.cache_layer_stride = g.cache_layer_stride * E;
+  a.num_cache_blocks = g.num_cache_blocks;
+
+  // bytes one launch moves decide how many vectors a lane carries: small
+  // launches are latency-bound and want every lane busy with one vector.
+  const int64_t launch_bytes = g.num_tokens * g.row_elems * E * 2 * g.num_layers;
+  int vpt = g_tune.write_vpt;
+  if (vpt <= 0) vpt = launch_bytes >= (int64_t(32) << 20) ? 4 : (launch_bytes >= (int64_t(8) << 20) ? 2 : 1);
+  const bool nt = g_tune.write_nt != 0;
+
+  // keep token*vecs_per_row inside 31 bits per launch
+  const int64_t max_tokens = std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / a.vecs_per_row - 4 * kThreads);
+  for (int64_t t0 = 0; t0 < g.num_tokens; t0 += max_tokens) {
+    const int64_t nt_tok = std::min(max_tokens, g.num_tokens - t0);
+    a.num_tokens = (uint32_t)nt_tok;
+    a.key = (const char*)key + t0 * a.key_token_stride;
+    a.value = (const char*)value + t0 * a.value_token_stride;
+    if (paged) {
+      a.batch_indices = batch_indices + t0;
+      a.positions = positions + t0;
+      launch_write<true>(a, vec, vpt, (uint32_t)(g.num_layers * 2), (hipStream_t)stream, nt);
+    } else {
+      a.slot_mapping = (const char*)slot_mapping + t0 * slot_bytes;
+      launch_write<false>(a, vec, vpt, (uint32_t)(g.num_layers * 2), (hipStream_t)stream, nt);
+    }
+    KVC_HIP(hipGetLastError());
+  }
+  return KVC_OK;
+}
+
+// --------------------------- tile copy launch -------------------------------
+template <int VEC, int UNROLL>
+void launch_tiles_nt(const TileArgs& a, unsigned grid, hipStream_t s, bool nt) {
+  if (nt) hipLaunchKernelGGL((copy_tiles_kernel<VEC, UNROLL, true>), dim3(grid), dim3(kThreads), 0, s, a);
+  else hipLaunchKernelGGL((copy_tiles_kernel<VEC, UNROLL, false>), dim3(grid), dim3(kThreads), 0, s, a);
+}
+
+template <int VEC>
+int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt, int64_t n) {
+  // do not carry more vectors per lane than the tile can fill
+  while (unroll > 1 && (int64_t)kThreads * VEC * (unroll / 2) >= a.tile_bytes) unroll /= 2;
+  const int64_t chunk = (int64_t)kThreads * VEC * unroll;
+  a.chunks_per_tile = (uint32_t)((a.tile_bytes + chunk - 1) / chunk);
+  a.total_chunks = (uint64_t)n * a.num_layers * a.chunks_per_tile;
+  uint64_t grid = a.total_chunks;
+  if (max_wgs > 0) grid = std::min<uint64_t>(grid, (uint64_t)max_wgs);
+  grid = std::min<uint64_t>(grid, 0x7fffffffull);
+  switch (unroll) {
+    case 1: launch_tiles_nt<VEC, 1>(a, (unsigned)grid, s, nt); break;
+    case 2: launch_tiles_nt<VEC, 2>(a, (unsigned)grid, s, nt); break;
+    case 4: launch_tiles_nt<VEC, 4>(a, (unsigned)grid, s, nt); break;
+    case 8: launch_tiles_nt<VEC, 8>(a, (unsigned)grid, s, nt); break;
+    default: launch_tiles_nt<VEC, 16>(a, (unsigned)grid, s, nt); break;
+  }
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+int launch_tiles(const TileArgs& a, int64_t n, int max_wgs, hipStream_t s) {
+  if (n == 0 || a.num_layers == 0 || a.tile_bytes == 0) return KVC_OK;
+  const int vec = common_vec({(uint64_t)(uintptr_t)a.src_base, (uint64_t)(uintptr_t)a.dst_base,
+                              (uint64_t)a.src_layer_stride, (uint64_t)a.src_block_stride,
+                              (uint64_t)a.dst_layer_stride, (uint64_t)a.dst_block_stride,
+                              (uint64_t)a.tile_bytes});
+  int unroll = g_tune.copy_unroll;
+  if (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8 && unroll != 16) unroll = 4;
+  const bool nt = g_tune.copy_nt != 0;
+  switch (vec) {
+    case 16: return launch_tiles_vec<16>(a, unroll, max_wgs, s, nt, n);
+    case 8: return launch_tiles_vec<8>(a, unroll, max_wgs, s, nt, n);
+    case 4: return launch_tiles_vec<4>(a, unroll, max_wgs, s, nt, n);
+    case 2: return launch_tiles_vec<2>(a, unroll, max_wgs, s, nt, n);
+    default: return launch_tiles_vec<1>(a, unroll, max_wgs, s, nt, n);
+  }
+}
+
+// --------------------------- swap plumbing ----------------------------------
+constexpr int64_t kIdAlign = 256;
+inline int64_t round_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+inline int64_t ids_region_bytes(int64_t n) { return round_up(2 * n * (int64_t)sizeof(int64_t), kIdAlign); }
+
+// Per-thread resources of the swap entry points: events that order the two
+// streams, and a pinned bounce buffer from which the id lists are uploaded (the
+// caller's lists may be pageable and may be freed as soon as the call returns).
+struct SwapCtx {
+  hipEvent_t start = nullptr, ids_done = nullptr, tail = nullptr;
+  hipEvent_t filled[2] = {nullptr, nullptr};   // staging slot holds fresh data
+  hipEvent_t drained[2] = {nullptr, nullptr};  // staging slot may be overwritten
+  int64_t* ids_host = nullptr;
+  int64_t ids_cap = 0;
+  bool ids_pending = false;
+  int device = -1;
+};
+thread_local SwapCtx g_swap;
+
+int swap_ctx_prepare(int64_t n) {
+  int dev = 0;
+  KVC_HIP(hipGetDevice(&dev));
+  SwapCtx& c = g_swap;
+  if (c.device != dev) {
+    if (c.device >= 0) {
+      // events belong to the device they were created on: start over
+      if (c.ids_pending) (void)hipEventSynchronize(c.ids_done);
+      c.ids_pending = false;
+      hipEvent_t* evs[] = {&c.start, &c.ids_done, &c.tail, &c.filled[0], &c.filled[1],
+                           &c.drained[0], &c.drained[1]};
+      for (hipEvent_t* e : evs) {
+        if (*e) (void)hipEventDestroy(*e);
+        *e = nullptr;
+      }
+    }
+    hipEvent_t* evs[] = {&c.start, &c.ids_done, &c.tail, &c.filled[0], &c.filled[1],
+                         &c.drained[0], &c.drained[1]};
+    for (hipEvent_t* e : evs) KVC_HIP(hipEventCreateWithFlags(e, hipEventDisableTiming));
+    c.device = dev;
+  }
+  if (c.ids_pending) {
+    KVC_HIP(hipEventSynchronize(c.ids_done));
+    c.ids_pending = false;
+  }
+  if (2 * n > c.ids_cap) {
+    if (c.ids_host) KVC_HIP(hipHostFree(c.ids_host));
+    c.ids_host = nullptr;
+    c.ids_cap = 0;
+    const int64_t cap = std::max<int64_t>(2 * n, 4096);
+    KVC_HIP(hipHostMalloc((void**)&c.ids_host, cap * sizeof(int64_t), hipHostMallocDefault));
+    c.ids_cap = cap;
+  }
+  return KVC_OK;
+}
+
+struct SwapGeom {
+  int64_t n, num_layers, layer_stride_bytes, block_bytes;
+  int64_t num_gpu_blocks, num_host_blocks, layer_begin, layer_end;
+};
+
+int check_swap(const char* fn, const void* pool, const void* host, const int64_t* gpu_ids,
+               const int64_t* host_ids, const SwapGeom& g, const void* staging,
+               int64_t staging_bytes, int mode, int64_t* chunk_blocks) {
+  if (g.n < 0 || g.num_layers < 0 || g.block_bytes < 0 || g.layer_stride_bytes < 0)
+    return fail(KVC_ERR_INVALID_ARG, "%s: negative size", fn);
+  if (g.layer_begin < 0 || g.layer_end < g.layer_begin || g.layer_end > g.num_layers)
+    return fail(KVC_ERR_INVALID_ARG, "%s: layer range [%lld, %lld) outside [0, %lld)", fn,
+                (long long)g.layer_begin, (long long)g.layer_end, (long long)g.num_layers);
+  if (mode != KVC_SWAP_STAGED && mode != KVC_SWAP_DIRECT)
+    return fail(KVC_ERR_INVALID_ARG, "%s: unknown swap mode %d", fn, mode);
+  const int64_t nl = g.layer_end - g.layer_begin;
+  *chunk_blocks = 0;
+  if (g.n == 0 || nl == 0 || g.block_bytes == 0) return KVC_OK;
+  if (!pool || !host || !gpu_ids || !host_ids)
+    return fail(KVC_ERR_INVALID_ARG, "%s: null pool/host/id pointer", fn);
+  if (g.layer_stride_bytes < g.block_bytes)
+    return fail(KVC_ERR_INVALID_ARG, "%s: layer stride smaller than a block", fn);
+  if (nl > 0xffffffffll) return fail(KVC_ERR_UNSUPPORTED, "%s: too many layers", fn);
+  for (int64_t i = 0; i < g.n; ++i) {
+    if (gpu_ids[i] < 0 || gpu_ids[i] >= g.num_gpu_blocks)
+      return fail(KVC_ERR_OUT_OF_RANGE, "%s: gpu block id %lld (entry %lld) outside [0, %lld)", fn,
+                  (long long)gpu_ids[i], (long long)i, (long long)g.num_gpu_blocks);
+    if (host_ids[i] < 0 || host_ids[i] >= g.num_host_blocks)
+      return fail(KVC_ERR_OUT_OF_RANGE, "%s: host block id %lld (entry %lld) outside [0, %lld)", fn,
+                  (long long)host_ids[i], (long long)i, (long long)g.num_host_blocks);
+  }
+  if (!staging) return fail(KVC_ERR_STAGING, "%s: null staging buffer", fn);
+  if ((uintptr_t)staging % kIdAlign)
+    return fail(KVC_ERR_STAGING, "%s: staging buffer must be %lld-byte aligned", fn, (long long)kIdAlign);
+  const int64_t ids_bytes = ids_region_bytes(g.n);
+  if (staging_bytes < ids_bytes)
+    return fail(KVC_ERR_STAGING, "%s: staging of %lld bytes cannot hold the id lists (%lld)", fn,
+                (long long)staging_bytes, (long long)ids_bytes);
+  if (mode == KVC_SWAP_STAGED) {
+    const int64_t per_block = round_up(nl * g.block_bytes, kIdAlign);
+    const int64_t cb = (staging_bytes - ids_bytes) / 2 / per_block;
+    if (cb < 1)
+      return fail(KVC_ERR_STAGING, "%s: staging of %lld bytes holds no ring slot (need >= %lld)", fn,
+                  (long long)staging_bytes, (long long)(ids_bytes + 2 * per_block));
+    *chunk_blocks = std::min(cb, g.n);
+  }
+  return KVC_OK;
+}
+
+// upload [gpu_ids | host_ids] to the head of the staging buffer on `s`
+int upload_ids(const int64_t* gpu_ids, const int64_t* host_ids, int64_t n, void* staging,
+               hipStream_t s) {
+  SwapCtx& c = g_swap;
+  std::memcpy(c.ids_host, gpu_ids, n * sizeof(int64_t));
+  std::memcpy(c.ids_host + n, host_ids, n * sizeof(int64_t));
+  KVC_HIP(hipMemcpyAsync(staging, c.ids_host, 2 * n * sizeof(int64_t), hipMemcpyHostToDevice, s));
+  KVC_HIP(hipEventRecord(c.ids_done, s));
+  c.ids_pending = true;
+  return KVC_OK;
+}
+
+// PCIe leg of one staged chunk: rows of `width` bytes, one per block of the
+// chunk, between the ring slot (dense) and the host pool (row pitch = a whole
+// host block). Runs of consecutive host ids go out as one extent.
+int copy_chunk_rows(char* slot, char* host_pool, const int64_t* host_ids, int64_t count,
+                    int64_t width, int64_t host_block_bytes, int64_t host_row_offset,
+                    bool to_host, hipStream_t s) {
+  int64_t i = 0;
+  while (i < count) {
+    int64_t j = i + 1;
+    while (j < count && host_ids[j] == host_ids[j - 1] + 1) ++j;
+    const int64_t run = j - i;
+    char* h = host_pool + host_ids[i] * host_block_bytes + host_row_offset;
+    char* d = slot + i * width;
+    if (width == host_block_bytes || run == 1) {
+      if (to_host) KVC_HIP(hipMemcpyAsync(h, d, run * width, hipMemcpyDeviceToHost, s));
+      else KVC_HIP(hipMemcpyAsync(d, h, run * width, hipMemcpyHostToDevice, s));
+    } else {
+      if (to_host)
+        KVC_HIP(hipMemcpy2DAsync(h, host_block_bytes, d, width, width, run, hipMemcpyDeviceToHost, s));
+      else
+        KVC_HIP(hipMemcpy2DAsync(d, width, h, host_block_bytes, width, run, hipMemcpyHostToDevice, s));
+    }
+    i = j;
+  }
+  return KVC_OK;
+}
+
+int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_t* gpu_ids,
+             const int64_t* host_ids, const SwapGeom& g, void* staging, int64_t staging_bytes,
+             int mode, void* kernel_stream, void* copy_stream) {
+  int64_t chunk_blocks = 0;
+  int rc = check_swap(fn, pool, host_pool, gpu_ids, host_ids, g, staging, staging_bytes, mode,
+                      &chunk_blocks);
+  if (rc != KVC_OK) return rc;
+  const int64_t nl = g.layer_end - g.layer_begin;
+  if (g.n == 0 || nl == 0 || g.block_bytes == 0) return KVC_OK;
+  rc = swap_ctx_prepare(g.n);
+  if (rc != KVC_OK) return rc;
+  SwapCtx& c = g_swap;
+  hipStream_t ks = (hipStream_t)kernel_stream;
+  hipStream_t cs = (hipStream_t)copy_stream;
+  const bool two_streams = ks != cs;
+
+  rc = upload_ids(gpu_ids, host_ids, g.n, staging, ks);
+  if (rc != KVC_OK) return rc;
+  const int64_t* d_gpu_ids = (const int64_t*)staging;
+  const int64_t* d_host_ids = d_gpu_ids + g.n;
+  const int64_t host_block_bytes = g.num_layers * g.block_bytes;
+  char* pool_l0 = pool + g.layer_begin * g.layer_stride_bytes;
+  const int64_t host_row_offset = g.layer_begin * g.block_bytes;
+
+  TileArgs t{};
+  t.id_stride = 1;
+  t.tile_bytes = g.block_bytes;
+  t.num_layers = (uint32_t)nl;
+
+  if (mode == KVC_SWAP_DIRECT) {
+    // pool <-> mapped host pool in a single kernel
+    if (out) {
+      t.src_base = pool_l0; t.src_ids = d_gpu_ids;
+      t.src_layer_stride = g.layer_stride_bytes; t.src_block_stride = g.block_bytes;
+      t.num_src_blocks = g.num_gpu_blocks;
+      t.dst_base = host_pool + host_row_offset; t.dst_ids = d_host_ids;
+      t.dst_layer_stride = g.block_bytes; t.dst_block_stride = host_block_bytes;
+      t.num_dst_blocks = g.num_host_blocks;
+    } else {
+      t.src_base = host_pool + host_row_offset; t.src_ids = d_host_ids;
+      t.src_layer_stride = g.block_bytes; t.src_block_stride = host_block_bytes;
+      t.num_src_blocks = g.num_host_blocks;
+      t.dst_base = pool_l0; t.dst_ids = d_gpu_ids;
+      t.dst_layer_stride = g.layer_stride_bytes; t.dst_block_stride = g.block_bytes;
+      t.num_dst_blocks = g.num_gpu_blocks;
+    }
+    return launch_tiles(t, g.n, g_tune.direct_max_wgs, ks);
+  }
+
+  // staged: two ring slots, kernel on ks, PCIe extents on cs
+  const int64_t width = nl * g.block_bytes;  // bytes of one block's layer range
+  const int64_t slot_bytes = round_up(width, kIdAlign) * chunk_blocks;
+  char* ring = (char*)staging + ids_region_bytes(g.n);
+  if (two_streams) {
+    KVC_HIP(hipEventRecord(c.start, ks));
+    KVC_HIP(hipStreamWaitEvent(cs, c.start, 0));
+  }
+  int64_t done = 0;
+  for (int64_t k = 0; done < g.n; ++k, done += chunk_blocks) {
+    const int64_t count = std::min(chunk_blocks, g.n - done);
+    const int sl = (int)(k & 1);
+    char* slot = ring + sl * slot_bytes;
+    if (out) {
+      // gather pool blocks -> slot (host layout [count, nl, block]) -> host
+      if (two_streams && k >= 2) KVC_HIP(hipStreamWaitEvent(ks, c.drained[sl], 0));
+      t.src_base = pool_l0; t.src_ids = d_gpu_ids + done;
+      t.src_layer_stride = g.layer_stride_bytes; t.src_block_stride = g.block_bytes;
+      t.num_src_blocks = g.num_gpu_blocks;
+      t.dst_base = slot; t.dst_ids = nullptr;
+      t.dst_layer_stride = g.block_bytes; t.dst_block_stride = width;
+      t.num_dst_blocks = count;
+      rc = launch_tiles(t, count, g_tune.copy_max_wgs, ks);
+      if (rc != KVC_OK) return rc;
+      if (two_streams) {
+        KVC_HIP(hipEventRecord(c.filled[sl], ks));
+        KVC_HIP(hipStreamWaitEvent(cs, c.filled[sl], 0));
+      }
+      rc = copy_chunk_rows(slot, host_pool, host_ids + done, count, width, host_block_bytes,
+                           host_row_offset, true, cs);
+      if (rc != KVC_OK) return rc;
+      if (two_streams) KVC_HIP(hipEventRecord(c.drained[sl], cs));
+    } else {
+      // host -> slot -> scatter into pool blocks
+      if (two_streams && k >= 2) KVC_HIP(hipStreamWaitEvent(cs, c.drained[sl], 0));
+      rc = copy_chunk_rows(slot, host_pool, host_ids + done, count, width, host_block_bytes,
+                           host_row_offset, false, cs);
+      if (rc != KVC_OK) return rc;
+      if (two_streams) {
+        KVC_HIP(hipEventRecord(c.filled[sl], cs));
+        KVC_HIP(hipStreamWaitEvent(ks, c.filled[sl], 0));
+      }
+      t.src_base = slot; t.src_ids = nullptr;
+      t.src_layer_stride = g.block_bytes; t.src_block_stride = width;
+      t.num_src_blocks = count;
+      t.dst_base = pool_l0; t.dst_ids = d_gpu_ids + done;
+      t.dst_layer_stride = g.layer_stride_bytes; t.dst_block_stride = g.block_bytes;
+      t.num_dst_blocks = g.num_gpu_blocks;
+      rc = launch_tiles(t, count, g_tune.copy_max_wgs, ks);
+      if (rc != KVC_OK) return rc;
+      if (two_streams) KVC_HIP(hipEventRecord(c.drained[sl], ks));
+    }
+  }
+  if (two_streams && out) {
+    // the last PCIe extents sit on the copy stream: fold them into kernel_stream
+    KVC_HIP(hipEventRecord(c.tail, cs));
+    KVC_HIP(hipStreamWaitEvent(ks, c.tail, 0));
+  }
+  return KVC_OK;
+}
+
+}  // namespace
+
+// ===========================================================================
+// C ABI
+// ===========================================================================
+extern "C" {
+
+int kvc_abi_version(void) { return KVC_ABI_VERSION; }
+
+const char* kvc_last_error_string(void) { return g_err; }
+
+// Tuning hook for sweeps (not part of the reference surface): returns 0, or
+// KVC_ERR_INVALID_ARG for an unknown key.
+int kvc_set_tuning(const char* key, int value) {
+  if (!key) return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: null key");
+  if (!strcmp(key, "copy_unroll")) g_tune.copy_unroll = value;
+  else if (!strcmp(key, "copy_nt")) g_tune.copy_nt = value;
+  else if (!strcmp(key, "copy_max_wgs")) g_tune.copy_max_wgs = value;
+  else if (!strcmp(key, "write_vpt")) g_tune.write_vpt = value;
+  else if (!strcmp(key, "write_nt")) g_tune.write_nt = value;
+  else if (!strcmp(key, "direct_max_wgs")) g_tune.direct_max_wgs = value;
+  else return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: unknown key '%s'", key);
+  return KVC_OK;
+}
+
+int kvc_reshape_and_cache_layers(const void* key, const void* value, void* key_cache,
+                                 void* value_cache, const void* slot_mapping, int slot_bytes,
+                                 int64_t num_tokens, int64_t row_elems, int64_t key_token_stride,
+                                 int64_t value_token_stride, int64_t block_size,
+                                 int64_t cache_block_stride, int64_t cache_slot_stride,
+                                 int64_t num_cache_blocks, int64_t num_layers,
+                                 int64_t key_layer_stride, int64_t value_layer_stride,
+                                 int64_t cache_layer_stride, int elem_bytes, void* stream) {
+  WriteGeom g{num_tokens, row_elems, key_token_stride, value_token_stride, block_size,
+              cache_block_stride, cache_slot_stride, num_cache_blocks, num_layers,
+              key_layer_stride, value_layer_stride, cache_layer_stride, elem_bytes};
+  return run_write("kvc_reshape_and_cache", key, value, key_cache, value_cache, slot_mapping,
+                   slot_bytes, nullptr, nullptr, nullptr, nullptr, 0, 0, g, stream);
+}
+
+int kvc_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                          const void* slot_mapping, int slot_bytes, int64_t num_tokens,
+                          int64_t row_elems, int64_t key_token_stride, int64_t value_token_stride,
+                          int64_t block_size, int64_t cache_block_stride, int64_t cache_slot_stride,
+                          int64_t num_cache_blocks, int elem_bytes, void* stream) {
+  return kvc_reshape_and_cache_layers(key, value, key_cache, value_cache, slot_mapping, slot_bytes,
+                                      num_tokens, row_elems, key_token_stride, value_token_stride,
+                                      block_size, cache_block_stride, cache_slot_stride,
+                                      num_cache_blocks, 1, 0, 0, 0, elem_bytes, stream);
+}
+
+int kvc_append_paged_kv_cache_layers(const void* append_key, const void* append_value,
+                                     const int32_t* batch_indices, const int32_t* positions,
+                                     void* paged_kv_cache, const int32_t* kv_indices,
+                                     const int32_t* kv_indptr, const int32_t* kv_last_page_len,
+                                     int64_t nnz, int64_t batch_size, int64_t num_kv_indices,
+                                     int64_t num_kv_heads, int64_t head_dim, int64_t page_size,
+                                     int64_t key_token_stride, int64_t value_token_stride,
+                                     int64_t page_stride, int64_t num_pages, int64_t num_layers,
+                                     int64_t key_layer_stride, int64_t value_layer_stride,
+                                     int64_t cache_layer_stride, int elem_bytes, void* stream) {
+  (void)kv_last_page_len;
+  if (num_kv_heads < 0 || head_dim < 0 || page_size <= 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_append_paged_kv_cache: bad H/D/page_size");
+  const int64_t row = num_kv_heads * head_dim;
+  if (nnz > 0 && !batch_indices)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_append_paged_kv_cache: null batch_indices");
+  if (page_stride < 2 * page_size * row)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_append_paged_kv_cache: page_stride %lld < 2*page_size*H*D",
+                (long long)page_stride);
+  WriteGeom g{nnz, row, key_token_stride, value_token_stride, page_size, page_stride, row,
+              num_pages, num_layers, key_layer_stride, value_layer_stride, cache_layer_stride,
+              elem_bytes};
+  char* vc = paged_kv_cache ? (char*)paged_kv_cache + page_size * row * (int64_t)elem_bytes : nullptr;
+  return run_write("kvc_append_paged_kv_cache", append_key, append_value, paged_kv_cache, vc,
+                   nullptr, 0, batch_indices, positions, kv_indices, kv_indptr, batch_size,
+                   num_kv_indices, g, stream);
+}
+
+int kvc_append_paged_kv_cache(const void* append_key, const void* append_value,
+                              const int32_t* batch_indices, const int32_t* positions,
+                              void* paged_kv_cache, const int32_t* kv_indices,
+                              const int32_t* kv_indptr, const int32_t* kv_last_page_len,
+                              int64_t nnz, int64_t batch_size, int64_t num_kv_indices,
+                              int64_t num_kv_heads, int64_t head_dim, int64_t page_size,
+                              int64_t key_token_stride, int64_t value_token_stride,
+                              int64_t page_stride, int64_t num_pages, int elem_bytes,
+                              void* stream) {
+  return kvc_append_paged_kv_cache_layers(append_key, append_value, batch_indices, positions,
+                                          paged_kv_cache, kv_indices, kv_indptr, kv_last_page_len,
+                                          nnz, batch_size, num_kv_indices, num_kv_heads, head_dim,
+                                          page_size, key_token_stride, value_token_stride,
+                                          page_stride, num_pages, 1, 0, 0, 0, elem_bytes, stream);
+}
+
+int kvc_get_seq_lens(const int32_t* kv_indptr, const int32_t* kv_last_page_len, int64_t batch_size,
+                     int64_t page_size, int32_t* seq_lens, void* stream) {
+  if (batch_size < 0 || page_size <= 0 || page_size > INT32_MAX)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_get_seq_lens: batch_size=%lld page_size=%lld",
+                (long long)batch_size, (long long)page_size);
+  if (batch_size == 0) return KVC_OK;
+  if (!kv_indptr || !kv_last_page_len || !seq_lens)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_get_seq_lens: null pointer");
+  const unsigned grid = (unsigned)((batch_size + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(seq_lens_kernel, dim3(grid), dim3(kThreads), 0, (hipStream_t)stream, kv_indptr,
+                     kv_last_page_len, batch_size, (int32_t)page_size, seq_lens);
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+int kvc_get_batch_indices_positions(const int32_t* append_indptr, const int32_t* seq_lens,
+                                    int64_t batch_size, int64_t nnz, int32_t* batch_indices,
+                                    int32_t* positions, void* stream) {
+  if (batch_size < 0 || nnz < 0 || batch_size > 0x7fffffffll)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_get_batch_indices_positions: batch_size=%lld nnz=%lld",
+                (long long)batch_size, (long long)nnz);
+  if (batch_size == 0 || nnz == 0) return KVC_OK;
+  if (!append_indptr || !seq_lens || !batch_indices || !positions)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_get_batch_indices_positions: null pointer");
+  hipLaunchKernelGGL(batch_indices_positions_kernel, dim3((unsigned)batch_size), dim3(kThreads), 0,
+                     (hipStream_t)stream, append_indptr, seq_lens, nnz, batch_indices, positions);
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pairs,
+                    int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                    int64_t num_blocks, void* stream) {
+  if (num_pairs < 0 || num_layers < 0 || block_bytes < 0 || num_blocks < 0 || layer_stride_bytes < 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_copy_blocks: negative size");
+  if (num_pairs == 0 || num_layers == 0 || block_bytes == 0) return KVC_OK;
+  if (!kv_caches || !block_maps) return fail(KVC_ERR_INVALID_ARG, "kvc_copy_blocks: null pointer");
+  if (layer_stride_bytes < block_bytes)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_copy_blocks: layer stride %lld < block bytes %lld",
+                (long long)layer_stride_bytes, (long long)block_bytes);
+  if (num_layers > 0xffffffffll) return fail(KVC_ERR_UNSUPPORTED, "kvc_copy_blocks: too many layers");
+  TileArgs t{};
+  t.src_base = (const char*)kv_caches;
+  t.dst_base = (char*)kv_caches;
+  t.src_ids = block_maps;
+  t.dst_ids = block_maps + 1;
+  t.id_stride = 2;
+  t.src_layer_stride = t.dst_layer_stride = layer_stride_bytes;
+  t.src_block_stride = t.dst_block_stride = block_bytes;
+  t.num_src_blocks = t.num_dst_blocks = num_blocks;
+  t.tile_bytes = block_bytes;
+  t.num_layers = (uint32_t)num_layers;
+  return launch_tiles(t, num_pairs, g_tune.copy_max_wgs, (hipStream_t)stream);
+}
+
+int64_t kvc_swap_staging_bytes(int64_t n, int64_t num_layers_in_range, int64_t block_bytes,
+                               int mode, int64_t chunk_blocks) {
+  if (n < 0 || num_layers_in_range < 0 || block_bytes < 0) return KVC_ERR_INVALID_ARG;
+  const int64_t ids = std::max<int64_t>(ids_region_bytes(n), kIdAlign);
+  if (mode == KVC_SWAP_DIRECT || n == 0) return ids;
+  const int64_t per_block = round_up(num_layers_in_range * block_bytes, kIdAlign);
+  if (per_block == 0) return ids;
+  if (chunk_blocks <= 0) {
+    // default ring slot: about 64 MiB, large enough for the DMA engines to run
+    // at link rate and small next to HBM
+    chunk_blocks = std::max<int64_t>(1, (int64_t(64) << 20) / per_block);
+  }
+  chunk_blocks = std::min(chunk_blocks, n);
+  return ids + 2 * per_block * chunk_blocks;
+}
+
+int kvc_swap_out(const void* pool, void* host_pool, const int64_t* src_ids, const int64_t* dst_ids,
+                 int64_t n, int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                 int64_t num_gpu_blocks, int64_t num_host_blocks, int64_t layer_begin,
+                 int64_t layer_end, void* staging, int64_t staging_bytes, int mode,
+                 void* kernel_stream, void* copy_stream) {
+  SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
+             layer_begin, layer_end};
+  return run_swap("kvc_swap_out", true, (char*)pool, (char*)host_pool, src_ids, dst_ids, g,
+                  staging, staging_bytes, mode, kernel_stream, copy_stream);
+}
+
+int kvc_swap_in(void* pool, const void* host_pool, const int64_t* src_ids, const int64_t* dst_ids,
+                int64_t n, int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                int64_t num_gpu_blocks, int64_t num_host_blocks, int64_t layer_begin,
+                int64_t layer_end, void* staging, int64_t staging_bytes, int mode,
+                void* kernel_stream, void* copy_stream) {
+  SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
+             layer_begin, layer_end};
+  return run_swap("kvc_swap_in", false, (char*)pool, (char*)host_pool, dst_ids, src_ids, g, staging,
+                  staging_bytes, mode, kernel_stream, copy_stream);
+}
+
+void* kvc_host_alloc_pinned(size_t bytes) {
+  void* p = nullptr;
+  if (bytes == 0) bytes = 1;
+  hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    fail(KVC_ERR_HIP, "hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    return nullptr;
+  }
+  return p;
+}
+
+int kvc_host_free_pinned(void* ptr) {
+  if (!ptr) return KVC_OK;
+  KVC_HIP(hipHostFree(ptr));
+  return KVC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,312 @@
+"""Swap engine between the HBM block pool and a pinned host pool.
+
+Mirrors the GPU<->Host part of runtime/worker/llm_worker/kv_worker.py of the
+reference: the pools' layouts (kv_worker.py:104-130), the direction table
+(kv_worker.py:190-195), `copy_kv(block_mappings, src, dst)` and its error
+behaviour (kv_worker.py:336-346), and the per-entry semantics
+  GPU->Host: host[dst_block_id, l] = gpu[l, src_block_id]   (kv_worker.py:213-227)
+  Host->GPU: gpu[l, dst_block_id] = host[src_block_id, l]   (kv_worker.py:197-211)
+Where the reference issues one driver memcpy per (layer, block), this engine
+hands the whole mapping list to libkvcache (`kvc_swap_out` / `kvc_swap_in`):
+a gather/scatter kernel plus large PCIe extents on a second stream, or one
+kernel that addresses the mapped host pool directly.
+
+The Host<->Disk legs (kv_worker.py:229-247) are plain NumPy row copies on a
+`.npy` memory map, as in the reference; they involve no GPU work.
+"""
+from __future__ import annotations
+
+import asyncio
+import ctypes
+import enum
+import os
+from dataclasses import dataclass, field
+from typing import Iterable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+class Device(enum.IntEnum):
+    """proto/worker.proto:13-17 of the reference."""
+    GPU = 0
+    Host = 1
+    Disk = 2
+
+
+@dataclass
+class BlockMappingEntry:
+    """proto/worker.proto:78-81."""
+    src_block_id: int
+    dst_block_id: int
+
+
+@dataclass
+class BlockMapping:
+    """proto/worker.proto:83-85: one mapping per sequence."""
+    entries: List[BlockMappingEntry] = field(default_factory=list)
+
+    @classmethod
+    def from_pairs(cls, pairs: Iterable[Tuple[int, int]]) -> "BlockMapping":
+        return cls([BlockMappingEntry(int(s), int(d)) for s, d in pairs])
+
+
+# kv_worker.py:17-22: bf16 travels as uint16 on the host
+dtype_map = {
+    torch.float32: np.float32,
+    torch.float16: np.float16,
+    torch.bfloat16: np.uint16,
+    torch.int32: np.int32,
+}
+
+SWAP_MODES = {"staged": _lib.KVC_SWAP_STAGED, "direct": _lib.KVC_SWAP_DIRECT}
+
+
+def flatten_block_mappings(block_mappings: Sequence[BlockMapping]) -> Tuple[np.ndarray, np.ndarray]:
+    """All entries of all mappings, in order, as (src_ids, dst_ids) int64 arrays.
+    Accepts anything with `.entries[*].src_block_id/.dst_block_id` (the protobuf
+    messages of the reference included)."""
+    src: List[int] = []
+    dst: List[int] = []
+    for mapping in block_mappings:
+        for entry in mapping.entries:
+            src.append(entry.src_block_id)
+            dst.append(entry.dst_block_id)
+    return np.asarray(src, dtype=np.int64), np.asarray(dst, dtype=np.int64)
+
+
+class PinnedHostPool:
+    """`[num_host_blocks, L, block_elems]` page-locked, device-addressable host
+    memory (replaces pycuda's `pagelocked_empty`, kv_worker.py:123-127)."""
+
+    def __init__(self, shape: Tuple[int, int, int], np_dtype):
+        self.shape = tuple(int(s) for s in shape)
+        self.np_dtype = np.dtype(np_dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.np_dtype.itemsize
+        self.ptr = _lib.lib().kvc_host_alloc_pinned(max(self.nbytes, 1))
+        if not self.ptr:
+            raise MemoryError(f"cannot pin {self.nbytes} bytes of host memory: {_lib.last_error()}")
+        buf = (ctypes.c_char * max(self.nbytes, 1)).from_address(self.ptr)
+        self.array = np.frombuffer(buf, dtype=self.np_dtype,
+                                   count=self.nbytes // self.np_dtype.itemsize).reshape(self.shape)
+
+    def close(self) -> None:
+        if self.ptr:
+            self.array = None
+            _lib.check(_lib.lib().kvc_host_free_pinned(self.ptr))
+            self.ptr = None
+
+
+def memmap_disk_kv_cache(kv_cache_file: str, shape: Tuple[int, ...], dtype, mode: str = "r+"):
+    """Open the disk tier's `.npy` memory map, recreating it when the stored
+    shape or dtype no longer match (kv_worker.py:48-85)."""
+    if os.path.exists(kv_cache_file):
+        try:
+            kv_cache = np.load(kv_cache_file, mmap_mode=mode)
+            if kv_cache.shape == tuple(shape) and kv_cache.dtype == np.dtype(dtype):
+                return kv_cache
+            del kv_cache
+        except Exception:
+            pass
+        os.remove(kv_cache_file)
+    return np.lib.format.open_memmap(kv_cache_file, mode="w+", dtype=dtype, shape=tuple(shape))
+
+
+class KVWorker:
+    """Owns the host pool and moves blocks between the tiers.
+
+    gpu_kv_caches: the model worker's pool `[L, num_gpu_blocks, ...]`
+      (`[L, nb, 2, bs, H, D]`), contiguous, on the GPU. The reference maps it
+      from an IPC handle in a second process (kv_worker.py:104-108); here the
+      tensor itself is passed.
+    """
+
+    def __init__(
+        self,
+        gpu_kv_caches: torch.Tensor,
+        num_host_blocks: int,
+        num_disk_blocks: int = 0,
+        disk_kv_cache_file: Optional[str] = None,
+        swap_mode: str = "staged",
+        staging_chunk_blocks: int = 0,
+    ):
+        if not gpu_kv_caches.is_cuda:
+            raise ValueError("gpu_kv_caches must live on the GPU")
+        if gpu_kv_caches.dim() < 3 or not gpu_kv_caches.is_contiguous():
+            raise ValueError("gpu_kv_caches must be a contiguous [L, num_gpu_blocks, ...] tensor")
+        if swap_mode not in SWAP_MODES:
+            raise ValueError(f"swap_mode must be one of {sorted(SWAP_MODES)}")
+        np_dtype = dtype_map.get(gpu_kv_caches.dtype)
+        if np_dtype is None:
+            raise TypeError(f"Unsupported dtype: {gpu_kv_caches.dtype}")
+
+        num_layers, num_gpu_blocks = gpu_kv_caches.shape[0], gpu_kv_caches.shape[1]
+        self.gpu_kv_caches = gpu_kv_caches.view(num_layers, num_gpu_blocks, -1)
+        block_elems = self.gpu_kv_caches.shape[2]
+        self.device = gpu_kv_caches.device
+        self.num_layers = num_layers
+        self.num_gpu_blocks = num_gpu_blocks
+        self.num_host_blocks = int(num_host_blocks)
+        self.num_disk_blocks = int(num_disk_blocks)
+        self.block_stride = block_elems * gpu_kv_caches.element_size()  # bytes, kv_worker.py:157
+        self.layer_stride = num_gpu_blocks * self.block_stride
+        self.swap_mode = swap_mode
+        self.staging_chunk_blocks = int(staging_chunk_blocks)
+
+        self._host_pool = PinnedHostPool((self.num_host_blocks, num_layers, block_elems), np_dtype)
+        self.host_kv_caches = self._host_pool.array
+        self.host_kv_caches_tensor = torch.from_numpy(self.host_kv_caches)
+
+        if self.num_disk_blocks > 0:
+            if not disk_kv_cache_file:
+                raise ValueError("disk_kv_cache_file is required when num_disk_blocks > 0")
+            self.disk_kv_caches = memmap_disk_kv_cache(
+                disk_kv_cache_file, (self.num_disk_blocks, num_layers, block_elems), np_dtype)
+        else:
+            self.disk_kv_caches = None
+
+        with torch.cuda.device(self.device):
+            self.dtoh_stream = torch.cuda.Stream()
+            self.htod_stream = torch.cuda.Stream()
+            self._dtoh_copy_stream = torch.cuda.Stream()
+            self._htod_copy_stream = torch.cuda.Stream()
+        self._staging = {"out": None, "in": None}
+
+        self.COPY_KV_OP_MAP = {
+            (Device.GPU, Device.Host): self._copy_kv_gpu_to_host,
+            (Device.Host, Device.GPU): self._copy_kv_host_to_gpu,
+            (Device.Host, Device.Disk): self._copy_kv_host_to_disk,
+            (Device.Disk, Device.Host): self._copy_kv_disk_to_host,
+        }
+
+    # ------------------------------------------------------------------ GPU legs
+    def _staging_for(self, direction: str, n: int, num_layers_in_range: int) -> torch.Tensor:
+        mode = SWAP_MODES[self.swap_mode]
+        need = _lib.lib().kvc_swap_staging_bytes(n, num_layers_in_range, self.block_stride, mode,
+                                                 self.staging_chunk_blocks)
+        if need < 0:
+            raise ValueError("bad swap geometry")
+        buf = self._staging[direction]
+        if buf is None or buf.numel() < need:
+            buf = torch.empty(int(need), dtype=torch.uint8, device=self.device)
+            self._staging[direction] = buf
+        return buf
+
+    def _swap(self, direction: str, src: np.ndarray, dst: np.ndarray, layer_begin: int,
+              layer_end: int, stream: torch.cuda.Stream, copy_stream: torch.cuda.Stream) -> None:
+        n = int(src.shape[0])
+        if n == 0 or layer_end <= layer_begin:
+            return
+        src = np.ascontiguousarray(src, dtype=np.int64)
+        dst = np.ascontiguousarray(dst, dtype=np.int64)
+        with torch.cuda.device(self.device):
+            # whatever the caller's current stream has queued on the pool comes first
+            stream.wait_stream(torch.cuda.current_stream(self.device))
+            staging = self._staging_for(direction, n, layer_end - layer_begin)
+            # the staging buffer may have been allocated on another stream
+            staging.record_stream(stream)
+            staging.record_stream(copy_stream)
+            fn = _lib.lib().kvc_swap_out if direction == "out" else _lib.lib().kvc_swap_in
+            _lib.check(fn(self.gpu_kv_caches.data_ptr(), self._host_pool.ptr,
+                          src.ctypes.data, dst.ctypes.data, n, self.num_layers, self.layer_stride,
+                          self.block_stride, self.num_gpu_blocks, self.num_host_blocks,
+                          layer_begin, layer_end, staging.data_ptr(), staging.numel(),
+                          SWAP_MODES[self.swap_mode], stream.cuda_stream, copy_stream.cuda_stream))
+
+    def save_kv_blocks_to_host_nowait(self, block_mappings: Sequence[BlockMapping],
+                                      stream: Optional[torch.cuda.Stream] = None,
+                                      layer_begin: int = 0, layer_end: Optional[int] = None) -> None:
+        """Enqueue GPU->Host for layers [layer_begin, layer_end) on `stream`."""
+        if len(block_mappings) == 0:
+            return
+        src, dst = flatten_block_mappings(block_mappings)
+        self._swap("out", src, dst, layer_begin, self.num_layers if layer_end is None else layer_end,
+                   stream or self.dtoh_stream, self._dtoh_copy_stream)
+
+    def load_kv_blocks_from_host_nowait(self, block_mappings: Sequence[BlockMapping],
+                                        stream: Optional[torch.cuda.Stream] = None,
+                                        layer_begin: int = 0, layer_end: Optional[int] = None) -> None:
+        """Enqueue Host->GPU for layers [layer_begin, layer_end) on `stream`."""
+        if len(block_mappings) == 0:
+            return
+        src, dst = flatten_block_mappings(block_mappings)
+        self._swap("in", src, dst, layer_begin, self.num_layers if layer_end is None else layer_end,
+                   stream or self.htod_stream, self._htod_copy_stream)
+
+    async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
+                                     stream: torch.cuda.Stream) -> None:
+        self.save_kv_blocks_to_host_nowait(block_mappings, stream)
+        await asyncio.to_thread(stream.synchronize)
+
+    async def load_kv_blocks_from_host(self, block_mappings: Sequence[BlockMapping],
+                                       stream: torch.cuda.Stream) -> None:
+        self.load_kv_blocks_from_host_nowait(block_mappings, stream)
+        await asyncio.to_thread(stream.synchronize)
+
+    # ----------------------------------------------------------------- disk legs
+    def _require_disk(self) -> None:
+        if self.disk_kv_caches is None:
+            raise ValueError("no disk KV cache configured (num_disk_blocks == 0)")
+
+    def load_kv_blocks_from_disk_sync(self, block_mappings: Sequence[BlockMapping]) -> None:
+        """host[dst] = disk[src] for every layer (kv_worker.py:229-237)."""
+        if len(block_mappings) == 0:
+            return
+        self._require_disk()
+        src, dst = flatten_block_mappings(block_mappings)
+        for s, d in zip(src.tolist(), dst.tolist()):
+            self.host_kv_caches[d] = self.disk_kv_caches[s]
+
+    def save_kv_blocks_to_disk_sync(self, block_mappings: Sequence[BlockMapping]) -> None:
+        """disk[dst] = host[src] for every layer (kv_worker.py:239-247)."""
+        if len(block_mappings) == 0:
+            return
+        self._require_disk()
+        src, dst = flatten_block_mappings(block_mappings)
+        for s, d in zip(src.tolist(), dst.tolist()):
+            self.disk_kv_caches[d] = self.host_kv_caches[s]
+
+    # ---------------------------------------------------------------- dispatcher
+    async def _copy_kv_gpu_to_host(self, block_mappings):
+        await self.save_kv_blocks_to_host(block_mappings, self.dtoh_stream)
+
+    async def _copy_kv_host_to_gpu(self, block_mappings):
+        await self.load_kv_blocks_from_host(block_mappings, self.htod_stream)
+
+    async def _copy_kv_host_to_disk(self, block_mappings):
+        await asyncio.to_thread(self.save_kv_blocks_to_disk_sync, block_mappings)
+
+    async def _copy_kv_disk_to_host(self, block_mappings):
+        await asyncio.to_thread(self.load_kv_blocks_from_disk_sync, block_mappings)
+
+    async def copy_kv(self, block_mappings: Sequence[BlockMapping], src: Device, dst: Device) -> None:
+        key = (src, dst)
+        if key not in self.COPY_KV_OP_MAP:
+            raise ValueError(f"Unsupported copy direction: {src} -> {dst}")
+        await self.COPY_KV_OP_MAP[key](block_mappings)
+
+    def copy_kv_sync(self, block_mappings: Sequence[BlockMapping], src: Device, dst: Device) -> None:
+        """`copy_kv` for callers without an event loop; returns when the copy is complete."""
+        key = (src, dst)
+        if key not in self.COPY_KV_OP_MAP:
+            raise ValueError(f"Unsupported copy direction: {src} -> {dst}")
+        if key == (Device.GPU, Device.Host):
+            self.save_kv_blocks_to_host_nowait(block_mappings)
+            self.dtoh_stream.synchronize()
+        elif key == (Device.Host, Device.GPU):
+            self.load_kv_blocks_from_host_nowait(block_mappings)
+            self.htod_stream.synchronize()
+        elif key == (Device.Host, Device.Disk):
+            self.save_kv_blocks_to_disk_sync(block_mappings)
+        else:
+            self.load_kv_blocks_from_disk_sync(block_mappings)
+
+    def close(self) -> None:
+        with torch.cuda.device(self.device):
+            torch.cuda.synchronize()
+        self.host_kv_caches_tensor = None
+        self.host_kv_caches = None
+        self._host_pool.close()
+        self._staging = {"out": None, "in": None}

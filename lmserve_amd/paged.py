@@ -1,0 +1,180 @@
+"""Page-table addressed K/V write and its index preparation.
+
+Drop-in for the three third-party calls on the reference's live write path
+(flashinfer-python 0.3.1.post1, pinned in runtime/worker/uv.lock:148-149):
+`append_paged_kv_cache` as called at
+runtime/worker/llm_worker/models/layers/attention.py:76-85, and
+`get_seq_lens` / `get_batch_indices_positions` as called at
+runtime/worker/llm_worker/model_worker.py:425-433. Names, argument order and
+tensor layouts are those calls'; the "NHD" single-tensor cache
+`[num_pages, 2, page_size, H, D]` is the only layout the reference uses
+(model_worker.py:65-66) and the only one served here.
+"""
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+from . import _lib
+from .cache_ops import _require_gpu, _rows, _stream_of
+
+
+def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
+    _require_gpu(t, name)
+    if t.dtype != torch.int32:
+        raise TypeError(f"{name} must be int32 (got {t.dtype})")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def get_seq_lens(kv_indptr: torch.Tensor, kv_last_page_len: torch.Tensor,
+                 page_size: int) -> torch.Tensor:
+    """`seq_lens[b] = max(kv_indptr[b+1]-kv_indptr[b]-1, 0)*page_size + kv_last_page_len[b]`."""
+    kv_indptr = _i32(kv_indptr, "kv_indptr")
+    kv_last_page_len = _i32(kv_last_page_len, "kv_last_page_len")
+    batch_size = kv_last_page_len.numel()
+    if kv_indptr.numel() != batch_size + 1:
+        raise ValueError("kv_indptr must have batch_size + 1 entries")
+    seq_lens = torch.empty(batch_size, dtype=torch.int32, device=kv_indptr.device)
+    with torch.cuda.device(kv_indptr.device):
+        _lib.check(_lib.lib().kvc_get_seq_lens(
+            kv_indptr.data_ptr(), kv_last_page_len.data_ptr(), batch_size, int(page_size),
+            seq_lens.data_ptr(), _stream_of(kv_indptr)))
+    return seq_lens
+
+
+def get_batch_indices_positions(append_indptr: torch.Tensor, seq_lens: torch.Tensor,
+                                nnz: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per appended token: the request it belongs to and its absolute position.
+
+    For request `b` with `n_b = append_indptr[b+1]-append_indptr[b]` new tokens
+    the j-th of them gets `batch_indices = b`, `positions = seq_lens[b] - n_b + j`.
+    With the reference's inputs `seq_lens[b]` is the request's context length,
+    so `positions` equals its `position_ids` (model_worker.py:346).
+    """
+    append_indptr = _i32(append_indptr, "append_indptr")
+    seq_lens = _i32(seq_lens, "seq_lens")
+    batch_size = seq_lens.numel()
+    if append_indptr.numel() != batch_size + 1:
+        raise ValueError("append_indptr must have batch_size + 1 entries")
+    batch_indices = torch.empty(int(nnz), dtype=torch.int32, device=append_indptr.device)
+    positions = torch.empty(int(nnz), dtype=torch.int32, device=append_indptr.device)
+    with torch.cuda.device(append_indptr.device):
+        _lib.check(_lib.lib().kvc_get_batch_indices_positions(
+            append_indptr.data_ptr(), seq_lens.data_ptr(), batch_size, int(nnz),
+            batch_indices.data_ptr(), positions.data_ptr(), _stream_of(append_indptr)))
+    return batch_indices, positions
+
+
+def _paged_common(append_key, append_value, batch_indices, positions, kv_indices, kv_indptr,
+                  kv_last_page_len, kv_layout):
+    if kv_layout != "NHD":
+        raise ValueError(f"kv_layout {kv_layout!r} is not supported (the reference uses 'NHD')")
+    batch_indices = _i32(batch_indices, "batch_indices")
+    positions = _i32(positions, "positions")
+    kv_indices = _i32(kv_indices, "kv_indices")
+    kv_indptr = _i32(kv_indptr, "kv_indptr")
+    kv_last_page_len = _i32(kv_last_page_len, "kv_last_page_len")
+    if batch_indices.numel() != positions.numel():
+        raise ValueError("batch_indices and positions differ in length")
+    return batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len
+
+
+def append_paged_kv_cache(
+    append_key: torch.Tensor,
+    append_value: torch.Tensor,
+    batch_indices: torch.Tensor,
+    positions: torch.Tensor,
+    paged_kv_cache: torch.Tensor,
+    kv_indices: torch.Tensor,
+    kv_indptr: torch.Tensor,
+    kv_last_page_len: torch.Tensor,
+    kv_layout: str = "NHD",
+) -> None:
+    """Write token `i` to page `kv_indices[kv_indptr[b] + p // page_size]`, entry
+    `p % page_size`, with `b = batch_indices[i]`, `p = positions[i]`.
+
+    append_key, append_value: `[nnz, H, D]`; paged_kv_cache:
+    `[num_pages, 2, page_size, H, D]` (one layer of the pool); index tensors
+    int32 on the device. In place; returns None.
+    """
+    if isinstance(paged_kv_cache, (tuple, list)):
+        raise ValueError("only the single-tensor NHD paged cache is supported")
+    for t, n in ((append_key, "append_key"), (append_value, "append_value"),
+                 (paged_kv_cache, "paged_kv_cache")):
+        _require_gpu(t, n)
+    batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len = _paged_common(
+        append_key, append_value, batch_indices, positions, kv_indices, kv_indptr,
+        kv_last_page_len, kv_layout)
+    if paged_kv_cache.dim() != 5 or paged_kv_cache.shape[1] != 2 or \
+            (paged_kv_cache.shape[0] > 0 and not paged_kv_cache[0].is_contiguous()):
+        raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
+    if append_key.dtype != paged_kv_cache.dtype or append_value.dtype != paged_kv_cache.dtype:
+        raise TypeError("append_key/append_value and paged_kv_cache must share one dtype")
+    num_pages, _, page_size, H, D = paged_kv_cache.shape
+    append_key, row, k_stride = _rows(append_key, "append_key")
+    append_value, row_v, v_stride = _rows(append_value, "append_value")
+    if row != H * D or row_v != H * D:
+        raise ValueError("append_key/append_value rows do not match the cache's H*D")
+    nnz = batch_indices.numel()
+    if append_key.shape[0] < nnz or append_value.shape[0] < nnz:
+        raise ValueError("fewer key/value rows than index entries")
+    if nnz == 0 or row == 0 or num_pages == 0:
+        return
+    page_stride = paged_kv_cache.stride(0) if num_pages > 1 else 2 * page_size * row
+    with torch.cuda.device(paged_kv_cache.device):
+        _lib.check(_lib.lib().kvc_append_paged_kv_cache(
+            append_key.data_ptr(), append_value.data_ptr(), batch_indices.data_ptr(),
+            positions.data_ptr(), paged_kv_cache.data_ptr(), kv_indices.data_ptr(),
+            kv_indptr.data_ptr(), kv_last_page_len.data_ptr(), nnz, kv_indptr.numel() - 1,
+            kv_indices.numel(), H, D, page_size, k_stride, v_stride, page_stride, num_pages,
+            paged_kv_cache.element_size(), _stream_of(paged_kv_cache)))
+
+
+def append_paged_kv_cache_layers(
+    append_key: torch.Tensor,
+    append_value: torch.Tensor,
+    batch_indices: torch.Tensor,
+    positions: torch.Tensor,
+    kv_caches: torch.Tensor,
+    kv_indices: torch.Tensor,
+    kv_indptr: torch.Tensor,
+    kv_last_page_len: torch.Tensor,
+    kv_layout: str = "NHD",
+) -> None:
+    """`append_paged_kv_cache` for every layer of the pool in one launch.
+
+    append_key, append_value: `[L, nnz, H, D]` contiguous; kv_caches:
+    `[L, num_pages, 2, page_size, H, D]` contiguous; one page table for all layers.
+    """
+    for t, n in ((append_key, "append_key"), (append_value, "append_value"),
+                 (kv_caches, "kv_caches")):
+        _require_gpu(t, n)
+    batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len = _paged_common(
+        append_key, append_value, batch_indices, positions, kv_indices, kv_indptr,
+        kv_last_page_len, kv_layout)
+    if kv_caches.dim() != 6 or kv_caches.shape[2] != 2 or not kv_caches.is_contiguous():
+        raise ValueError("kv_caches must be contiguous [L, num_pages, 2, page_size, H, D]")
+    if append_key.dtype != kv_caches.dtype or append_value.dtype != kv_caches.dtype:
+        raise TypeError("append_key/append_value and kv_caches must share one dtype")
+    L, num_pages, _, page_size, H, D = kv_caches.shape
+    row = H * D
+    if append_key.dim() != 4 or append_key.shape != append_value.shape \
+            or append_key.shape[0] != L or append_key.shape[2] * append_key.shape[3] != row:
+        raise ValueError("append_key/append_value must be [L, nnz, H, D] matching the pool")
+    append_key = append_key.contiguous()
+    append_value = append_value.contiguous()
+    nnz = batch_indices.numel()
+    tokens = append_key.shape[1]
+    if tokens < nnz:
+        raise ValueError("fewer key/value rows than index entries")
+    if nnz == 0 or row == 0 or num_pages == 0 or L == 0:
+        return
+    with torch.cuda.device(kv_caches.device):
+        _lib.check(_lib.lib().kvc_append_paged_kv_cache_layers(
+            append_key.data_ptr(), append_value.data_ptr(), batch_indices.data_ptr(),
+            positions.data_ptr(), kv_caches.data_ptr(), kv_indices.data_ptr(),
+            kv_indptr.data_ptr(), kv_last_page_len.data_ptr(), nnz, kv_indptr.numel() - 1,
+            kv_indices.numel(), H, D, page_size, row, row, 2 * page_size * row, num_pages,
+            L, tokens * row, tokens * row, num_pages * 2 * page_size * row,
+            kv_caches.element_size(), _stream_of(kv_caches)))

@@ -1,0 +1,265 @@
+"""TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+CPU restatements of the reference's paged KV-cache data movement, used only as
+the checker for the HIP library (tests/, the smoke check, bench.py's
+cpu_baseline leg). Nothing under lmserve_amd/ may import this module.
+
+Three independent formulations live here so that they can be checked against
+each other and against closed forms:
+
+  *_np     vectorised NumPy (fancy indexing on shaped views)
+  c_*      the plain-C loops of oracle/kvc_oracle.c through ctypes
+  *_loops  element-by-element pure Python following the reference kernels'
+           flat address arithmetic; only for tiny inputs
+
+All operate IN PLACE on NumPy arrays of any item size (bf16 is carried as
+uint16, as the reference's host pool does: kv_worker.py:17-22). Citations are
+paths under the reference's runtime/worker/llm_worker/. Pinning status is listed
+in the header of kvc_oracle.c; parity of the three page-table functions with
+the third-party flashinfer binary itself is UNPINNED.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional, Tuple
+
+import numpy as np
+
+ORACLE_DIR = os.path.dirname(os.path.abspath(__file__))
+C_LIB_PATH = os.path.join(ORACLE_DIR, "libkvc_oracle.so")
+
+# --------------------------------------------------------------------------- NumPy
+
+
+def fill_key_cache_np(key, value, key_cache, value_cache, slot_mapping) -> None:
+    """ops/cache_ops.py:39-59 + ops/triton/cache_kernels.py:39-58: caches are
+    addressed flat as [num_slots, H*D]."""
+    T = len(slot_mapping)
+    row = key.shape[1] * key.shape[2]
+    slots = np.asarray(slot_mapping, dtype=np.int64)
+    key_cache.reshape(-1, row)[slots] = key.reshape(T, row)
+    value_cache.reshape(-1, row)[slots] = value.reshape(T, row)
+
+
+def reshape_and_cache_np(key, value, kv_cache, slot_mapping) -> None:
+    """One layer of the pool [nb, 2, bs, H, D] (model_worker.py:221-228);
+    slot = blk*bs + e."""
+    bs = kv_cache.shape[2]
+    slots = np.asarray(slot_mapping, dtype=np.int64)
+    kv_cache[slots // bs, 0, slots % bs] = key
+    kv_cache[slots // bs, 1, slots % bs] = value
+
+
+def append_paged_kv_cache_np(append_key, append_value, batch_indices, positions, paged_kv_cache,
+                             kv_indices, kv_indptr, kv_last_page_len=None) -> None:
+    """The flashinfer call at models/layers/attention.py:76-85, NHD layout."""
+    page_size = paged_kv_cache.shape[2]
+    b = np.asarray(batch_indices, dtype=np.int64)
+    p = np.asarray(positions, dtype=np.int64)
+    pages = np.asarray(kv_indices, dtype=np.int64)[np.asarray(kv_indptr, dtype=np.int64)[b]
+                                                   + p // page_size]
+    paged_kv_cache[pages, 0, p % page_size] = append_key[:len(b)]
+    paged_kv_cache[pages, 1, p % page_size] = append_value[:len(b)]
+
+
+def get_seq_lens_np(kv_indptr, kv_last_page_len, page_size) -> np.ndarray:
+    """The flashinfer call at model_worker.py:427-431."""
+    kv_indptr = np.asarray(kv_indptr, dtype=np.int64)
+    full = np.maximum(kv_indptr[1:] - kv_indptr[:-1] - 1, 0)
+    return (full * page_size + np.asarray(kv_last_page_len, dtype=np.int64)).astype(np.int32)
+
+
+def get_batch_indices_positions_np(append_indptr, seq_lens, nnz) -> Tuple[np.ndarray, np.ndarray]:
+    """The flashinfer call at model_worker.py:425-433."""
+    append_indptr = np.asarray(append_indptr, dtype=np.int64)
+    n_new = append_indptr[1:] - append_indptr[:-1]
+    batch = np.repeat(np.arange(len(n_new), dtype=np.int64), n_new)
+    within = np.arange(int(append_indptr[-1]), dtype=np.int64) - append_indptr[:-1][batch]
+    pos = np.asarray(seq_lens, dtype=np.int64)[batch] - n_new[batch] + within
+    assert len(batch) <= nnz
+    return batch.astype(np.int32), pos.astype(np.int32)
+
+
+def copy_blocks_np(kv_caches, block_maps) -> None:
+    """ops/cache_ops.py:8-36 + ops/triton/cache_kernels.py:5-36 on the pool
+    viewed as [L, nb, block_elems]; NumPy evaluates the right-hand side first,
+    i.e. snapshot semantics."""
+    L, nb = kv_caches.shape[0], kv_caches.shape[1]
+    pool = kv_caches.reshape(L, nb, -1)
+    maps = np.asarray(block_maps, dtype=np.int64)
+    src, dst = maps[0::2], maps[1::2]
+    pool[:, dst] = pool[:, src]
+
+
+def save_blocks_to_host_np(gpu, host, src_ids, dst_ids, layer_begin=0, layer_end=None) -> None:
+    """kv_worker.py:213-227: host[dst, l] = gpu[l, src]; gpu [L, nb, E], host [nhb, L, E]."""
+    layer_end = gpu.shape[0] if layer_end is None else layer_end
+    src = np.asarray(src_ids, dtype=np.int64)
+    dst = np.asarray(dst_ids, dtype=np.int64)
+    host[dst, layer_begin:layer_end] = gpu[layer_begin:layer_end][:, src].swapaxes(0, 1)
+
+
+def load_blocks_from_host_np(gpu, host, src_ids, dst_ids, layer_begin=0, layer_end=None) -> None:
+    """kv_worker.py:197-211: gpu[l, dst] = host[src, l]."""
+    layer_end = gpu.shape[0] if layer_end is None else layer_end
+    src = np.asarray(src_ids, dtype=np.int64)
+    dst = np.asarray(dst_ids, dtype=np.int64)
+    gpu[layer_begin:layer_end][:, dst] = host[src, layer_begin:layer_end].swapaxes(0, 1)
+
+
+# ----------------------------------------------------------------- pure-Python loops
+
+
+def fill_key_cache_loops(key, value, key_cache, value_cache, slot_mapping) -> None:
+    """Element-by-element flat addressing of cache_kernels.py:39-58."""
+    H, D = key.shape[1], key.shape[2]
+    kf, vf = key.reshape(-1), value.reshape(-1)
+    kcf, vcf = key_cache.reshape(-1), value_cache.reshape(-1)
+    for i in range(len(slot_mapping)):
+        start = i * H * D
+        cache_start = int(slot_mapping[i]) * H * D
+        for off in range(H * D):
+            kcf[cache_start + off] = kf[start + off]
+            vcf[cache_start + off] = vf[start + off]
+
+
+def copy_blocks_loops(kv_caches, block_maps) -> None:
+    """Element-by-element flat addressing of cache_kernels.py:13-36."""
+    flat = kv_caches.reshape(-1)
+    L = kv_caches.shape[0]
+    numel_per_layer = kv_caches[0].size
+    numel_per_block = kv_caches[0][0].size
+    for j in range(len(block_maps) // 2):
+        src, dst = int(block_maps[2 * j]), int(block_maps[2 * j + 1])
+        for l in range(L):
+            base = l * numel_per_layer
+            for k in range(numel_per_block):
+                flat[base + dst * numel_per_block + k] = flat[base + src * numel_per_block + k]
+
+
+def append_paged_kv_cache_loops(append_key, append_value, batch_indices, positions,
+                                paged_kv_cache, kv_indices, kv_indptr) -> None:
+    page_size, H, D = paged_kv_cache.shape[2:]
+    for i in range(len(batch_indices)):
+        b, p = int(batch_indices[i]), int(positions[i])
+        page = int(kv_indices[int(kv_indptr[b]) + p // page_size])
+        e = p % page_size
+        for h in range(H):
+            for d in range(D):
+                paged_kv_cache[page, 0, e, h, d] = append_key[i, h, d]
+                paged_kv_cache[page, 1, e, h, d] = append_value[i, h, d]
+
+
+def save_blocks_to_host_loops(gpu, host, src_ids, dst_ids) -> None:
+    for l in range(gpu.shape[0]):
+        for s, d in zip(src_ids, dst_ids):
+            for k in range(gpu.shape[2]):
+                host[int(d), l, k] = gpu[l, int(s), k]
+
+
+def load_blocks_from_host_loops(gpu, host, src_ids, dst_ids) -> None:
+    for l in range(gpu.shape[0]):
+        for s, d in zip(src_ids, dst_ids):
+            for k in range(gpu.shape[2]):
+                gpu[l, int(d), k] = host[int(s), l, k]
+
+
+# ----------------------------------------------------------------------- C via ctypes
+
+_clib: Optional[ctypes.CDLL] = None
+
+
+def build_c_oracle() -> str:
+    """Compile oracle/kvc_oracle.c with the Makefile beside it."""
+    subprocess.run(["make", "-s", "-B", "-C", ORACLE_DIR, "libkvc_oracle.so"], check=True)
+    return C_LIB_PATH
+
+
+def c_lib() -> ctypes.CDLL:
+    global _clib
+    if _clib is None:
+        if not os.path.exists(C_LIB_PATH):
+            build_c_oracle()
+        _clib = ctypes.CDLL(C_LIB_PATH)
+    return _clib
+
+
+def _p(a: np.ndarray) -> ctypes.c_void_p:
+    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be C-contiguous"
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _i64(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.int64)
+
+
+def _i32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+_L = ctypes.c_int64
+
+
+def c_fill_key_cache(key, value, key_cache, value_cache, slot_mapping) -> None:
+    slots = _i64(slot_mapping)
+    c_lib().oracle_fill_key_cache(_p(key), _p(value), _p(key_cache), _p(value_cache), _p(slots),
+                                  _L(len(slots)), _L(key.shape[1]), _L(key.shape[2]),
+                                  _L(key.itemsize))
+
+
+def c_reshape_and_cache(key, value, kv_cache, slot_mapping) -> None:
+    slots = _i64(slot_mapping)
+    _, _, bs, H, D = kv_cache.shape
+    c_lib().oracle_reshape_and_cache(_p(key), _p(value), _p(kv_cache), _p(slots), _L(len(slots)),
+                                     _L(bs), _L(H), _L(D), _L(key.itemsize))
+
+
+def c_append_paged_kv_cache(append_key, append_value, batch_indices, positions, paged_kv_cache,
+                            kv_indices, kv_indptr, kv_last_page_len=None) -> None:
+    bi, pos, ind, ptr = _i32(batch_indices), _i32(positions), _i32(kv_indices), _i32(kv_indptr)
+    _, _, page_size, H, D = paged_kv_cache.shape
+    c_lib().oracle_append_paged_kv_cache(_p(append_key), _p(append_value), _p(bi), _p(pos),
+                                         _p(paged_kv_cache), _p(ind), _p(ptr), _L(len(bi)), _L(H),
+                                         _L(D), _L(page_size), _L(append_key.itemsize))
+
+
+def c_get_seq_lens(kv_indptr, kv_last_page_len, page_size) -> np.ndarray:
+    ptr, last = _i32(kv_indptr), _i32(kv_last_page_len)
+    out = np.zeros(len(last), dtype=np.int32)
+    c_lib().oracle_get_seq_lens(_p(ptr), _p(last), _L(len(last)), ctypes.c_int32(page_size), _p(out))
+    return out
+
+
+def c_get_batch_indices_positions(append_indptr, seq_lens, nnz) -> Tuple[np.ndarray, np.ndarray]:
+    ptr, sl = _i32(append_indptr), _i32(seq_lens)
+    bi = np.zeros(nnz, dtype=np.int32)
+    pos = np.zeros(nnz, dtype=np.int32)
+    c_lib().oracle_get_batch_indices_positions(_p(ptr), _p(sl), _L(len(sl)), _p(bi), _p(pos))
+    return bi, pos
+
+
+def c_copy_blocks(kv_caches, block_maps) -> None:
+    maps = _i64(block_maps)
+    c_lib().oracle_copy_blocks(_p(kv_caches), _p(maps), _L(len(maps) // 2), _L(kv_caches.shape[0]),
+                               _L(kv_caches[0].size), _L(kv_caches[0][0].size),
+                               _L(kv_caches.itemsize))
+
+
+def c_save_blocks_to_host(gpu, host, src_ids, dst_ids, layer_begin=0, layer_end=None) -> None:
+    src, dst = _i64(src_ids), _i64(dst_ids)
+    L, nb = gpu.shape[0], gpu.shape[1]
+    block_bytes = gpu[0][0].size * gpu.itemsize
+    c_lib().oracle_save_blocks_to_host(_p(gpu), _p(host), _p(src), _p(dst), _L(len(src)), _L(L),
+                                       _L(nb), _L(block_bytes), _L(layer_begin),
+                                       _L(L if layer_end is None else layer_end))
+
+
+def c_load_blocks_from_host(gpu, host, src_ids, dst_ids, layer_begin=0, layer_end=None) -> None:
+    src, dst = _i64(src_ids), _i64(dst_ids)
+    L, nb = gpu.shape[0], gpu.shape[1]
+    block_bytes = gpu[0][0].size * gpu.itemsize
+    c_lib().oracle_load_blocks_from_host(_p(gpu), _p(host), _p(src), _p(dst), _L(len(src)), _L(L),
+                                         _L(nb), _L(block_bytes), _L(layer_begin),
+                                         _L(L if layer_end is None else layer_end))

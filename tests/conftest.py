@@ -1,0 +1,24 @@
+import os
+import sys
+
+import pytest
+
+REPO_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if REPO_ROOT not in sys.path:
+    sys.path.insert(0, REPO_ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """The CUDA/HIP device the GPU tests run on; they fail (not skip) without one,
+    and without the built HIP library."""
+    import torch
+    from lmserve_amd import _lib
+
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    _lib.lib()  # raises if libkvcache.so is not built
+    return torch.device("cuda:0")

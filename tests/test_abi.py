@@ -1,0 +1,117 @@
+"""The C-ABI library loads and exports every symbol include/kvcache.h declares.
+
+No kernel is launched here: only symbol lookup and entry points that return
+before their first HIP call (argument validation, pure host arithmetic).
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from lmserve_amd import _lib
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(REPO, "include", "kvcache.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kvc_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_functions()
+    for must in ("kvc_reshape_and_cache", "kvc_reshape_and_cache_layers",
+                 "kvc_append_paged_kv_cache", "kvc_append_paged_kv_cache_layers",
+                 "kvc_get_seq_lens", "kvc_get_batch_indices_positions", "kvc_copy_blocks",
+                 "kvc_swap_out", "kvc_swap_in", "kvc_swap_staging_bytes",
+                 "kvc_host_alloc_pinned", "kvc_host_free_pinned", "kvc_last_error_string",
+                 "kvc_abi_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(handle, name), f"{name} is declared in kvcache.h but not exported"
+
+
+def test_python_binding_types_every_declared_symbol():
+    for name in declared_functions():
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature in lmserve_amd/_lib.py"
+
+
+def test_binding_arity_matches_the_header():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    for name, (_, argtypes) in _lib.SIGNATURES.items():
+        m = re.search(r"\b" + name + r"\s*\(([^;]*?)\)\s*;", text, flags=re.S)
+        if m is None:
+            continue  # tuning hook: exported, not part of the public header
+        params = m.group(1).strip()
+        n = 0 if params in ("", "void") else len(params.split(","))
+        assert n == len(argtypes), f"{name}: header has {n} parameters, binding {len(argtypes)}"
+
+
+def test_abi_version():
+    assert _lib.lib().kvc_abi_version() == 1
+
+
+def test_argument_validation_returns_codes_not_crashes():
+    L = _lib.lib()
+    assert L.kvc_copy_blocks(None, None, -1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
+    assert "negative" in _lib.last_error()
+    # empty work is OK even with null pointers
+    assert L.kvc_copy_blocks(None, None, 0, 32, 1 << 32, 65536, 65536, None) == _lib.KVC_OK
+    assert L.kvc_reshape_and_cache(None, None, None, None, None, 8, 0, 1024, 1024, 1024, 16,
+                                   32768, 1024, 64, 2, None) == _lib.KVC_OK
+    # unsupported element width / slot width
+    assert L.kvc_reshape_and_cache(1, 1, 1, 1, 1, 8, 4, 1024, 1024, 1024, 16, 32768, 1024, 64, 3,
+                                   None) == _lib.KVC_ERR_UNSUPPORTED
+    assert L.kvc_reshape_and_cache(256, 256, 256, 256, 256, 2, 4, 1024, 1024, 1024, 16, 32768,
+                                   1024, 64, 2, None) == _lib.KVC_ERR_UNSUPPORTED
+    # token stride smaller than a row
+    assert L.kvc_reshape_and_cache(256, 256, 256, 256, 256, 8, 4, 1024, 512, 1024, 16, 32768,
+                                   1024, 64, 2, None) == _lib.KVC_ERR_INVALID_ARG
+    with pytest.raises(ValueError):
+        _lib.check(_lib.KVC_ERR_INVALID_ARG)
+    with pytest.raises(TypeError):
+        _lib.check(_lib.KVC_ERR_UNSUPPORTED)
+    with pytest.raises(IndexError):
+        _lib.check(_lib.KVC_ERR_OUT_OF_RANGE)
+
+
+def test_swap_rejects_out_of_range_host_lists_before_touching_the_gpu():
+    L = _lib.lib()
+    src = np.asarray([0, 5, 99], dtype=np.int64)
+    dst = np.asarray([0, 1, 2], dtype=np.int64)
+    rc = L.kvc_swap_out(4096, 4096, src.ctypes.data, dst.ctypes.data, 3, 2, 64 * 1024, 1024, 64, 8,
+                        0, 2, 4096, 1 << 20, _lib.KVC_SWAP_STAGED, None, None)
+    assert rc == _lib.KVC_ERR_OUT_OF_RANGE and "99" in _lib.last_error()
+    rc = L.kvc_swap_in(4096, 4096, dst.ctypes.data, src.ctypes.data, 3, 2, 64 * 1024, 1024, 64, 8,
+                       0, 2, 4096, 1 << 20, _lib.KVC_SWAP_STAGED, None, None)
+    assert rc == _lib.KVC_ERR_OUT_OF_RANGE
+    # bad layer range, unknown mode, staging too small
+    ok = np.asarray([0, 1, 2], dtype=np.int64)
+    assert L.kvc_swap_out(4096, 4096, ok.ctypes.data, ok.ctypes.data, 3, 2, 64 * 1024, 1024, 64, 8,
+                          1, 3, 4096, 1 << 20, 0, None, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_swap_out(4096, 4096, ok.ctypes.data, ok.ctypes.data, 3, 2, 64 * 1024, 1024, 64, 8,
+                          0, 2, 4096, 1 << 20, 7, None, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_swap_out(4096, 4096, ok.ctypes.data, ok.ctypes.data, 3, 2, 64 * 1024, 1024, 64, 8,
+                          0, 2, 4096, 512, 0, None, None) == _lib.KVC_ERR_STAGING
+
+
+def test_staging_size_arithmetic():
+    L = _lib.lib()
+    blk, nl = 65536, 80
+    ids = 2 * 8192 * 8
+    # default ring slot: as many whole blocks as fit 64 MiB
+    per_block = nl * blk
+    chunk = (64 << 20) // per_block
+    assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 0) == ids + 2 * chunk * per_block
+    assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 4) == ids + 8 * per_block
+    assert L.kvc_swap_staging_bytes(3, nl, blk, _lib.KVC_SWAP_STAGED, 100) == 256 + 6 * per_block
+    assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_DIRECT, 0) == ids
+    assert L.kvc_swap_staging_bytes(-1, nl, blk, 0, 0) < 0

@@ -1,0 +1,177 @@
+"""GPU parity of the HBM <-> pinned-host swap against the CPU oracle (bit-exact
+on the whole host pool and the whole GPU pool), both transfer modes."""
+import asyncio
+
+import numpy as np
+import pytest
+import torch
+
+import lmserve_amd as kvc
+from lmserve_amd import workloads as wl
+from oracle import kvc_oracle as orc
+from tests.helpers import bits_of, random_pool, sentinel_pool, to_bf16
+
+pytestmark = pytest.mark.gpu
+
+MODES = ["staged", "direct"]
+
+
+def _mappings(src, dst, pieces=3):
+    """Split (src, dst) id lists into several BlockMappings, as one arrives per sequence."""
+    cuts = np.linspace(0, len(src), pieces + 1).astype(int)
+    return [kvc.BlockMapping.from_pairs(zip(src[a:b].tolist(), dst[a:b].tolist()))
+            for a, b in zip(cuts[:-1], cuts[1:])]
+
+
+def _worker(gpu, L, nb, block_shape, nhb, mode, chunk=0, seed=0):
+    pool = random_pool((L, nb) + block_shape, seed)
+    dpool = to_bf16(pool, gpu)
+    w = kvc.KVWorker(dpool, nhb, swap_mode=mode, staging_chunk_blocks=chunk)
+    w.host_kv_caches[...] = sentinel_pool(w.host_kv_caches.shape, seed + 1)
+    return pool, dpool, w
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("chunk", [0, 1, 3])
+def test_swap_out_then_in_matches_oracle(gpu, mode, chunk):
+    s = wl.LLAMA_3_8B
+    L, nb, nhb, n = 5, 64, 24, 11
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, mode, chunk, seed=chunk)
+    try:
+        rng = np.random.default_rng(10 + chunk)
+        perm = rng.permutation(nb)
+        old, new = perm[:n].astype(np.int64), perm[n:2 * n].astype(np.int64)
+        # host ids: a run of 4, singles, and a run of 3, so extents of every kind occur
+        host_ids = np.asarray([5, 6, 7, 8, 20, 2, 11, 12, 13, 0, 17], dtype=np.int64)
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        host_np = w.host_kv_caches.copy()
+        orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids)
+        w.copy_kv_sync(_mappings(old, host_ids), kvc.Device.GPU, kvc.Device.Host)
+        assert np.array_equal(w.host_kv_caches, host_np)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)   # pool untouched
+
+        orc.c_load_blocks_from_host(gpu_np, host_np, host_ids, new)
+        w.copy_kv_sync(_mappings(host_ids, new), kvc.Device.Host, kvc.Device.GPU)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+        assert np.array_equal(w.host_kv_caches, host_np)                    # host untouched
+        # round trip: payload of the old blocks now sits in the new blocks
+        assert np.array_equal(gpu_np[:, new], pool.reshape(L, nb, -1)[:, old])
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_swap_layer_ranges_compose_to_the_full_swap(gpu, mode):
+    """One call per layer range (the reference's layer-pipelined protocol) equals
+    one call for all layers, and each call touches only its own layers."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb, n = 6, 32, 16, 7
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, mode, chunk=2, seed=4)
+    try:
+        rng = np.random.default_rng(5)
+        old = rng.permutation(nb)[:n].astype(np.int64)
+        host_ids = rng.permutation(nhb)[:n].astype(np.int64)
+        maps = _mappings(old, host_ids, pieces=2)
+        gpu_np = pool.reshape(L, nb, -1)
+        host_np = w.host_kv_caches.copy()
+        for lb, le in ((0, 1), (1, 4), (4, 6)):
+            orc.save_blocks_to_host_np(gpu_np, host_np, old, host_ids, lb, le)
+            w.save_kv_blocks_to_host_nowait(maps, layer_begin=lb, layer_end=le)
+            w.dtoh_stream.synchronize()
+            assert np.array_equal(w.host_kv_caches, host_np), (lb, le)
+        full = sentinel_pool(host_np.shape, 5)
+        orc.c_save_blocks_to_host(gpu_np.copy(), full, old, host_ids)
+        assert np.array_equal(host_np[host_ids], full[host_ids])
+
+        new = np.setdiff1d(np.arange(nb), old)[:n].astype(np.int64)
+        back = _mappings(host_ids, new, pieces=1)
+        want = gpu_np.copy()
+        for lb, le in ((3, 6), (0, 3)):
+            orc.load_blocks_from_host_np(want, host_np, host_ids, new, lb, le)
+            w.load_kv_blocks_from_host_nowait(back, layer_begin=lb, layer_end=le)
+            w.htod_stream.synchronize()
+            assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), want), (lb, le)
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_swap_odd_block_bytes_and_other_dtypes(gpu, mode):
+    """Blocks whose byte size is not a multiple of 16, and fp32 / fp16 pools."""
+    for dtype, np_dtype, block_shape in ((torch.bfloat16, np.uint16, (2, 3, 1, 5)),
+                                         (torch.float16, np.float16, (2, 4, 2, 8)),
+                                         (torch.float32, np.float32, (2, 4, 1, 6))):
+        L, nb, nhb, n = 3, 20, 9, 6
+        rng = np.random.default_rng(11)
+        width = np.dtype(np_dtype).itemsize
+        raw = rng.integers(0, 1 << (8 * width), size=(L, nb) + block_shape,
+                           dtype=np.uint16 if width == 2 else np.uint32)
+        t = torch.from_numpy(raw.view(np.int16 if width == 2 else np.int32).copy()).view(dtype).to(gpu)
+        w = kvc.KVWorker(t, nhb, swap_mode=mode)
+        try:
+            assert w.host_kv_caches.dtype == np.dtype(np_dtype)
+            w.host_kv_caches.view(raw.dtype)[...] = 0
+            old = rng.permutation(nb)[:n].astype(np.int64)
+            hid = rng.permutation(nhb)[:n].astype(np.int64)
+            want = np.zeros((nhb, L, raw[0, 0].size), dtype=raw.dtype)
+            orc.c_save_blocks_to_host(raw.reshape(L, nb, -1), want, old, hid)
+            w.copy_kv_sync(_mappings(old, hid), kvc.Device.GPU, kvc.Device.Host)
+            assert np.array_equal(w.host_kv_caches.view(raw.dtype), want)
+        finally:
+            w.close()
+
+
+def test_copy_kv_async_dispatcher_errors_and_empty_lists(gpu):
+    pool, dpool, w = _worker(gpu, 2, 16, (2, 16, 1, 64), 8, "staged", seed=7)
+    try:
+        host0 = w.host_kv_caches.copy()
+        asyncio.run(w.copy_kv([], kvc.Device.GPU, kvc.Device.Host))       # no mappings: no-op
+        w.copy_kv_sync([kvc.BlockMapping()], kvc.Device.GPU, kvc.Device.Host)  # empty mapping
+        assert np.array_equal(w.host_kv_caches, host0)
+        with pytest.raises(ValueError, match="Unsupported copy direction"):
+            asyncio.run(w.copy_kv([], kvc.Device.GPU, kvc.Device.Disk))
+        with pytest.raises(ValueError, match="Unsupported copy direction"):
+            w.copy_kv_sync([], kvc.Device.GPU, kvc.Device.GPU)
+        with pytest.raises(IndexError):
+            w.copy_kv_sync([kvc.BlockMapping.from_pairs([(16, 0)])], kvc.Device.GPU, kvc.Device.Host)
+        with pytest.raises(IndexError):
+            w.copy_kv_sync([kvc.BlockMapping.from_pairs([(0, 8)])], kvc.Device.GPU, kvc.Device.Host)
+        assert np.array_equal(w.host_kv_caches, host0)
+        # the async path moves data too
+        maps = [kvc.BlockMapping.from_pairs([(3, 1), (9, 6)])]
+        asyncio.run(w.copy_kv(maps, kvc.Device.GPU, kvc.Device.Host))
+        want = host0.copy()
+        orc.save_blocks_to_host_np(pool.reshape(2, 16, -1), want, [3, 9], [1, 6])
+        assert np.array_equal(w.host_kv_caches, want)
+    finally:
+        w.close()
+    with pytest.raises(TypeError, match="Unsupported dtype"):
+        kvc.KVWorker(torch.zeros(2, 4, 8, dtype=torch.int8, device=gpu), 2)
+
+
+def test_disk_tier_round_trip(gpu, tmp_path):
+    """GPU -> Host -> Disk -> Host -> GPU carries the payload bit-exactly, and
+    the disk file is reopened when shape and dtype match."""
+    path = str(tmp_path / "disk-kv-cache-0.npy")
+    L, nb, nhb, ndb = 2, 16, 6, 5
+    pool, dpool, w = _worker(gpu, L, nb, (2, 16, 1, 64), nhb, "staged", seed=8)
+    try:
+        w.close()
+        w = kvc.KVWorker(dpool, nhb, num_disk_blocks=ndb, disk_kv_cache_file=path)
+        w.copy_kv_sync([kvc.BlockMapping.from_pairs([(2, 0), (7, 3)])], kvc.Device.GPU, kvc.Device.Host)
+        w.copy_kv_sync([kvc.BlockMapping.from_pairs([(0, 4), (3, 1)])], kvc.Device.Host, kvc.Device.Disk)
+        w.disk_kv_caches.flush()
+        w.close()
+        w = kvc.KVWorker(dpool, nhb, num_disk_blocks=ndb, disk_kv_cache_file=path)  # reopen
+        w.copy_kv_sync([kvc.BlockMapping.from_pairs([(4, 5), (1, 2)])], kvc.Device.Disk, kvc.Device.Host)
+        w.copy_kv_sync([kvc.BlockMapping.from_pairs([(5, 10), (2, 11)])], kvc.Device.Host, kvc.Device.GPU)
+        got = bits_of(dpool).reshape(L, nb, -1)
+        src = pool.reshape(L, nb, -1)
+        assert np.array_equal(got[:, 10], src[:, 2]) and np.array_equal(got[:, 11], src[:, 7])
+        with pytest.raises(ValueError):
+            kvc.KVWorker(dpool, nhb).copy_kv_sync([kvc.BlockMapping.from_pairs([(0, 0)])],
+                                                  kvc.Device.Host, kvc.Device.Disk)
+    finally:
+        w.close()

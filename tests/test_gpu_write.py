@@ -1,0 +1,271 @@
+"""GPU parity of the K/V write entry points against the CPU oracle (bit-exact).
+
+Every comparison is over the WHOLE destination pool, so stray writes show.
+"""
+import numpy as np
+import pytest
+import torch
+
+import lmserve_amd as kvc
+from lmserve_amd import _lib
+from lmserve_amd import workloads as wl
+from oracle import kvc_oracle as orc
+from tests.helpers import bf16_bits, bits_of, sentinel_pool, to_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, dev, dtype=torch.bfloat16):
+    """NumPy bit patterns -> device tensor of a same-width dtype."""
+    if dtype == torch.bfloat16 or dtype == torch.float16:
+        return torch.from_numpy(a.view(np.int16).copy()).view(dtype).to(dev)
+    return torch.from_numpy(a.view(np.int32).copy()).view(dtype).to(dev)
+
+
+def _host(t):
+    t = t.detach().cpu().contiguous()
+    if t.element_size() == 2:
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.view(torch.int32).numpy().view(np.uint32)
+
+
+def _bits(shape, seed, width):
+    if width == 2:
+        return bf16_bits(shape, seed)
+    rng = np.random.default_rng(seed)
+    return rng.integers(0, 1 << 32, size=shape, dtype=np.uint32)
+
+
+def _pool(shape, seed, width):
+    if width == 2:
+        return sentinel_pool(shape, seed)
+    rng = np.random.default_rng(seed + 1000)
+    return rng.integers(0, 1 << 32, size=shape, dtype=np.uint32)
+
+
+FILL_CASES = [
+    # T, H, D, num_slots, dtype, slot dtype
+    (256, 8, 64, 64 * 16, torch.bfloat16, torch.int64),    # config-1 rows, reduced pool
+    (256, 8, 128, 96 * 16, torch.bfloat16, torch.int64),   # Llama-3-8B rows
+    (77, 4, 128, 200, torch.float16, torch.int32),
+    (33, 3, 5, 64, torch.bfloat16, torch.int64),           # 30-byte rows: 2-byte vectors
+    (19, 1, 6, 40, torch.bfloat16, torch.int64),           # 12-byte rows: 4-byte vectors
+    (21, 1, 4, 40, torch.bfloat16, torch.int32),           # 8-byte rows
+    (50, 2, 64, 128, torch.float32, torch.int64),
+    (1, 8, 128, 16, torch.bfloat16, torch.int64),
+    (0, 8, 128, 16, torch.bfloat16, torch.int64),
+]
+
+
+@pytest.mark.parametrize("T,H,D,num_slots,dtype,slot_dtype", FILL_CASES)
+def test_fill_key_cache_matches_oracle(gpu, T, H, D, num_slots, dtype, slot_dtype):
+    width = torch.empty(0, dtype=dtype).element_size()
+    rng = np.random.default_rng(T * 131 + H)
+    slots = rng.permutation(num_slots)[:T].astype(np.int64)
+    key, value = _bits((T, H, D), 1, width), _bits((T, H, D), 2, width)
+    kc, vc = _pool((num_slots, H, D), 3, width), _pool((num_slots, H, D), 4, width)
+    want_k, want_v = kc.copy(), vc.copy()
+    orc.c_fill_key_cache(key, value, want_k, want_v, slots)
+    dk, dv = _dev(kc, gpu, dtype), _dev(vc, gpu, dtype)
+    kvc.fill_key_cache(_dev(key, gpu, dtype), _dev(value, gpu, dtype), dk, dv,
+                       torch.from_numpy(slots).to(gpu).to(slot_dtype))
+    torch.cuda.synchronize()
+    assert np.array_equal(_host(dk), want_k)
+    assert np.array_equal(_host(dv), want_v)
+
+
+@pytest.mark.parametrize("vpt", [1, 2, 4])
+@pytest.mark.parametrize("nt", [0, 1])
+def test_fill_key_cache_every_launch_shape(gpu, vpt, nt):
+    """All vectors-per-lane / store-kind instantiations give the same bits."""
+    T, H, D, num_slots = 301, 8, 128, 512
+    rng = np.random.default_rng(7)
+    slots = rng.permutation(num_slots)[:T].astype(np.int64)
+    key, value = bf16_bits((T, H, D), 1), bf16_bits((T, H, D), 2)
+    kc, vc = sentinel_pool((num_slots, H, D), 3), sentinel_pool((num_slots, H, D), 4)
+    want_k, want_v = kc.copy(), vc.copy()
+    orc.fill_key_cache_np(key, value, want_k, want_v, slots)
+    dk, dv = to_bf16(kc, gpu), to_bf16(vc, gpu)
+    _lib.set_tuning("write_vpt", vpt)
+    _lib.set_tuning("write_nt", nt)
+    try:
+        kvc.fill_key_cache(to_bf16(key, gpu), to_bf16(value, gpu), dk, dv,
+                           torch.from_numpy(slots).to(gpu))
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_tuning("write_vpt", 0)
+        _lib.set_tuning("write_nt", 0)
+    assert np.array_equal(bits_of(dk), want_k) and np.array_equal(bits_of(dv), want_v)
+
+
+def test_config1_llama_1b_write_all_layers(gpu):
+    """BASELINE config 1 at its full size: 16 layers, pool of 1024 blocks, 256
+    tokens on seeded random distinct free slots; per-layer op and the one-launch
+    form must both equal the oracle on the whole 512 MiB pool."""
+    s = wl.LLAMA_3_2_1B
+    nb, T = 1024, 256
+    slots = wl.random_free_slots(s, nb, T, seed=0)
+    L, H, D, bs = s.num_layers, s.num_kv_heads, s.head_dim, s.block_size
+    key, value = bf16_bits((L, T, H, D), 10), bf16_bits((L, T, H, D), 11)
+    pool = sentinel_pool((L, nb, 2, bs, H, D), 12)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
+    dkey, dval = to_bf16(key, gpu), to_bf16(value, gpu)
+    dslots = torch.from_numpy(slots).to(gpu)
+
+    per_layer = to_bf16(pool, gpu)
+    for l in range(L):
+        kvc.reshape_and_cache(dkey[l], dval[l], per_layer[l], dslots)
+    fused = to_bf16(pool, gpu)
+    kvc.reshape_and_cache_layers(dkey, dval, fused, dslots)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(per_layer), want)
+    assert np.array_equal(bits_of(fused), want)
+
+
+def test_reshape_and_cache_strided_tokens_and_guarded_slots(gpu):
+    """K/V rows taken as slices of a fused projection (token stride > row), and
+    slots that are negative or beyond the pool are skipped, not written."""
+    T, H, D, nb, bs = 40, 2, 64, 8, 16
+    rng = np.random.default_rng(3)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    fused = bf16_bits((T, 3 * H * D), 5)
+    key = np.ascontiguousarray(fused[:, H * D:2 * H * D]).reshape(T, H, D)
+    value = np.ascontiguousarray(fused[:, 2 * H * D:]).reshape(T, H, D)
+    bad = slots.copy()
+    bad[3] = -1
+    bad[17] = nb * bs
+    bad[29] = nb * bs + 5
+    keep = np.asarray([i for i in range(T) if i not in (3, 17, 29)])
+    pool = sentinel_pool((nb, 2, bs, H, D), 6)
+    want = pool.copy()
+    orc.c_reshape_and_cache(np.ascontiguousarray(key[keep]), np.ascontiguousarray(value[keep]),
+                            want, slots[keep])
+    dfused = to_bf16(fused, gpu)
+    dk = dfused[:, H * D:2 * H * D].view(T, H, D)
+    dv = dfused[:, 2 * H * D:].view(T, H, D)
+    assert not dk.is_contiguous()
+    dpool = to_bf16(pool, gpu)
+    kvc.reshape_and_cache(dk, dv, dpool, torch.from_numpy(bad).to(gpu))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), want)
+
+
+def _paged_case(gpu, workload, L, seed):
+    s = workload.shape
+    nb, bs, H, D = workload.num_blocks, s.block_size, s.num_kv_heads, s.head_dim
+    idx = workload.index
+    T = workload.num_tokens
+    key, value = bf16_bits((L, T, H, D), seed), bf16_bits((L, T, H, D), seed + 1)
+    pool = sentinel_pool((L, nb, 2, bs, H, D), seed + 2)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_append_paged_kv_cache(key[l], value[l], idx.batch_indices, idx.positions, want[l],
+                                    idx.kv_block_indices, idx.kv_block_indptrs)
+    # the slot-mapped oracle must agree (scheduler rule), before the GPU is involved
+    want2 = pool.copy()
+    for l in range(L):
+        orc.reshape_and_cache_np(key[l], value[l], want2[l], idx.slot_mapping)
+    assert np.array_equal(want, want2)
+    dev = kvc.to_device(idx, bs, gpu)
+    dkey, dval = to_bf16(key, gpu), to_bf16(value, gpu)
+    return pool, want, dev, dkey, dval
+
+
+@pytest.mark.parametrize("kind", ["decode", "chunked_prefill", "mixed"])
+def test_append_paged_kv_cache_matches_oracle(gpu, kind):
+    if kind == "decode":
+        w = wl.decode_step(wl.LLAMA_3_8B, num_blocks=512, batch=48, max_context=150, seed=1)
+    elif kind == "chunked_prefill":
+        w = wl.chunked_prefill(wl.QWEN_2_5_7B, num_blocks=512, num_seqs=4, chunk_tokens=256,
+                               min_context=100, max_context=1500, seed=2)
+    else:
+        rng = np.random.default_rng(9)
+        filled = [0, 37, 5, 64, 200, 16, 15]
+        new = [70, 1, 1, 33, 1, 16, 2]
+        w = wl._write_workload(wl.LLAMA_3_2_1B, 256, filled, new, rng)
+    L = 3
+    pool, want, dev, dkey, dval = _paged_case(gpu, w, L, 40)
+    # device-side index prep must reproduce the host arrays
+    assert np.array_equal(dev.batch_indices.cpu().numpy(), w.index.batch_indices)
+    assert np.array_equal(dev.positions.cpu().numpy(), w.index.positions)
+
+    per_layer = to_bf16(pool, gpu)
+    for l in range(L):
+        kvc.append_paged_kv_cache(dkey[l], dval[l], dev.batch_indices, dev.positions, per_layer[l],
+                                  dev.kv_block_indices, dev.kv_block_indptrs, dev.kv_last_block_lens)
+    fused = to_bf16(pool, gpu)
+    kvc.append_paged_kv_cache_layers(dkey, dval, dev.batch_indices, dev.positions, fused,
+                                     dev.kv_block_indices, dev.kv_block_indptrs,
+                                     dev.kv_last_block_lens)
+    slotted = to_bf16(pool, gpu)
+    kvc.reshape_and_cache_layers(dkey, dval, slotted, dev.slot_mapping)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(per_layer), want)
+    assert np.array_equal(bits_of(fused), want)
+    assert np.array_equal(bits_of(slotted), want)
+
+
+def test_append_paged_skips_tokens_with_bad_indices(gpu):
+    w = wl.decode_step(wl.LLAMA_3_2_1B, num_blocks=64, batch=8, max_context=60, seed=4)
+    s = w.shape
+    idx = w.index
+    T, H, D, bs, nb = w.num_tokens, s.num_kv_heads, s.head_dim, s.block_size, w.num_blocks
+    key, value = bf16_bits((T, H, D), 1), bf16_bits((T, H, D), 2)
+    pool = sentinel_pool((nb, 2, bs, H, D), 3)
+    bi = idx.batch_indices.copy()
+    pos = idx.positions.copy()
+    bi[2] = -1          # no such request
+    bi[5] = 8           # beyond the batch
+    pos[6] = 1 << 20    # beyond the page table
+    keep = np.asarray([0, 1, 3, 4, 7])
+    want = pool.copy()
+    orc.c_append_paged_kv_cache(np.ascontiguousarray(key[keep]), np.ascontiguousarray(value[keep]),
+                                bi[keep], pos[keep], want, idx.kv_block_indices,
+                                idx.kv_block_indptrs)
+    dpool = to_bf16(pool, gpu)
+
+    def up(a):
+        return torch.from_numpy(a).to(gpu)
+
+    kvc.append_paged_kv_cache(to_bf16(key, gpu), to_bf16(value, gpu), up(bi), up(pos), dpool,
+                              up(idx.kv_block_indices), up(idx.kv_block_indptrs),
+                              up(idx.kv_last_block_lens))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), want)
+
+
+def test_write_runs_on_the_current_stream(gpu):
+    """The op is enqueued on torch's current stream: a copy of the pool taken on
+    the same side stream right after the call must already see the write."""
+    T, H, D, nb, bs = 64, 8, 128, 32, 16
+    rng = np.random.default_rng(2)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    key, value = bf16_bits((T, H, D), 1), bf16_bits((T, H, D), 2)
+    pool = sentinel_pool((nb, 2, bs, H, D), 3)
+    want = pool.copy()
+    orc.reshape_and_cache_np(key, value, want, slots)
+    dk, dv, dpool, ds = to_bf16(key, gpu), to_bf16(value, gpu), to_bf16(pool, gpu), \
+        torch.from_numpy(slots).to(gpu)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        kvc.reshape_and_cache(dk, dv, dpool, ds)
+        snap = dpool.clone()
+    side.synchronize()
+    assert np.array_equal(bits_of(snap), want)
+
+
+def test_dtype_mismatch_raises(gpu):
+    k = torch.zeros(2, 1, 8, dtype=torch.float16, device=gpu)
+    pool = torch.zeros(4, 2, 4, 1, 8, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(TypeError):
+        kvc.reshape_and_cache(k, k, pool, torch.zeros(2, dtype=torch.int64, device=gpu))
+    with pytest.raises(TypeError):
+        kvc.append_paged_kv_cache(k.bfloat16(), k.bfloat16(),
+                                  torch.zeros(2, dtype=torch.int64, device=gpu),
+                                  torch.zeros(2, dtype=torch.int32, device=gpu), pool,
+                                  torch.zeros(2, dtype=torch.int32, device=gpu),
+                                  torch.zeros(2, dtype=torch.int32, device=gpu),
+                                  torch.zeros(1, dtype=torch.int32, device=gpu))

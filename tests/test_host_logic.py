@@ -1,0 +1,171 @@
+"""Host-side logic of the operator surface: pair-list flattening, mapping
+flattening, index construction, workload generators, and the loud failures of
+the operators when they are handed CPU tensors."""
+import numpy as np
+import pytest
+import torch
+
+import lmserve_amd as kvc
+from lmserve_amd import workloads as wl
+from lmserve_amd.index_prep import InferInput, make_kv_index_inputs
+from oracle import kvc_oracle as orc
+
+
+def test_flatten_block_maps_keeps_dict_order_and_fans_out():
+    assert kvc.flatten_block_maps({}) == []
+    assert kvc.flatten_block_maps({5: [1, 2], 3: [9]}) == [5, 1, 5, 2, 3, 9]
+
+
+def test_check_block_maps():
+    kvc.check_block_maps([0, 1, 2, 3, 4, 4], 8)          # self pair is fine
+    with pytest.raises(IndexError):
+        kvc.check_block_maps([0, 8], 8)
+    with pytest.raises(ValueError):
+        kvc.check_block_maps([0, 2, 1, 2], 8)            # duplicate dst
+    with pytest.raises(ValueError):
+        kvc.check_block_maps([0, 1, 1, 2], 8)            # chain: 1 is dst and src
+
+
+def test_flatten_block_mappings_concatenates_in_order():
+    a = kvc.BlockMapping.from_pairs([(1, 10), (2, 11)])
+    b = kvc.BlockMapping.from_pairs([(7, 3)])
+    src, dst = kvc.flatten_block_mappings([a, kvc.BlockMapping(), b])
+    assert src.tolist() == [1, 2, 7] and dst.tolist() == [10, 11, 3]
+    assert src.dtype == np.int64
+    src, dst = kvc.flatten_block_mappings([])
+    assert src.shape == (0,)
+
+
+def test_device_enum_matches_the_wire_values():
+    assert (int(kvc.Device.GPU), int(kvc.Device.Host), int(kvc.Device.Disk)) == (0, 1, 2)
+
+
+def test_make_kv_index_inputs_orders_prefill_first_and_builds_the_page_table():
+    bs = 4
+    inputs = [
+        InferInput(0, [1], 1, 6, 7, [3, 9]),                 # decode
+        InferInput(1, [1] * 5, 5, 0, 5, [4, 2]),             # prefill chunk
+        InferInput(2, [1], 1, 3, 4, [7]),                    # decode
+        InferInput(3, [1] * 3, 3, 8, 11, [1, 5, 6]),         # chunked prefill continuation
+    ]
+    idx = make_kv_index_inputs(inputs, bs)
+    assert idx.order == [1, 3, 0, 2]                         # stable sort by -input_len
+    assert idx.cu_seqlens_q.tolist() == [0, 5, 8, 9, 10]
+    assert idx.prefill_input_len == 8
+    assert idx.position_ids.tolist() == [0, 1, 2, 3, 4, 8, 9, 10, 6, 3]
+    assert idx.kv_block_indices.tolist() == [4, 2, 1, 5, 6, 3, 9, 7]
+    assert idx.kv_block_indptrs.tolist() == [0, 2, 5, 7, 8]
+    assert idx.kv_last_block_lens.tolist() == [1, 3, 3, 4]
+    assert idx.batch_indices.tolist() == [0] * 5 + [1] * 3 + [2, 3]
+    # slot(pos) = table[pos // bs] * bs + pos % bs
+    assert idx.slot_mapping.tolist() == [16, 17, 18, 19, 8, 24, 25, 26, 9 * 4 + 2, 7 * 4 + 3]
+    # and the page-table oracles give the same (batch, position) pairs from these arrays
+    seq_lens = orc.get_seq_lens_np(idx.kv_block_indptrs, idx.kv_last_block_lens, bs)
+    bi, pos = orc.get_batch_indices_positions_np(idx.cu_seqlens_q, seq_lens, 10)
+    assert bi.tolist() == idx.batch_indices.tolist() and pos.tolist() == idx.positions.tolist()
+
+
+def test_make_kv_index_inputs_rejects_inconsistent_requests():
+    with pytest.raises(ValueError):
+        make_kv_index_inputs([InferInput(0, [1, 1], 2, 0, 3, [0])], 4)   # len mismatch
+    with pytest.raises(ValueError):
+        make_kv_index_inputs([InferInput(0, [1] * 5, 5, 0, 5, [0])], 4)  # too few blocks
+
+
+def test_workloads_have_the_configured_shapes_and_distinct_slots():
+    s = wl.random_free_slots()
+    assert s.shape == (256,) and len(set(s.tolist())) == 256 and s.max() < 1024 * 16
+    assert np.array_equal(s, wl.random_free_slots())         # seeded
+
+    dec = wl.decode_step(num_blocks=65536, batch=256)
+    assert dec.num_tokens == 256 and dec.shape.row_bytes == 2048
+    slots = dec.index.slot_mapping
+    assert len(set(slots.tolist())) == 256 and slots.max() < 65536 * 16
+    for req in dec.inputs:
+        assert req.input_len == 1 and req.context_len == req.filled_token_len + 1
+    assert dec.algorithmic_bytes(1) == 2 * 256 * 2 * 2048 + 8 * 256
+
+    pre = wl.chunked_prefill()
+    assert pre.num_tokens == 2048 and pre.shape.row_bytes == 1024
+    assert len(set(pre.index.slot_mapping.tolist())) == 2048
+    for req in pre.inputs:
+        assert 1024 <= req.filled_token_len <= 32768 and req.input_len == 512
+
+    flat, d = wl.copy_on_write_pairs()
+    assert flat.shape == (8192,) and len(d) == 4096
+    kvc.check_block_maps(flat.tolist(), 65536)
+    assert kvc.flatten_block_maps(d) == flat.tolist()
+
+    out_ids, host_ids, in_ids = wl.swap_round_trip()
+    assert len(set(out_ids.tolist()) | set(in_ids.tolist())) == 16384
+    assert host_ids.tolist() == list(range(8192))
+
+
+def test_kv_shapes():
+    assert wl.LLAMA_3_8B.block_bytes == 64 * 1024 and wl.LLAMA_3_2_1B.block_bytes == 32 * 1024
+    assert wl.QWEN_2_5_7B.row_bytes == 1024 and wl.LLAMA_3_1_70B.num_layers == 80
+
+
+def test_operators_refuse_cpu_tensors_loudly():
+    pool = torch.zeros(2, 4, 2, 4, 1, 8, dtype=torch.bfloat16)
+    k = torch.zeros(3, 1, 8, dtype=torch.bfloat16)
+    slots = torch.zeros(3, dtype=torch.int64)
+    i32 = torch.zeros(3, dtype=torch.int32)
+    with pytest.raises(ValueError, match="GPU"):
+        kvc.copy_blocks(pool, {0: [1]})
+    with pytest.raises(ValueError, match="GPU"):
+        kvc.fill_key_cache(k, k, pool[0, :, 0], pool[0, :, 1], slots)
+    with pytest.raises(ValueError, match="GPU"):
+        kvc.reshape_and_cache(k, k, pool[0], slots)
+    with pytest.raises(ValueError, match="GPU"):
+        kvc.append_paged_kv_cache(k, k, i32, i32, pool[0], i32, i32, i32)
+    with pytest.raises(ValueError, match="GPU"):
+        kvc.KVWorker(pool, 4)
+
+
+def test_torch_cpu_statements_agree_with_the_oracle():
+    """The multi-threaded torch-CPU baseline is itself checked against the oracle."""
+    from oracle import torch_cpu
+    from tests.helpers import bf16_bits, random_pool, sentinel_pool, to_bf16, bits_of
+
+    T, H, D, nb, bs, L = 40, 2, 8, 16, 4, 3
+    rng = np.random.default_rng(1)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    key, value = bf16_bits((T, H, D), 2), bf16_bits((T, H, D), 3)
+    pool = sentinel_pool((nb, 2, bs, H, D), 4)
+    want = pool.copy()
+    orc.c_reshape_and_cache(key, value, want, slots)
+    got = to_bf16(pool)
+    torch_cpu.reshape_and_cache_cpu(to_bf16(key), to_bf16(value), got, torch.from_numpy(slots))
+    assert np.array_equal(bits_of(got), want)
+
+    kc, vc = sentinel_pool((nb * bs, H, D), 5), sentinel_pool((nb * bs, H, D), 6)
+    wk, wv = kc.copy(), vc.copy()
+    orc.c_fill_key_cache(key, value, wk, wv, slots)
+    gk, gv = to_bf16(kc), to_bf16(vc)
+    torch_cpu.fill_key_cache_cpu(to_bf16(key), to_bf16(value), gk, gv, torch.from_numpy(slots))
+    assert np.array_equal(bits_of(gk), wk) and np.array_equal(bits_of(gv), wv)
+
+    big = random_pool((L, nb, 2, bs, H, D), 7)
+    perm = rng.permutation(nb)
+    src, dst = perm[:4].astype(np.int64), perm[4:8].astype(np.int64)
+    want = big.copy()
+    orc.c_copy_blocks(want, np.stack([src, dst], 1).reshape(-1))
+    got = to_bf16(big)
+    torch_cpu.copy_blocks_cpu(got, torch.from_numpy(src), torch.from_numpy(dst))
+    assert np.array_equal(bits_of(got), want)
+
+    gpu = random_pool((L, nb, 32), 8)
+    host = sentinel_pool((6, L, 32), 9)
+    want_host = host.copy()
+    hid = np.asarray([4, 0, 5, 2], dtype=np.int64)
+    orc.c_save_blocks_to_host(gpu, want_host, src, hid)
+    got_host = torch.from_numpy(host.view(np.int16).copy())
+    torch_cpu.swap_out_cpu(torch.from_numpy(gpu.view(np.int16)), got_host, torch.from_numpy(src),
+                           torch.from_numpy(hid))
+    assert np.array_equal(got_host.numpy().view(np.uint16), want_host)
+    want_gpu = gpu.copy()
+    orc.c_load_blocks_from_host(want_gpu, want_host, hid, dst)
+    got_gpu = torch.from_numpy(gpu.view(np.int16).copy())
+    torch_cpu.swap_in_cpu(got_gpu, got_host, torch.from_numpy(hid), torch.from_numpy(dst))
+    assert np.array_equal(got_gpu.numpy().view(np.uint16), want_gpu)
