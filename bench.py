@@ -7,15 +7,17 @@ Headline (`value`): BASELINE config 2, the Llama-3-8B decode-step KV write
 (256 sequences x 1 new token, 32 layers, 8 KV heads x 128, block_size 16, bf16,
 pool of 65536 blocks = 128 GiB). One step = the K/V write of one decode step
 over all 32 layers through `kvc_reshape_and_cache_layers` (one launch). Inputs
-are resident in HBM before the timed region; K/V sources and slot sets rotate
-between steps so no step finds its lines in the 256 MiB last-level cache.
+are resident in HBM before the timed region. K/V sources and slot sets rotate
+over 16 sets (512 MiB of sources) so no step finds its lines in the 256 MiB
+last-level cache. The K timed steps are K eager launches on torch's current
+stream; `ops` repeats the measurement with the launches replayed from a hipGraph.
 
 The same JSON line carries `roofline` (algorithmic bytes of one launch over the
-kernel's mean duration measured with events on the launch stream, against
+launch's mean duration measured with events on the launch stream, against
 8 TB/s), `cpu_baseline` (the torch-CPU statement of the same step on the host
 cores, bounded sample) and `ops`: every other configuration and entry point
 (per-layer launches, page-table addressing, chunked prefill, copy_blocks, swap)
-with its own µs/call and GB/s.
+with its own us/call and GB/s.
 """
 from __future__ import annotations
 
@@ -30,7 +32,8 @@ if REPO_ROOT not in sys.path:
     sys.path.insert(0, REPO_ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-ROTATE = 8  # distinct K/V source buffers and slot sets cycled through
+ROTATE_DECODE = 16   # 16 x 32 MiB of K/V sources
+ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 
 
 def log(*a):
@@ -40,30 +43,58 @@ def log(*a):
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=200)
-    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--steps", type=int, default=320)
+    p.add_argument("--warmup", type=int, default=32)
     p.add_argument("--ops", default="write,prefill,copy,swap",
-                   help="comma list of extra measurements: write (per-layer/paged variants), "
-                        "prefill, copy, swap; 'none' for the headline only")
+                   help="comma list of extra measurements: write (per-layer / page-table variants "
+                        "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
+                        "calib (a plain 1 GiB device copy, for counter calibration); "
+                        "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=1024,
-                   help="blocks per swap direction (config 5 uses 8192 = 40 GiB pinned)")
+                   help="blocks per swap direction (config 5 itself is 8192 = 40 GiB pinned)")
     p.add_argument("--pool-blocks", type=int, default=65536)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
     return p.parse_args()
 
 
-def time_region(fn, steps, warmup, torch):
-    """W untimed + K timed calls of fn(i); returns (wall ms/step, event ms/step)."""
+def time_region(fn, steps, warmup, torch, graph_of=0):
+    """W untimed + K timed calls of fn(i); returns (wall ms/step, event ms/step).
+
+    graph_of > 0: the launches of `graph_of` consecutive steps are captured once
+    into a hipGraph and the timed region replays it (steps // graph_of) times,
+    then runs the remaining steps eagerly -- exactly K steps either way, without
+    the host's per-launch cost between them."""
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
+    graph = None
+    if graph_of > 0 and steps >= graph_of:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(graph_of):
+                fn(i)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(graph_of):
+                fn(i)
+        graph.replay()
+        torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    for i in range(steps):
-        fn(warmup + i)
+    if graph is not None:
+        for _ in range(steps // graph_of):
+            graph.replay()
+        for i in range(steps % graph_of):
+            fn(i)
+    else:
+        for i in range(steps):
+            fn(warmup + i)
     end.record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -75,7 +106,8 @@ def entry(name, bytes_per_call, ms_wall, ms_event, calls_per_step=1, **extra):
     gbps = bytes_per_call / (us * 1e-6) / 1e9 if us > 0 else 0.0
     d = {"name": name, "us_per_call": round(us, 3), "gbps": round(gbps, 1),
          "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
-         "bytes_per_call": int(bytes_per_call), "wall_us_per_call": round(ms_wall * 1e3 / calls_per_step, 3)}
+         "bytes_per_call": int(bytes_per_call),
+         "wall_us_per_call": round(ms_wall * 1e3 / calls_per_step, 3)}
     d.update(extra)
     return d
 
@@ -92,92 +124,75 @@ def alloc_pool(torch, shape_cfg, num_blocks, dev):
     raise RuntimeError("cannot allocate the KV pool")
 
 
-def write_inputs(torch, np, kvc, workload_fn, shape_cfg, L, num_blocks, dev, **kw):
-    """ROTATE sets of (key, value, slot_mapping, paged index tensors) for a write config."""
+def write_inputs(torch, kvc, workload_fn, shape_cfg, L, num_blocks, dev, rotate, **kw):
+    """`rotate` sets of (workload, key, value, device index tensors) for a write config."""
     sets = []
-    for r in range(ROTATE):
+    for r in range(rotate):
         w = workload_fn(shape_cfg, num_blocks=num_blocks, seed=r, **kw)
-        T = w.num_tokens
-        key = torch.randn(L, T, shape_cfg.num_kv_heads, shape_cfg.head_dim, device=dev,
+        key = torch.randn(L, w.num_tokens, shape_cfg.num_kv_heads, shape_cfg.head_dim, device=dev,
                           dtype=torch.float32).to(torch.bfloat16)
         value = torch.randn_like(key)
-        idx = kvc.to_device(w.index, shape_cfg.block_size, dev)
-        sets.append((w, key, value, idx))
+        sets.append((w, key, value, kvc.to_device(w.index, shape_cfg.block_size, dev)))
     return sets
 
 
-def bench_write_config(torch, np, kvc, tag, sets, pool, L, steps, warmup, variants):
-    """Measure the write entry points on one configuration. Returns list of entries."""
-    out = []
+def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
+    """Measure the write entry points on one configuration.
+    Returns (list of entries, {variant: (wall ms, event ms)})."""
+    out, results = [], {}
+    R = len(sets)
     w0 = sets[0][0]
     bytes_fused = w0.algorithmic_bytes(L)
     bytes_layer = w0.algorithmic_bytes(1)
 
     def fused_slot(i):
-        _, k, v, idx = sets[i % ROTATE]
+        _, k, v, idx = sets[i % R]
         kvc.reshape_and_cache_layers(k, v, pool, idx.slot_mapping)
 
     def fused_paged(i):
-        _, k, v, idx = sets[i % ROTATE]
+        _, k, v, idx = sets[i % R]
         kvc.append_paged_kv_cache_layers(k, v, idx.batch_indices, idx.positions, pool,
                                          idx.kv_block_indices, idx.kv_block_indptrs,
                                          idx.kv_last_block_lens)
 
     def per_layer_paged(i):
-        _, k, v, idx = sets[i % ROTATE]
+        _, k, v, idx = sets[i % R]
         for l in range(L):
             kvc.append_paged_kv_cache(k[l], v[l], idx.batch_indices, idx.positions, pool[l],
                                       idx.kv_block_indices, idx.kv_block_indptrs,
                                       idx.kv_last_block_lens)
 
     def per_layer_slot(i):
-        _, k, v, idx = sets[i % ROTATE]
+        _, k, v, idx = sets[i % R]
         for l in range(L):
             kvc.reshape_and_cache(k[l], v[l], pool[l], idx.slot_mapping)
 
-    results = {}
-    if "fused_slot" in variants:
-        ms_w, ms_e = time_region(fused_slot, steps, warmup, torch)
-        results["fused_slot"] = (ms_w, ms_e)
-        out.append(entry(f"{tag}/reshape_and_cache_layers (1 launch, {L} layers)", bytes_fused,
-                         ms_w, ms_e))
-    if "fused_paged" in variants:
-        ms_w, ms_e = time_region(fused_paged, steps, warmup, torch)
-        out.append(entry(f"{tag}/append_paged_kv_cache_layers (1 launch, {L} layers)", bytes_fused,
-                         ms_w, ms_e))
-    if "per_layer_paged" in variants:
-        n = max(5, steps // 8)
-        ms_w, ms_e = time_region(per_layer_paged, n, max(2, warmup // 4), torch)
-        out.append(entry(f"{tag}/append_paged_kv_cache (per layer, {L} launches per step)",
-                         bytes_layer, ms_w, ms_e, calls_per_step=L))
-    if "per_layer_slot" in variants:
-        n = max(5, steps // 8)
-        ms_w, ms_e = time_region(per_layer_slot, n, max(2, warmup // 4), torch)
-        out.append(entry(f"{tag}/reshape_and_cache (per layer, {L} launches per step)",
-                         bytes_layer, ms_w, ms_e, calls_per_step=L))
-    if "per_layer_graph" in variants:
-        # the per-layer launches of one step captured once and replayed: what a
-        # graph-captured decode loop pays per layer
+    table = {
+        "fused_slot": (fused_slot, f"reshape_and_cache_layers (1 launch, {L} layers)", bytes_fused, 1),
+        "fused_paged": (fused_paged, f"append_paged_kv_cache_layers (1 launch, {L} layers)",
+                        bytes_fused, 1),
+        "per_layer_paged": (per_layer_paged, f"append_paged_kv_cache (per layer, {L} launches per step)",
+                            bytes_layer, L),
+        "per_layer_slot": (per_layer_slot, f"reshape_and_cache (per layer, {L} launches per step)",
+                           bytes_layer, L),
+    }
+    for variant in variants:
+        name, mode = variant.split(":")
+        fn, label, nbytes, calls = table[name]
+        n = steps if calls == 1 else max(R, steps // 8 // R * R)
+        wu = warmup if calls == 1 else max(2, warmup // 8)
         try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                per_layer_paged(0)
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                per_layer_paged(0)
-            n = max(5, steps // 4)
-            ms_w, ms_e = time_region(lambda i: graph.replay(), n, 3, torch)
-            out.append(entry(f"{tag}/append_paged_kv_cache (per layer, hipGraph replay of {L} launches)",
-                             bytes_layer, ms_w, ms_e, calls_per_step=L))
-        except Exception as exc:  # graph capture is an extra, never the headline
-            log(f"hipGraph variant skipped: {exc!r}")
+            ms_w, ms_e = time_region(fn, n, wu, torch, graph_of=R if mode == "graph" else 0)
+        except Exception as exc:  # a failed graph capture never takes the bench down
+            log(f"{tag}/{label} [{mode}] skipped: {exc!r}")
+            continue
+        results[variant] = (ms_w, ms_e)
+        out.append(entry(f"{tag}/{label}", nbytes, ms_w, ms_e, calls_per_step=calls,
+                         launch="hipGraph replay" if mode == "graph" else "eager (Python + ctypes per call)"))
     return out, results
 
 
-def cpu_baseline_write(torch, np, shape_cfg, L, seconds):
+def cpu_baseline_write(torch, shape_cfg, L, seconds):
     """torch-CPU statement of the same step on a pool scaled to fit host RAM
     (same tokens, same rows, same bytes moved)."""
     from lmserve_amd import workloads as wl
@@ -197,7 +212,7 @@ def cpu_baseline_write(torch, np, shape_cfg, L, seconds):
         torch_cpu.reshape_and_cache_layers_cpu(key, value, pool, slots)
         n += 1
         el = time.perf_counter() - t0
-        if el >= seconds or n >= 2000:
+        if el >= seconds or n >= 20000:
             break
     per_step = el / n
     gbps = w.algorithmic_bytes(L) / per_step / 1e9
@@ -214,7 +229,6 @@ def main():
         print("bench.py measures one GPU only: this path has no cross-GPU step "
               f"(--gpus {args.gpus} is not supported)", file=sys.stderr)
         sys.exit(2)
-    import numpy as np
     import torch
 
     import lmserve_amd as kvc
@@ -232,15 +246,16 @@ def main():
     s8 = wl.LLAMA_3_8B
     pool, L = alloc_pool(torch, s8, args.pool_blocks, dev)
     log(f"pool {tuple(pool.shape)} = {pool.numel() * 2 / 2**30:.1f} GiB")
-    sets = write_inputs(torch, np, kvc, wl.decode_step, s8, L, args.pool_blocks, dev, batch=256)
-    variants = ["fused_slot"]
+    sets = write_inputs(torch, kvc, wl.decode_step, s8, L, args.pool_blocks, dev, ROTATE_DECODE,
+                        batch=256)
+    variants = ["fused_slot:eager"]
     if "write" in ops:
-        variants += ["fused_paged", "per_layer_paged", "per_layer_slot", "per_layer_graph"]
-    entries, res = bench_write_config(torch, np, kvc, "cfg2 decode", sets, pool, L, args.steps,
+        variants += ["fused_slot:graph", "fused_paged:eager", "per_layer_paged:graph",
+                     "per_layer_slot:graph", "per_layer_paged:eager"]
+    entries, res = bench_write_config(torch, kvc, "cfg2 decode", sets, pool, L, args.steps,
                                       args.warmup, variants)
-    ms_wall, ms_event = res["fused_slot"]
-    head = entries[0]
     extra += entries[1:]
+    ms_wall, ms_event = res["fused_slot:eager"]
     bytes_step = sets[0][0].algorithmic_bytes(L)
     value_gbps = bytes_step / (ms_wall * 1e-3) / 1e9
     achieved = bytes_step / (ms_event * 1e-3) / 1e9
@@ -248,25 +263,33 @@ def main():
 
     # ------------------------------------------------ config 4: copy_blocks (same pool)
     if "copy" in ops:
-        flat, _ = wl.copy_on_write_pairs(args.pool_blocks, 4096, seed=0)
         maps = [torch.from_numpy(wl.copy_on_write_pairs(args.pool_blocks, 4096, seed=r)[0]).to(dev)
                 for r in range(2)]
         nbytes = 2 * 4096 * L * s8.block_bytes + 16 * 4096
         ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool, maps[i % 2]),
                                  max(5, min(args.steps, 20)), 3, torch)
         extra.append(entry(f"cfg4 copy_blocks (4096 pairs x {L} layers, 64 KiB blocks)", nbytes,
-                           ms_w, ms_e))
+                           ms_w, ms_e, launch="eager"))
     del pool
     torch.cuda.empty_cache()
+
+    if "calib" in ops:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        ms_w, ms_e = time_region(lambda i: b.copy_(a), 10, 2, torch)
+        extra.append(entry("calibration: plain device copy of 1 GiB (torch copy_)", 2 << 30, ms_w, ms_e,
+                           launch="eager"))
+        del a, b
+        torch.cuda.empty_cache()
 
     # ------------------------------------------------ config 3: chunked-prefill write
     if "prefill" in ops:
         sq = wl.QWEN_2_5_7B
         pool3, L3 = alloc_pool(torch, sq, 16384, dev)
-        sets3 = write_inputs(torch, np, kvc, wl.chunked_prefill, sq, L3, 16384, dev)
-        e3, _ = bench_write_config(torch, np, kvc, "cfg3 chunked prefill", sets3, pool3, L3,
-                                   max(10, args.steps // 2), max(3, args.warmup // 2),
-                                   ["fused_slot", "fused_paged", "per_layer_paged"])
+        sets3 = write_inputs(torch, kvc, wl.chunked_prefill, sq, L3, 16384, dev, ROTATE_PREFILL)
+        e3, _ = bench_write_config(torch, kvc, "cfg3 chunked prefill", sets3, pool3, L3,
+                                   max(ROTATE_PREFILL, args.steps // 2), max(3, args.warmup // 2),
+                                   ["fused_slot:graph", "fused_paged:graph", "per_layer_paged:graph"])
         extra += e3
         del sets3, pool3
         torch.cuda.empty_cache()
@@ -281,11 +304,12 @@ def main():
         out_maps = [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))]
         in_maps = [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))]
         nbytes = n * L5 * s70.block_bytes
-        for mode in ("staged", "direct"):
+        for mode in ("direct", "staged"):
             worker = kvc.KVWorker(pool5, n, swap_mode=mode)
             try:
-                for direction, maps, src, dst in (("swap_out", out_maps, kvc.Device.GPU, kvc.Device.Host),
-                                                  ("swap_in", in_maps, kvc.Device.Host, kvc.Device.GPU)):
+                for direction, maps, src, dst in (
+                        ("swap_out", out_maps, kvc.Device.GPU, kvc.Device.Host),
+                        ("swap_in", in_maps, kvc.Device.Host, kvc.Device.GPU)):
                     worker.copy_kv_sync(maps, src, dst)  # warm-up (first touch of the pinned pool)
                     times = []
                     for _ in range(3):
@@ -305,7 +329,7 @@ def main():
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline_write(torch, np, s8, L, args.cpu_seconds)
+        cpu = cpu_baseline_write(torch, s8, L, args.cpu_seconds)
 
     line = {
         "metric": "achieved HBM GB/s, KV write (Llama-3-8B decode step)",
@@ -324,9 +348,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": "BASELINE config 2: Llama-3-8B decode-step KV write, 256 seqs x 1 token, "
                                f"{L} layers, 8 KV heads x 128, block_size 16, bf16 lanes, pool "
-                               f"{args.pool_blocks} blocks ({L * args.pool_blocks * s8.block_bytes / 2**30:.0f} GiB)",
+                               f"{args.pool_blocks} blocks "
+                               f"({L * args.pool_blocks * s8.block_bytes / 2**30:.0f} GiB)",
                    "entry": "kvc_reshape_and_cache_layers (all layers in one launch)",
-                   "rotation": f"{ROTATE} K/V source sets and slot sets cycled"},
+                   "launch": "one eager launch per step on torch's current stream",
+                   "rotation": f"{ROTATE_DECODE} K/V source sets and slot sets cycled"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel": "write_rows_kernel", "bytes_per_launch": int(bytes_step),

@@ -57,7 +57,7 @@ const char* kvc_last_error_string(void);
 /* Launch-shape knobs for measurement sweeps; process-wide, not thread-safe
  * against concurrent launches. No counterpart in the reference. Keys:
  * "copy_unroll" (1,2,4,8,16), "copy_nt" (0/1), "copy_max_wgs" (0 = one
- * workgroup per chunk), "write_vpt" (0 = by size, 1, 2, 4), "write_nt" (0/1),
+ * workgroup per chunk), "write_vpt" (0 = by size, 1, 2, 4, 8), "write_nt" (bit 0: non-temporal stores, bit 1: loads), "write_order" (0/1),
  * "direct_max_wgs". Unknown key: KVC_ERR_INVALID_ARG. */
 int kvc_set_tuning(const char* key, int value);
 

@@ -57,7 +57,30 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
 
 
 def _stream_of(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    """Raw hipStream_t of torch's current stream on the tensor's device."""
+    return torch._C._cuda_getCurrentRawStream(t.device.index)
+
+
+class _on_device_of:
+    """Make the tensor's device current for the launch; free when it already is
+    (the common case), unlike `torch.cuda.device`, which always switches twice."""
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, t: torch.Tensor):
+        self.idx = t.device.index
+        self.prev = -1
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 def copy_blocks(
@@ -95,7 +118,7 @@ def copy_blocks(
     elem = kv_caches.element_size()
     numel_per_layer = kv_caches[0].numel()
     numel_per_block = numel_per_layer // num_blocks
-    with torch.cuda.device(kv_caches.device):
+    with _on_device_of(kv_caches):
         _lib.check(_lib.lib().kvc_copy_blocks(
             kv_caches.data_ptr(), block_maps_tensor.data_ptr(), num_pairs, num_layers,
             numel_per_layer * elem, numel_per_block * elem, num_blocks, _stream_of(kv_caches)))
@@ -151,7 +174,7 @@ def fill_key_cache(
     if not slot_mapping.is_contiguous():
         slot_mapping = slot_mapping.contiguous()
     num_slots = min(key_cache.numel(), value_cache.numel()) // row
-    with torch.cuda.device(key_cache.device):
+    with _on_device_of(key_cache):
         _lib.check(_lib.lib().kvc_reshape_and_cache(
             key.data_ptr(), value.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
             slot_mapping.data_ptr(), slot_bytes, num_tokens, row, k_stride, v_stride,
@@ -200,7 +223,7 @@ def reshape_and_cache(
     slot_mapping, slot_bytes = _slot_args(slot_mapping)
     elem = kv_cache.element_size()
     block_stride = kv_cache.stride(0) if nb > 1 else 2 * bs * row
-    with torch.cuda.device(kv_cache.device):
+    with _on_device_of(kv_cache):
         _lib.check(_lib.lib().kvc_reshape_and_cache(
             key.data_ptr(), value.data_ptr(), kv_cache.data_ptr(),
             kv_cache.data_ptr() + bs * row * elem, slot_mapping.data_ptr(), slot_bytes,
@@ -241,7 +264,7 @@ def reshape_and_cache_layers(
         return
     slot_mapping, slot_bytes = _slot_args(slot_mapping)
     elem = kv_caches.element_size()
-    with torch.cuda.device(kv_caches.device):
+    with _on_device_of(kv_caches):
         _lib.check(_lib.lib().kvc_reshape_and_cache_layers(
             key.data_ptr(), value.data_ptr(), kv_caches.data_ptr(),
             kv_caches.data_ptr() + bs * row * elem, slot_mapping.data_ptr(), slot_bytes,

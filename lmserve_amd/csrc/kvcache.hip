@@ -3,11 +3,13 @@
 // Three kernels carry the whole path; all are HBM-bound byte movers, so the
 // design is about coalescing and bytes in flight, not arithmetic:
 //
-//   write_rows_kernel   one 16-byte vector per lane, lanes of a wavefront cover
-//                       consecutive vectors of a token row: the source side is a
-//                       dense stream, the cache side is one contiguous row per
-//                       (token, K|V, layer). blockIdx.y = (layer, K|V) so every
-//                       base pointer is wave-uniform.
+//   write_rows_kernel   a workgroup owns ONE token and a run of 16-byte vectors
+//                       out of that token's rows (K and V of every layer in
+//                       the launch). The slot lookup is workgroup-uniform, so
+//                       the index chain is resolved once on the scalar unit and
+//                       each lane only streams: VPT loads issued back to back,
+//                       then VPT stores; lanes of a wavefront cover consecutive
+//                       vectors of a row on both sides.
 //   copy_tiles_kernel   a "tile" is one block of one layer (block_bytes
 //                       contiguous on both sides). A workgroup owns a chunk of
 //                       256 lanes x UNROLL x 16 bytes, issues all its loads
@@ -63,7 +65,8 @@ struct Tuning {
   int copy_nt = 1;          // non-temporal loads/stores in copy_tiles
   int copy_max_wgs = 0;     // 0 = one workgroup per chunk, else grid cap
   int write_vpt = 0;        // vectors per lane in write_rows, 0 = by size
-  int write_nt = 0;         // non-temporal stores in write_rows
+  int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
+  int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
   int direct_max_wgs = 512; // grid cap of the direct (PCIe-bound) swap kernel
 };
 Tuning g_tune;
@@ -110,80 +113,110 @@ struct WriteArgs {
   int64_t batch_size;
   int64_t num_kv_indices;
   // geometry; every stride in BYTES
-  uint32_t num_tokens;     // tokens of this launch (host splits huge T)
+  uint32_t num_tokens;       // tokens of this launch (host splits huge T)
   uint32_t vecs_per_row;
-  int vpr_shift;           // log2(vecs_per_row) or -1
+  int vpr_shift;             // log2(vecs_per_row) or -1
+  uint32_t items_per_token;  // 2 * num_layers * vecs_per_row; item = (layer, K|V, vec)
+  uint32_t num_groups;       // workgroups per token
+  int groups_fastest;        // blockIdx.x = token * num_groups + group (else group * T + token)
   int64_t key_token_stride, value_token_stride;
   int64_t key_layer_stride, value_layer_stride;
   int64_t block_size;
-  int bs_shift;            // log2(block_size) or -1
+  int bs_shift;              // log2(block_size) or -1
   int64_t cache_block_stride, cache_slot_stride, cache_layer_stride;
   int64_t num_cache_blocks;
 };
 
-template <int VEC, int VPT, bool PAGED, bool NT>
+// One workgroup = one token x a run of VPT*blockDim.x vectors out of the
+// token's 2*L rows (K and V of every layer). The token, hence its slot and
+// every base address, is uniform across the workgroup.
+// Order of work: the source addresses need only the token, so every lane first
+// issues its VPT independent 16-byte loads; the index chain (slot_mapping, or
+// batch_indices -> kv_indptr -> kv_indices) is resolved on the scalar unit
+// while those loads are in flight; the stores follow. A token whose slot is
+// invalid simply returns with its loads unused.
+template <int VEC, int VPT, bool PAGED, bool NT, bool NTL>
 __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   using V = typename VecOf<VEC>::type;
-  const uint32_t layer = blockIdx.y >> 1;
-  const uint32_t is_v = blockIdx.y & 1u;
-  const char* src_base = (is_v ? a.value + (int64_t)layer * a.value_layer_stride
-                               : a.key + (int64_t)layer * a.key_layer_stride);
-  char* dst_base = (is_v ? a.value_cache : a.key_cache) + (int64_t)layer * a.cache_layer_stride;
-  const int64_t tok_stride = is_v ? a.value_token_stride : a.key_token_stride;
-  const uint32_t total = a.num_tokens * a.vecs_per_row;  // host guarantees < 2^31
-
-  V data[VPT];
-  char* dst[VPT];
-#pragma unroll
-  for (int j = 0; j < VPT; ++j) {
-    const uint32_t g = (blockIdx.x * VPT + j) * kThreads + threadIdx.x;
-    dst[j] = nullptr;
-    if (g >= total) continue;
-    uint32_t t, vec;
-    if (a.vpr_shift >= 0) {
-      t = g >> a.vpr_shift;
-      vec = g & (a.vecs_per_row - 1u);
-    } else {
-      t = g / a.vecs_per_row;
-      vec = g - t * a.vecs_per_row;
-    }
-    int64_t blk, off;
-    if constexpr (PAGED) {
-      const int64_t b = a.batch_indices[t];
-      const int64_t p = a.positions[t];
-      if (b < 0 || b >= a.batch_size || p < 0) continue;
-      int64_t pg, e;
-      if (a.bs_shift >= 0) {
-        pg = p >> a.bs_shift;
-        e = p & (a.block_size - 1);
-      } else {
-        pg = p / a.block_size;
-        e = p - pg * a.block_size;
-      }
-      const int64_t it = (int64_t)a.kv_indptr[b] + pg;
-      if (it < 0 || it >= a.num_kv_indices) continue;
-      blk = a.kv_indices[it];
-      off = e;
-    } else {
-      const int64_t s = (a.slot_bytes == 8)
-                            ? reinterpret_cast<const int64_t*>(a.slot_mapping)[t]
-                            : (int64_t) reinterpret_cast<const int32_t*>(a.slot_mapping)[t];
-      if (s < 0) continue;
-      if (a.bs_shift >= 0) {
-        blk = s >> a.bs_shift;
-        off = s & (a.block_size - 1);
-      } else {
-        blk = s / a.block_size;
-        off = s - blk * a.block_size;
-      }
-    }
-    if (blk < 0 || blk >= a.num_cache_blocks) continue;
-    data[j] = *reinterpret_cast<const V*>(src_base + (int64_t)t * tok_stride + (int64_t)vec * VEC);
-    dst[j] = dst_base + blk * a.cache_block_stride + off * a.cache_slot_stride + (int64_t)vec * VEC;
+  // blockIdx.x = group * num_tokens + token by default: neighbouring workgroups
+  // read neighbouring token rows of the same layers
+  uint32_t group, t;
+  if (a.groups_fastest) {
+    t = blockIdx.x / a.num_groups;
+    group = blockIdx.x - t * a.num_groups;
+  } else {
+    group = blockIdx.x / a.num_tokens;
+    t = blockIdx.x - group * a.num_tokens;
   }
+  const char* key_row = a.key + (int64_t)t * a.key_token_stride;
+  const char* value_row = a.value + (int64_t)t * a.value_token_stride;
+  const uint32_t first = group * (VPT * blockDim.x) + threadIdx.x;
+  V data[VPT];
+  int64_t dst_off[VPT];  // offset inside the slot's row set, < 0 = no item
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    if (dst[j]) st<NT>(reinterpret_cast<V*>(dst[j]), data[j]);
+    const uint32_t item = first + j * blockDim.x;
+    dst_off[j] = -1;
+    if (item < a.items_per_token) {
+      uint32_t r, vec;
+      if (a.vpr_shift >= 0) {
+        r = item >> a.vpr_shift;
+        vec = item & (a.vecs_per_row - 1u);
+      } else {
+        r = item / a.vecs_per_row;
+        vec = item - r * a.vecs_per_row;
+      }
+      const int64_t layer = r >> 1;
+      const bool is_v = r & 1u;
+      const char* src = (is_v ? value_row + layer * a.value_layer_stride
+                              : key_row + layer * a.key_layer_stride) + (int64_t)vec * VEC;
+      data[j] = ld<NTL>(reinterpret_cast<const V*>(src));
+      // bit 0 carries K|V; VEC-aligned offsets leave it free only for VEC >= 2,
+      // so keep the flag in the sign-safe top instead: offsets are far below 2^62
+      dst_off[j] = (layer * a.cache_layer_stride + (int64_t)vec * VEC) | ((int64_t)is_v << 62);
+    }
+  }
+
+  int64_t blk, off;
+  if constexpr (PAGED) {
+    const int64_t b = a.batch_indices[t];
+    const int64_t p = a.positions[t];
+    if (b < 0 || b >= a.batch_size || p < 0) return;
+    int64_t pg;
+    if (a.bs_shift >= 0) {
+      pg = p >> a.bs_shift;
+      off = p & (a.block_size - 1);
+    } else {
+      pg = p / a.block_size;
+      off = p - pg * a.block_size;
+    }
+    const int64_t it = (int64_t)a.kv_indptr[b] + pg;
+    if (it < 0 || it >= a.num_kv_indices) return;
+    blk = a.kv_indices[it];
+  } else {
+    const int64_t s = (a.slot_bytes == 8)
+                          ? reinterpret_cast<const int64_t*>(a.slot_mapping)[t]
+                          : (int64_t) reinterpret_cast<const int32_t*>(a.slot_mapping)[t];
+    if (s < 0) return;
+    if (a.bs_shift >= 0) {
+      blk = s >> a.bs_shift;
+      off = s & (a.block_size - 1);
+    } else {
+      blk = s / a.block_size;
+      off = s - blk * a.block_size;
+    }
+  }
+  if (blk < 0 || blk >= a.num_cache_blocks) return;
+  const int64_t slot_off = blk * a.cache_block_stride + off * a.cache_slot_stride;
+  char* kc_row = a.key_cache + slot_off;
+  char* vc_row = a.value_cache + slot_off;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    if (dst_off[j] >= 0) {
+      const bool is_v = (dst_off[j] >> 62) & 1;
+      char* dst = (is_v ? vc_row : kc_row) + (dst_off[j] & ~(int64_t(1) << 62));
+      st<NT>(reinterpret_cast<V*>(dst), data[j]);
+    }
   }
 }
 
@@ -293,33 +326,41 @@ inline int common_vec(std::initializer_list<uint64_t> vals) {
   return (int)acc;
 }
 
+struct WriteLaunch {
+  unsigned grid;     // workgroups
+  unsigned threads;  // lanes per workgroup
+  int vpt;
+  bool nt;   // non-temporal stores
+  bool ntl;  // non-temporal loads
+};
+
 template <int VEC, int VPT, bool PAGED>
-void launch_write_nt(const WriteArgs& a, dim3 grid, hipStream_t s, bool nt) {
-  if (nt) hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, true>), grid, dim3(kThreads), 0, s, a);
-  else hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, false>), grid, dim3(kThreads), 0, s, a);
+void launch_write_nt(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
+  const dim3 grid(l.grid), block(l.threads);
+  if (l.nt && l.ntl) hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, true, true>), grid, block, 0, s, a);
+  else if (l.nt) hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, true, false>), grid, block, 0, s, a);
+  else if (l.ntl) hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, false, true>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((write_rows_kernel<VEC, VPT, PAGED, false, false>), grid, block, 0, s, a);
 }
 
 template <int VEC, bool PAGED>
-void launch_write_vpt(const WriteArgs& a, int vpt, uint32_t layers2, hipStream_t s, bool nt) {
-  const uint64_t total = (uint64_t)a.num_tokens * a.vecs_per_row;
-  auto grid = [&](int v) {
-    return dim3((unsigned)((total + (uint64_t)kThreads * v - 1) / ((uint64_t)kThreads * v)), layers2, 1);
-  };
-  switch (vpt) {
-    case 1: launch_write_nt<VEC, 1, PAGED>(a, grid(1), s, nt); break;
-    case 2: launch_write_nt<VEC, 2, PAGED>(a, grid(2), s, nt); break;
-    default: launch_write_nt<VEC, 4, PAGED>(a, grid(4), s, nt); break;
+void launch_write_vpt(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
+  switch (l.vpt) {
+    case 1: launch_write_nt<VEC, 1, PAGED>(a, l, s); break;
+    case 2: launch_write_nt<VEC, 2, PAGED>(a, l, s); break;
+    case 4: launch_write_nt<VEC, 4, PAGED>(a, l, s); break;
+    default: launch_write_nt<VEC, 8, PAGED>(a, l, s); break;
   }
 }
 
 template <bool PAGED>
-void launch_write(const WriteArgs& a, int vec, int vpt, uint32_t layers2, hipStream_t s, bool nt) {
+void launch_write(const WriteArgs& a, int vec, const WriteLaunch& l, hipStream_t s) {
   switch (vec) {
-    case 16: launch_write_vpt<16, PAGED>(a, vpt, layers2, s, nt); break;
-    case 8: launch_write_vpt<8, PAGED>(a, vpt, layers2, s, nt); break;
-    case 4: launch_write_vpt<4, PAGED>(a, vpt, layers2, s, nt); break;
-    case 2: launch_write_vpt<2, PAGED>(a, vpt, layers2, s, nt); break;
-    default: launch_write_vpt<1, PAGED>(a, vpt, layers2, s, nt); break;
+    case 16: launch_write_vpt<16, PAGED>(a, l, s); break;
+    case 8: launch_write_vpt<8, PAGED>(a, l, s); break;
+    case 4: launch_write_vpt<4, PAGED>(a, l, s); break;
+    case 2: launch_write_vpt<2, PAGED>(a, l, s); break;
+    default: launch_write_vpt<1, PAGED>(a, l, s); break;
   }
 }
 
@@ -408,27 +449,43 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
   a.cache_layer_stride = g.cache_layer_stride * E;
   a.num_cache_blocks = g.num_cache_blocks;
 
-  // bytes one launch moves decide how many vectors a lane carries: small
-  // launches are latency-bound and want every lane busy with one vector.
-  const int64_t launch_bytes = g.num_tokens * g.row_elems * E * 2 * g.num_layers;
-  int vpt = g_tune.write_vpt;
-  if (vpt <= 0) vpt = launch_bytes >= (int64_t(32) << 20) ? 4 : (launch_bytes >= (int64_t(8) << 20) ? 2 : 1);
-  const bool nt = g_tune.write_nt != 0;
+  const int64_t items64 = 2 * g.num_layers * (int64_t)a.vecs_per_row;
+  if (items64 > 0x7fffffffll)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
+  a.items_per_token = (uint32_t)items64;
 
-  // keep token*vecs_per_row inside 31 bits per launch
-  const int64_t max_tokens = std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / a.vecs_per_row - 4 * kThreads);
+  // Vectors per lane: a small launch is latency-bound and wants every lane busy
+  // with one vector; a large one wants several loads in flight per lane.
+  const int64_t launch_bytes = g.num_tokens * g.row_elems * E * 2 * g.num_layers;
+  WriteLaunch l{};
+  l.vpt = g_tune.write_vpt;
+  if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8)
+    l.vpt = launch_bytes >= (int64_t(32) << 20) ? 4 : (launch_bytes >= (int64_t(8) << 20) ? 2 : 1);
+  while (l.vpt > 1 && (int64_t)(l.vpt / 2) * kThreads >= items64) l.vpt /= 2;
+  const int64_t lanes = (items64 + l.vpt - 1) / l.vpt;
+  l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes + 63) / 64 * 64);
+  l.nt = (g_tune.write_nt & 1) != 0;
+  l.ntl = (g_tune.write_nt & 2) != 0;
+  const int64_t groups = (items64 + (int64_t)l.vpt * l.threads - 1) / ((int64_t)l.vpt * l.threads);
+
+  a.num_groups = (uint32_t)groups;
+  a.groups_fastest = g_tune.write_order;
+
+  // keep groups * tokens inside 31 bits per launch
+  const int64_t max_tokens = std::max<int64_t>(1, 0x7fffffffll / groups);
   for (int64_t t0 = 0; t0 < g.num_tokens; t0 += max_tokens) {
-    const int64_t nt_tok = std::min(max_tokens, g.num_tokens - t0);
-    a.num_tokens = (uint32_t)nt_tok;
+    const int64_t n_tok = std::min(max_tokens, g.num_tokens - t0);
+    a.num_tokens = (uint32_t)n_tok;
+    l.grid = (unsigned)(n_tok * groups);
     a.key = (const char*)key + t0 * a.key_token_stride;
     a.value = (const char*)value + t0 * a.value_token_stride;
     if (paged) {
       a.batch_indices = batch_indices + t0;
       a.positions = positions + t0;
-      launch_write<true>(a, vec, vpt, (uint32_t)(g.num_layers * 2), (hipStream_t)stream, nt);
+      launch_write<true>(a, vec, l, (hipStream_t)stream);
     } else {
       a.slot_mapping = (const char*)slot_mapping + t0 * slot_bytes;
-      launch_write<false>(a, vec, vpt, (uint32_t)(g.num_layers * 2), (hipStream_t)stream, nt);
+      launch_write<false>(a, vec, l, (hipStream_t)stream);
     }
     KVC_HIP(hipGetLastError());
   }
@@ -754,6 +811,7 @@ int kvc_set_tuning(const char* key, int value) {
   else if (!strcmp(key, "copy_max_wgs")) g_tune.copy_max_wgs = value;
   else if (!strcmp(key, "write_vpt")) g_tune.write_vpt = value;
   else if (!strcmp(key, "write_nt")) g_tune.write_nt = value;
+  else if (!strcmp(key, "write_order")) g_tune.write_order = value;
   else if (!strcmp(key, "direct_max_wgs")) g_tune.direct_max_wgs = value;
   else return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: unknown key '%s'", key);
   return KVC_OK;

@@ -17,7 +17,7 @@ from typing import Tuple
 import torch
 
 from . import _lib
-from .cache_ops import _require_gpu, _rows, _stream_of
+from .cache_ops import _on_device_of, _require_gpu, _rows, _stream_of
 
 
 def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
@@ -36,7 +36,7 @@ def get_seq_lens(kv_indptr: torch.Tensor, kv_last_page_len: torch.Tensor,
     if kv_indptr.numel() != batch_size + 1:
         raise ValueError("kv_indptr must have batch_size + 1 entries")
     seq_lens = torch.empty(batch_size, dtype=torch.int32, device=kv_indptr.device)
-    with torch.cuda.device(kv_indptr.device):
+    with _on_device_of(kv_indptr):
         _lib.check(_lib.lib().kvc_get_seq_lens(
             kv_indptr.data_ptr(), kv_last_page_len.data_ptr(), batch_size, int(page_size),
             seq_lens.data_ptr(), _stream_of(kv_indptr)))
@@ -59,7 +59,7 @@ def get_batch_indices_positions(append_indptr: torch.Tensor, seq_lens: torch.Ten
         raise ValueError("append_indptr must have batch_size + 1 entries")
     batch_indices = torch.empty(int(nnz), dtype=torch.int32, device=append_indptr.device)
     positions = torch.empty(int(nnz), dtype=torch.int32, device=append_indptr.device)
-    with torch.cuda.device(append_indptr.device):
+    with _on_device_of(append_indptr):
         _lib.check(_lib.lib().kvc_get_batch_indices_positions(
             append_indptr.data_ptr(), seq_lens.data_ptr(), batch_size, int(nnz),
             batch_indices.data_ptr(), positions.data_ptr(), _stream_of(append_indptr)))
@@ -122,7 +122,7 @@ def append_paged_kv_cache(
     if nnz == 0 or row == 0 or num_pages == 0:
         return
     page_stride = paged_kv_cache.stride(0) if num_pages > 1 else 2 * page_size * row
-    with torch.cuda.device(paged_kv_cache.device):
+    with _on_device_of(paged_kv_cache):
         _lib.check(_lib.lib().kvc_append_paged_kv_cache(
             append_key.data_ptr(), append_value.data_ptr(), batch_indices.data_ptr(),
             positions.data_ptr(), paged_kv_cache.data_ptr(), kv_indices.data_ptr(),
@@ -170,7 +170,7 @@ def append_paged_kv_cache_layers(
         raise ValueError("fewer key/value rows than index entries")
     if nnz == 0 or row == 0 or num_pages == 0 or L == 0:
         return
-    with torch.cuda.device(kv_caches.device):
+    with _on_device_of(kv_caches):
         _lib.check(_lib.lib().kvc_append_paged_kv_cache_layers(
             append_key.data_ptr(), append_value.data_ptr(), batch_indices.data_ptr(),
             positions.data_ptr(), kv_caches.data_ptr(), kv_indices.data_ptr(),

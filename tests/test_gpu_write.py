@@ -74,8 +74,8 @@ def test_fill_key_cache_matches_oracle(gpu, T, H, D, num_slots, dtype, slot_dtyp
     assert np.array_equal(_host(dv), want_v)
 
 
-@pytest.mark.parametrize("vpt", [1, 2, 4])
-@pytest.mark.parametrize("nt", [0, 1])
+@pytest.mark.parametrize("vpt", [1, 2, 4, 8])
+@pytest.mark.parametrize("nt", [0, 1, 2, 3])
 def test_fill_key_cache_every_launch_shape(gpu, vpt, nt):
     """All vectors-per-lane / store-kind instantiations give the same bits."""
     T, H, D, num_slots = 301, 8, 128, 512
@@ -94,7 +94,7 @@ def test_fill_key_cache_every_launch_shape(gpu, vpt, nt):
         torch.cuda.synchronize()
     finally:
         _lib.set_tuning("write_vpt", 0)
-        _lib.set_tuning("write_nt", 0)
+        _lib.set_tuning("write_nt", 1)
     assert np.array_equal(bits_of(dk), want_k) and np.array_equal(bits_of(dv), want_v)
 
 
