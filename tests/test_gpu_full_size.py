@@ -1,0 +1,161 @@
+"""The BASELINE configurations at their full sizes, checked through properties
+that do not need a CPU copy of the pool: gather-back of the written rows, a
+census of changed elements over the whole pool, a closed-form block pattern
+for copy and swap, and the swap-out -> swap-in round trip."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import lmserve_amd as kvc
+from lmserve_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+SWAP_BLOCKS = int(os.environ.get("KVC_TEST_SWAP_BLOCKS", "8192"))
+
+
+def _check_write(pool, key, value, slots_np, bs):
+    """pool [L, nb, 2, bs, H, D] was all-zero before the write."""
+    L = pool.shape[0]
+    dev = pool.device
+    slots = torch.from_numpy(slots_np).to(dev)
+    blk, off = slots // bs, slots % bs
+    written = 0
+    for l in range(L):
+        assert torch.equal(pool[l][blk, 0, off], key[l]), f"layer {l}: K rows differ"
+        assert torch.equal(pool[l][blk, 1, off], value[l]), f"layer {l}: V rows differ"
+        nz = int(torch.count_nonzero(pool[l].view(torch.int16)))
+        want = int(torch.count_nonzero(key[l].view(torch.int16))) + \
+            int(torch.count_nonzero(value[l].view(torch.int16)))
+        assert nz == want, f"layer {l}: {nz} non-zero elements in the pool, {want} were written"
+        written += nz
+    return written
+
+
+def _clear_slots(pool, slots_np, bs):
+    slots = torch.from_numpy(slots_np).to(pool.device)
+    pool[:, slots // bs, :, slots % bs] = 0
+
+
+def test_config2_decode_write_full_pool(gpu):
+    """Llama-3-8B decode step on the 128 GiB pool: one-launch and per-layer forms,
+    slot-mapped and page-table addressed."""
+    s = wl.LLAMA_3_8B
+    nb, L, bs = 65536, s.num_layers, s.block_size
+    w = wl.decode_step(s, num_blocks=nb, batch=256, seed=0)
+    pool = torch.zeros(L, nb, 2, bs, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16, device=gpu)
+    assert pool[0].numel() == 2 ** 31          # one layer overflows 32-bit element offsets
+    key = torch.randn(L, 256, s.num_kv_heads, s.head_dim, device=gpu).to(torch.bfloat16)
+    value = torch.randn_like(key)
+    idx = kvc.to_device(w.index, bs, gpu)
+    slots = w.index.slot_mapping
+    assert (slots.max() // bs) * s.block_elems >= 2 ** 31 - 2 ** 27   # blocks reach the top of a layer
+
+    kvc.reshape_and_cache_layers(key, value, pool, idx.slot_mapping)
+    assert _check_write(pool, key, value, slots, bs) > 0
+    _clear_slots(pool, slots, bs)
+    assert int(torch.count_nonzero(pool[L - 1].view(torch.int16))) == 0
+
+    kvc.append_paged_kv_cache_layers(key, value, idx.batch_indices, idx.positions, pool,
+                                     idx.kv_block_indices, idx.kv_block_indptrs, idx.kv_last_block_lens)
+    _check_write(pool, key, value, slots, bs)
+    _clear_slots(pool, slots, bs)
+
+    for l in range(L):
+        kvc.append_paged_kv_cache(key[l], value[l], idx.batch_indices, idx.positions, pool[l],
+                                  idx.kv_block_indices, idx.kv_block_indptrs, idx.kv_last_block_lens)
+    _check_write(pool, key, value, slots, bs)
+
+
+def test_config3_chunked_prefill_write_full(gpu):
+    """Qwen2.5-7B: a 2048-token chunk over 4 sequences with 1k-32k of context."""
+    s = wl.QWEN_2_5_7B
+    nb, L, bs = 16384, s.num_layers, s.block_size
+    w = wl.chunked_prefill(s, num_blocks=nb, seed=0)
+    assert w.num_tokens == 2048
+    pool = torch.zeros(L, nb, 2, bs, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16, device=gpu)
+    key = torch.randn(L, 2048, s.num_kv_heads, s.head_dim, device=gpu).to(torch.bfloat16)
+    value = torch.randn_like(key)
+    idx = kvc.to_device(w.index, bs, gpu)
+    assert np.array_equal(idx.positions.cpu().numpy(), w.index.position_ids)
+    kvc.append_paged_kv_cache_layers(key, value, idx.batch_indices, idx.positions, pool,
+                                     idx.kv_block_indices, idx.kv_block_indptrs, idx.kv_last_block_lens)
+    _check_write(pool, key, value, w.index.slot_mapping, bs)
+    _clear_slots(pool, w.index.slot_mapping, bs)
+    for l in range(L):
+        kvc.reshape_and_cache(key[l], value[l], pool[l], idx.slot_mapping)
+    _check_write(pool, key, value, w.index.slot_mapping, bs)
+
+
+def _pattern_terms(nb, block_elems, dev):
+    blk = (torch.arange(nb, device=dev, dtype=torch.int64) * 7919 + 13).to(torch.int16)
+    elem = (torch.arange(block_elems, device=dev, dtype=torch.int64) * 31 + 5).to(torch.int16)
+    return blk, elem
+
+
+def _fill_pattern(pool3, blk_term, elem_term):
+    """pool3 [L, nb, E] int16: value(l, b, e) = blk_term[b] + elem_term[e] + 257*l (wrapping)."""
+    for l in range(pool3.shape[0]):
+        torch.add(blk_term[:, None], elem_term[None, :] + 257 * l, out=pool3[l])
+
+
+def _check_pattern(pool3, holder_of, blk_term, elem_term, what):
+    """Block b of every layer must hold the pattern of block holder_of[b]."""
+    expect_blk = blk_term[holder_of]
+    for l in range(pool3.shape[0]):
+        ok = torch.equal(pool3[l], expect_blk[:, None] + (elem_term[None, :] + 257 * l))
+        assert ok, f"{what}: layer {l} differs from the expected block pattern"
+
+
+def test_config4_copy_blocks_full_pool(gpu):
+    """4096 copy-on-write pairs over all 32 layers of the 128 GiB pool (16 GiB moved)."""
+    s = wl.LLAMA_3_8B
+    nb, L = 65536, s.num_layers
+    pool = torch.empty(L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16,
+                       device=gpu)
+    pool3 = pool.view(torch.int16).view(L, nb, -1)
+    blk_term, elem_term = _pattern_terms(nb, pool3.shape[2], gpu)
+    _fill_pattern(pool3, blk_term, elem_term)
+    flat, pairs = wl.copy_on_write_pairs(nb, 4096, seed=0)
+    kvc.copy_blocks(pool, pairs, validate=True)
+    holder = torch.arange(nb, device=gpu)
+    holder[torch.from_numpy(flat[1::2]).to(gpu)] = torch.from_numpy(flat[0::2]).to(gpu)
+    _check_pattern(pool3, holder, blk_term, elem_term, "copy_blocks")
+    # idempotent
+    kvc.copy_blocks(pool, torch.from_numpy(flat).to(gpu))
+    _check_pattern(pool3, holder, blk_term, elem_term, "copy_blocks twice")
+
+
+@pytest.mark.parametrize("mode", ["direct", "staged"])
+def test_config5_swap_round_trip_full(gpu, mode):
+    """Llama-3.1-70B shape: scattered blocks -> contiguous pinned host buffer ->
+    fresh random blocks; the payload must arrive bit-exact and nothing else may change."""
+    s = wl.LLAMA_3_1_70B
+    nb, L, n = 16384, s.num_layers, SWAP_BLOCKS
+    pool = torch.empty(L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16,
+                       device=gpu)
+    pool3 = pool.view(torch.int16).view(L, nb, -1)
+    blk_term, elem_term = _pattern_terms(nb, pool3.shape[2], gpu)
+    _fill_pattern(pool3, blk_term, elem_term)
+    old, host_ids, new = wl.swap_round_trip(nb, n, seed=0)
+    worker = kvc.KVWorker(pool, n, swap_mode=mode)
+    try:
+        worker.copy_kv_sync([kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))],
+                            kvc.Device.GPU, kvc.Device.Host)
+        # host side, sampled: host[i, l, :] is block old[i] of layer l
+        host = worker.host_kv_caches.view(np.int16)
+        elem_np = elem_term.cpu().numpy()
+        blk_np = blk_term.cpu().numpy()
+        for i in list(range(0, n, max(1, n // 48))) + [n - 1]:
+            for l in (0, L // 2, L - 1):
+                want = (blk_np[old[i]] + elem_np + np.int16(257 * l)).astype(np.int16)
+                assert np.array_equal(host[i, l], want), f"host block {i}, layer {l}"
+        worker.copy_kv_sync([kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))],
+                            kvc.Device.Host, kvc.Device.GPU)
+    finally:
+        worker.close()
+    holder = torch.arange(nb, device=gpu)
+    holder[torch.from_numpy(new).to(gpu)] = torch.from_numpy(old).to(gpu)
+    _check_pattern(pool3, holder, blk_term, elem_term, f"swap round trip ({mode})")
