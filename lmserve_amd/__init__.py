@@ -4,6 +4,7 @@
     paged       append_paged_kv_cache(_layers), get_seq_lens, get_batch_indices_positions
     kv_worker   KVWorker (GPU <-> pinned host swap), Device, BlockMapping
     index_prep  host-side block-table / slot-mapping construction
+    kv_pool     pool sizing, allocator id order, layer-sync handle and model-side hooks
 
 Every operator runs a hand-written HIP kernel from libkvcache.so through the
 C ABI of include/kvcache.h; nothing here computes on the CPU.
@@ -12,6 +13,8 @@ from . import _lib
 from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_block_maps,
                         reshape_and_cache, reshape_and_cache_layers)
 from .index_prep import InferInput, KVIndexInputs, make_kv_index_inputs, to_device
+from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
+                      allocate_kv_caches, plan_cache)
 from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
                         flatten_block_mappings)
 from .paged import (append_paged_kv_cache, append_paged_kv_cache_layers,
@@ -24,5 +27,7 @@ __all__ = [
     "get_batch_indices_positions",
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",
     "flatten_block_mappings",
+    "BlockAllocator", "CachePlan", "KVWorkerHandle", "LayerSyncHooks", "allocate_kv_caches",
+    "plan_cache",
     "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device",
 ]

@@ -121,6 +121,15 @@ class KVWorker:
       (`[L, nb, 2, bs, H, D]`), contiguous, on the GPU. The reference maps it
       from an IPC handle in a second process (kv_worker.py:104-108); here the
       tensor itself is passed.
+    swap_mode: "direct" (default; one kernel addresses the mapped host pool,
+      no staging traffic) or "staged" (gather/scatter kernel + large DMA extents
+      on a second stream).
+    kv_worker_handle: a `kv_pool.KVWorkerHandle`; when given, `copy_kv` between
+      GPU and Host follows the reference's layer-pipelined protocol
+      (kv_worker.py:249-295): a save waits for the model's doorbell and
+      `post_events[l]` before touching layer l, a load records `pre_events[l]`
+      and rings the model's doorbell after layer l. Without it the whole layer
+      range moves in one call.
     """
 
     def __init__(
@@ -129,8 +138,9 @@ class KVWorker:
         num_host_blocks: int,
         num_disk_blocks: int = 0,
         disk_kv_cache_file: Optional[str] = None,
-        swap_mode: str = "staged",
+        swap_mode: str = "direct",
         staging_chunk_blocks: int = 0,
+        kv_worker_handle=None,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -173,6 +183,7 @@ class KVWorker:
             self._dtoh_copy_stream = torch.cuda.Stream()
             self._htod_copy_stream = torch.cuda.Stream()
         self._staging = {"out": None, "in": None}
+        self.kv_worker_handle = kv_worker_handle
 
         self.COPY_KV_OP_MAP = {
             (Device.GPU, Device.Host): self._copy_kv_gpu_to_host,
@@ -237,12 +248,36 @@ class KVWorker:
 
     async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
                                      stream: torch.cuda.Stream) -> None:
-        self.save_kv_blocks_to_host_nowait(block_mappings, stream)
+        """GPU->Host (kv_worker.py:272-295). With a handle: per layer, wait for the
+        model's doorbell, make `stream` wait for `post_events[layer]`, then save
+        that layer of every mapped block."""
+        handle = self.kv_worker_handle
+        if handle is None:
+            self.save_kv_blocks_to_host_nowait(block_mappings, stream)
+        elif len(block_mappings) > 0:
+            for layer_idx in range(self.num_layers):
+                while handle.kv_queue.empty():
+                    await asyncio.sleep(1e-5)
+                handle.kv_queue.get()
+                stream.wait_event(handle.post_events[layer_idx])
+                self.save_kv_blocks_to_host_nowait(block_mappings, stream, layer_idx, layer_idx + 1)
+                await asyncio.sleep(0)  # let other tasks of the loop run
         await asyncio.to_thread(stream.synchronize)
 
     async def load_kv_blocks_from_host(self, block_mappings: Sequence[BlockMapping],
                                        stream: torch.cuda.Stream) -> None:
-        self.load_kv_blocks_from_host_nowait(block_mappings, stream)
+        """Host->GPU (kv_worker.py:249-270). With a handle: after each layer's
+        copies are enqueued, record `pre_events[layer]` on `stream` and ring the
+        model's doorbell."""
+        handle = self.kv_worker_handle
+        if handle is None:
+            self.load_kv_blocks_from_host_nowait(block_mappings, stream)
+        elif len(block_mappings) > 0:
+            for layer_idx in range(self.num_layers):
+                self.load_kv_blocks_from_host_nowait(block_mappings, stream, layer_idx, layer_idx + 1)
+                await asyncio.sleep(0)
+                handle.pre_events[layer_idx].record(stream)
+                handle.model_queue.put(b"")
         await asyncio.to_thread(stream.synchronize)
 
     # ----------------------------------------------------------------- disk legs

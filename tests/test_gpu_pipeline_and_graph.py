@@ -1,0 +1,210 @@
+"""The layer-pipelined swap protocol (events + doorbell queues between a model
+thread and the swap engine) and hipGraph replay of the write/copy operators."""
+import asyncio
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+import lmserve_amd as kvc
+from lmserve_amd import workloads as wl
+from oracle import kvc_oracle as orc
+from tests.helpers import bf16_bits, bits_of, random_pool, sentinel_pool, to_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _busy(dev, n=3):
+    """Some real GPU time on the current stream (stands in for a layer's compute)."""
+    a = torch.ones(2048, 2048, device=dev)
+    for _ in range(n):
+        a = a @ a * 1e-4
+    return a
+
+
+@pytest.mark.parametrize("mode", ["direct", "staged"])
+def test_write_through_waits_for_each_layers_kv_write(gpu, mode):
+    """GPU->Host runs concurrently with the forward pass; layer l may be saved
+    only after the model recorded post_events[l], so the host copy must hold
+    the K/V written in THIS step for every layer."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb, bs, H, D = 6, 32, 8, s.block_size, s.num_kv_heads, s.head_dim
+    pool_np = random_pool((L, nb, 2, bs, H, D), 1)
+    dpool = to_bf16(pool_np, gpu)
+    handle = kvc.KVWorkerHandle.create(L)
+    worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle)
+    hooks = kvc.LayerSyncHooks(handle)
+    hooks.enable_record_after_execute = True
+    try:
+        worker.host_kv_caches[...] = sentinel_pool(worker.host_kv_caches.shape, 2)
+        blocks = np.asarray([3, 17, 9, 30], dtype=np.int64)           # blocks written to this step
+        host_ids = np.asarray([5, 0, 2, 7], dtype=np.int64)
+        T = len(blocks) * bs
+        slots = (blocks[:, None] * bs + np.arange(bs)[None, :]).reshape(-1)
+        key, value = bf16_bits((L, T, H, D), 3), bf16_bits((L, T, H, D), 4)
+        want_pool = pool_np.copy()
+        for l in range(L):
+            orc.reshape_and_cache_np(key[l], value[l], want_pool[l], slots)
+        want_host = worker.host_kv_caches.copy()
+        orc.save_blocks_to_host_np(want_pool.reshape(L, nb, -1), want_host, blocks, host_ids)
+
+        maps = [kvc.BlockMapping.from_pairs(zip(blocks.tolist(), host_ids.tolist()))]
+        errors = []
+
+        def kv_thread():
+            try:
+                asyncio.run(worker.copy_kv(maps, kvc.Device.GPU, kvc.Device.Host))
+            except Exception as exc:  # surfaced in the main thread below
+                errors.append(exc)
+
+        th = threading.Thread(target=kv_thread, daemon=True)
+        th.start()
+        dk, dv, dslots = to_bf16(key, gpu), to_bf16(value, gpu), torch.from_numpy(slots).to(gpu)
+        model_stream = torch.cuda.Stream()
+        with torch.cuda.stream(model_stream):
+            for l in range(L):
+                hooks.pre(l)
+                _busy(gpu)                                   # the save must not overtake this
+                kvc.reshape_and_cache(dk[l], dv[l], dpool[l], dslots)
+                hooks.post(l)
+        th.join(timeout=60)
+        assert not th.is_alive() and not errors, errors
+        model_stream.synchronize()
+        assert np.array_equal(bits_of(dpool), want_pool)
+        assert np.array_equal(worker.host_kv_caches, want_host)
+        assert handle.kv_queue.empty()
+    finally:
+        worker.close()
+
+
+@pytest.mark.parametrize("mode", ["direct", "staged"])
+def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode):
+    """Host->GPU: the model waits per layer on pre_events[l] (after the doorbell)
+    and must then see that layer's fetched blocks."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb = 5, 24, 8
+    pool_np = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), 5)
+    dpool = to_bf16(pool_np, gpu)
+    handle = kvc.KVWorkerHandle.create(L)
+    worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle)
+    hooks = kvc.LayerSyncHooks(handle)
+    hooks.enable_wait_before_execute = True
+    hooks.timeout = 30
+    try:
+        host = random_pool(worker.host_kv_caches.shape, 6)
+        worker.host_kv_caches[...] = host
+        src = np.asarray([1, 6, 4], dtype=np.int64)
+        dst = np.asarray([20, 2, 11], dtype=np.int64)
+        maps = [kvc.BlockMapping.from_pairs(zip(src.tolist(), dst.tolist()))]
+        th = threading.Thread(target=lambda: asyncio.run(
+            worker.copy_kv(maps, kvc.Device.Host, kvc.Device.GPU)), daemon=True)
+        th.start()
+        seen = []
+        model_stream = torch.cuda.Stream()
+        with torch.cuda.stream(model_stream):
+            for l in range(L):
+                hooks.pre(l)                                 # blocks until layer l is on its way
+                seen.append(dpool[l, torch.from_numpy(dst).to(gpu)].clone())
+                hooks.post(l)
+        th.join(timeout=60)
+        assert not th.is_alive()
+        model_stream.synchronize()
+        for l in range(L):
+            got = bits_of(seen[l]).reshape(len(dst), -1)
+            assert np.array_equal(got, host[src, l]), f"layer {l} was read before its fetch landed"
+        assert handle.model_queue.empty()
+    finally:
+        worker.close()
+
+
+def test_allocator_order_drives_a_realistic_decode_step(gpu):
+    """Block tables produced by the FIFO allocator under churn, written through
+    the page-table path, equal the oracle."""
+    s = wl.LLAMA_3_2_1B
+    nb, bs, L = 128, s.block_size, 2
+    alloc = kvc.BlockAllocator(nb)
+    rng = np.random.default_rng(0)
+    live = {}
+    for step in range(40):                                    # churn: sequences come and go
+        sid = step
+        live[sid] = alloc.alloc_blocks(int(rng.integers(1, 6)))
+        if len(live) > 8:
+            victim = list(live)[int(rng.integers(0, len(live)))]
+            alloc.free_blocks(live.pop(victim))
+    reqs = []
+    for i, (sid, blocks) in enumerate(live.items()):
+        ctx = int(rng.integers((len(blocks) - 1) * bs + 1, len(blocks) * bs + 1))
+        new = 1 if i % 2 else min(ctx, int(rng.integers(2, 20)))
+        reqs.append(kvc.InferInput(sid, [0] * new, new, ctx - new, ctx, blocks))
+    idx = kvc.make_kv_index_inputs(reqs, bs)
+    assert sorted(set(idx.kv_block_indices.tolist())) != list(range(len(set(idx.kv_block_indices.tolist()))))
+    T = len(idx.slot_mapping)
+    key, value = bf16_bits((L, T, s.num_kv_heads, s.head_dim), 1), bf16_bits((L, T, s.num_kv_heads, s.head_dim), 2)
+    pool = sentinel_pool((L, nb, 2, bs, s.num_kv_heads, s.head_dim), 3)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_append_paged_kv_cache(key[l], value[l], idx.batch_indices, idx.positions, want[l],
+                                    idx.kv_block_indices, idx.kv_block_indptrs)
+    dev = kvc.to_device(idx, bs, gpu)
+    dpool = to_bf16(pool, gpu)
+    kvc.append_paged_kv_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dev.batch_indices,
+                                     dev.positions, dpool, dev.kv_block_indices, dev.kv_block_indptrs,
+                                     dev.kv_last_block_lens)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), want)
+
+
+def test_graph_replay_of_write_and_copy_matches_eager_every_time(gpu):
+    """A captured decode step (per-layer page-table writes + a block copy) is
+    replayed several times with new K/V in the static input buffers and eager
+    work in between; every replay must equal the oracle."""
+    s = wl.LLAMA_3_8B
+    L, nb, bs = 4, 128, s.block_size
+    w = wl.decode_step(s, num_blocks=nb, batch=24, max_context=60, seed=3)
+    idx = kvc.to_device(w.index, bs, gpu)
+    T = w.num_tokens
+    pool_np = sentinel_pool((L, nb, 2, bs, s.num_kv_heads, s.head_dim), 1)
+    dpool = to_bf16(pool_np, gpu)
+    static_k = torch.zeros(L, T, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16, device=gpu)
+    static_v = torch.zeros_like(static_k)
+    used = set(w.index.kv_block_indices.tolist())
+    free = [b for b in range(nb) if b not in used]
+    flat = np.asarray([int(w.index.kv_block_indices[0]), free[0],
+                       int(w.index.kv_block_indices[1]), free[1]], dtype=np.int64)
+    dmaps = torch.from_numpy(flat).to(gpu)
+
+    def step():
+        for l in range(L):
+            kvc.append_paged_kv_cache(static_k[l], static_v[l], idx.batch_indices, idx.positions,
+                                      dpool[l], idx.kv_block_indices, idx.kv_block_indptrs,
+                                      idx.kv_last_block_lens)
+        kvc.copy_blocks(dpool, dmaps)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+
+    want = pool_np.copy()
+    for rep in range(4):
+        key, value = bf16_bits((L, T, s.num_kv_heads, s.head_dim), 10 + rep), \
+            bf16_bits((L, T, s.num_kv_heads, s.head_dim), 20 + rep)
+        dpool.copy_(to_bf16(pool_np, gpu))                    # eager work between replays
+        static_k.copy_(to_bf16(key, gpu))
+        static_v.copy_(to_bf16(value, gpu))
+        _busy(gpu, 1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want[...] = pool_np
+        for l in range(L):
+            orc.c_append_paged_kv_cache(key[l], value[l], w.index.batch_indices, w.index.positions,
+                                        want[l], w.index.kv_block_indices, w.index.kv_block_indptrs)
+        orc.c_copy_blocks(want, flat)
+        assert np.array_equal(bits_of(dpool), want), f"replay {rep} differs from the oracle"

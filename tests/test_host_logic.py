@@ -169,3 +169,32 @@ def test_torch_cpu_statements_agree_with_the_oracle():
     got_gpu = torch.from_numpy(gpu.view(np.int16).copy())
     torch_cpu.swap_in_cpu(got_gpu, got_host, torch.from_numpy(hid), torch.from_numpy(dst))
     assert np.array_equal(got_gpu.numpy().view(np.uint16), want_gpu)
+
+
+def test_block_allocator_hands_out_ids_in_fifo_order():
+    a = kvc.BlockAllocator(6)
+    assert a.alloc_blocks(4) == [0, 1, 2, 3]
+    a.free_block(1)
+    a.free_block(0)
+    assert a.alloc_blocks(3) == [4, 5, 1]          # freed ids queue up behind the untouched ones
+    assert a.alloc_block() == 0
+    with pytest.raises(RuntimeError):
+        a.alloc_block()
+    a.alloc_block_by_id(2)                          # shared prefix block: ref count 2
+    a.free_block(2)
+    assert a.get_block_usage() == 1.0
+    a.free_block(2)
+    assert a.alloc_block() == 2
+    assert a.can_alloc_blocks(0) and not a.can_alloc_blocks(1)
+    b = kvc.BlockAllocator(10)
+    assert b.can_alloc_blocks(9, 0.9) and not b.can_alloc_blocks(10, 0.9)
+    b.alloc_block_by_id(7)
+    assert b.alloc_blocks(8) == [0, 1, 2, 3, 4, 5, 6, 8]
+
+
+def test_plan_cache_matches_the_configured_pools():
+    p = kvc.plan_cache(128 << 30, 16 << 30, 0, 32, 8, 128, 16, torch.bfloat16)
+    assert (p.kv_block_size, p.num_gpu_blocks, p.num_host_blocks, p.num_disk_blocks) == \
+        (32768, 65536, 8192, 0)
+    p = kvc.plan_cache(80 << 30, 40 << 30, 1 << 30, 80, 8, 128, 16, torch.float16)
+    assert (p.num_gpu_blocks, p.num_host_blocks, p.num_disk_blocks) == (16384, 8192, 204)
