@@ -35,6 +35,13 @@ HBM_PEAK_GBPS = 8000.0
 ROTATE_DECODE = 16   # 16 x 32 MiB of K/V sources
 ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 
+# HBM bytes per launch of the headline kernel (config 2, all layers in one launch)
+# from two rocprofv3 --pmc runs: FETCH_SIZE 16479.4 KiB x 1.9999 + WRITE_SIZE
+# 32789.7 KiB x 1.0000, the factors being what the same counters read for a
+# plain elementwise kernel of known size (1 GiB read, 1 GiB written); summary in
+# profiles/hbm_traffic_fetch_size_write_size.txt. Only valid for the default workload.
+MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67325444
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -274,11 +281,12 @@ def main():
     torch.cuda.empty_cache()
 
     if "calib" in ops:
-        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        # a plain elementwise kernel of known size: reads 1 GiB, writes 1 GiB
+        a = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
         b = torch.empty_like(a)
-        ms_w, ms_e = time_region(lambda i: b.copy_(a), 10, 2, torch)
-        extra.append(entry("calibration: plain device copy of 1 GiB (torch copy_)", 2 << 30, ms_w, ms_e,
-                           launch="eager"))
+        ms_w, ms_e = time_region(lambda i: torch.add(a, 1, out=b), 10, 2, torch)
+        extra.append(entry("calibration: plain elementwise kernel, 1 GiB read + 1 GiB written "
+                           "(torch.add(int32, 1))", 2 << 30, ms_w, ms_e, launch="eager"))
         del a, b
         torch.cuda.empty_cache()
 
@@ -354,7 +362,9 @@ def main():
                    "launch": "one eager launch per step on torch's current stream",
                    "rotation": f"{ROTATE_DECODE} K/V source sets and slot sets cycled"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_CFG2_ONE_LAUNCH
+                     if (L == 32 and args.pool_blocks == 65536) else None,
                      "kernel": "write_rows_kernel", "bytes_per_launch": int(bytes_step),
                      "us_per_launch": round(ms_event * 1e3, 3)},
         "cpu_baseline": cpu,

@@ -56,6 +56,17 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
                          "the KV-cache operators have no CPU path")
 
 
+def _inner_contiguous(t: torch.Tensor) -> bool:
+    """True when every slice `t[i]` is contiguous (dim 0 may have any stride)."""
+    expected = 1
+    shape, stride = t.shape, t.stride()
+    for d in range(len(shape) - 1, 0, -1):
+        if shape[d] != 1 and stride[d] != expected:
+            return False
+        expected *= shape[d]
+    return True
+
+
 def _stream_of(t: torch.Tensor) -> int:
     """Raw hipStream_t of torch's current stream on the tensor's device."""
     return torch._C._cuda_getCurrentRawStream(t.device.index)
@@ -206,11 +217,13 @@ def reshape_and_cache(
     for t, n in ((key, "key"), (value, "value"), (kv_cache, "kv_cache"),
                  (slot_mapping, "slot_mapping")):
         _require_gpu(t, n)
-    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2 or not kv_cache[0].is_contiguous():
-        raise ValueError("kv_cache must be [num_blocks, 2, block_size, H, D] with contiguous blocks")
+    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2:
+        raise ValueError("kv_cache must be [num_blocks, 2, block_size, H, D]")
     if key.dtype != kv_cache.dtype or value.dtype != kv_cache.dtype:
         raise TypeError("key/value and kv_cache must share one dtype")
     nb, _, bs, H, D = kv_cache.shape
+    if not _inner_contiguous(kv_cache):
+        raise ValueError("every block of kv_cache must be contiguous [2, block_size, H, D]")
     key, row, k_stride = _rows(key, "key")
     value, row_v, v_stride = _rows(value, "value")
     if row != H * D or row_v != H * D or key.shape[0] != value.shape[0]:

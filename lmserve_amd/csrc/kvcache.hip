@@ -67,7 +67,8 @@ struct Tuning {
   int write_vpt = 0;        // vectors per lane in write_rows, 0 = by size
   int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
-  int direct_max_wgs = 512; // grid cap of the direct (PCIe-bound) swap kernel
+  int direct_max_wgs = 64;  // grid cap of the direct swap kernel: PCIe saturates with a few
+                            // dozen workgroups, the rest of the GPU stays free for the model
 };
 Tuning g_tune;
 

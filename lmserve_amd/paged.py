@@ -17,7 +17,7 @@ from typing import Tuple
 import torch
 
 from . import _lib
-from .cache_ops import _on_device_of, _require_gpu, _rows, _stream_of
+from .cache_ops import _inner_contiguous, _on_device_of, _require_gpu, _rows, _stream_of
 
 
 def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
@@ -106,12 +106,13 @@ def append_paged_kv_cache(
     batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len = _paged_common(
         append_key, append_value, batch_indices, positions, kv_indices, kv_indptr,
         kv_last_page_len, kv_layout)
-    if paged_kv_cache.dim() != 5 or paged_kv_cache.shape[1] != 2 or \
-            (paged_kv_cache.shape[0] > 0 and not paged_kv_cache[0].is_contiguous()):
-        raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
+    if paged_kv_cache.dim() != 5 or paged_kv_cache.shape[1] != 2:
+        raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D]")
     if append_key.dtype != paged_kv_cache.dtype or append_value.dtype != paged_kv_cache.dtype:
         raise TypeError("append_key/append_value and paged_kv_cache must share one dtype")
     num_pages, _, page_size, H, D = paged_kv_cache.shape
+    if not _inner_contiguous(paged_kv_cache):
+        raise ValueError("every page of paged_kv_cache must be contiguous [2, page_size, H, D]")
     append_key, row, k_stride = _rows(append_key, "append_key")
     append_value, row_v, v_stride = _rows(append_value, "append_value")
     if row != H * D or row_v != H * D:
