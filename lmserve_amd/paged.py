@@ -179,3 +179,72 @@ def append_paged_kv_cache_layers(
             kv_indices.numel(), H, D, page_size, row, row, 2 * page_size * row, num_pages,
             L, tokens * row, tokens * row, num_pages * 2 * page_size * row,
             kv_caches.element_size(), _stream_of(kv_caches)))
+
+
+class PagedKVWritePlan:
+    """The page-table write with its per-step arguments checked ONCE.
+
+    A forward pass calls `append_paged_kv_cache` once per layer with the same
+    five index tensors (runtime/worker/llm_worker/models/layers/attention.py:76-85
+    inside the layer loop of models/llama.py:236-242). Building a plan per step
+    (where the reference builds `InputParams`, model_worker.py:435-446) and
+    calling `plan.append(key, value, kv_caches[i])` per layer leaves only three
+    pointer reads and the library call on the host's critical path.
+
+    The plan keeps references to the index tensors, so their memory stays valid
+    for as long as the plan lives.
+    """
+
+    def __init__(self, batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len,
+                 num_kv_heads: int, head_dim: int, page_size: int, dtype: torch.dtype,
+                 kv_layout: str = "NHD"):
+        (self.batch_indices, self.positions, self.kv_indices, self.kv_indptr,
+         self.kv_last_page_len) = _paged_common(None, None, batch_indices, positions, kv_indices,
+                                                kv_indptr, kv_last_page_len, kv_layout)
+        self.device = self.batch_indices.device
+        self.dtype = dtype
+        self.H, self.D, self.page_size = int(num_kv_heads), int(head_dim), int(page_size)
+        self.row = self.H * self.D
+        self.nnz = self.batch_indices.numel()
+        self.elem = torch.empty(0, dtype=dtype).element_size()
+        self._fn = _lib.lib().kvc_append_paged_kv_cache
+        # [key, value, bi, pos, cache, indices, indptr, last, nnz, B, n_idx, H, D, ps,
+        #  k_stride, v_stride, page_stride, num_pages, elem, stream]
+        self._args = [0, 0, self.batch_indices.data_ptr(), self.positions.data_ptr(), 0,
+                      self.kv_indices.data_ptr(), self.kv_indptr.data_ptr(),
+                      self.kv_last_page_len.data_ptr(), self.nnz, self.kv_indptr.numel() - 1,
+                      self.kv_indices.numel(), self.H, self.D, self.page_size,
+                      self.row, self.row, 2 * self.page_size * self.row, 0, self.elem, 0]
+        self._cache_shape_tail = (2, self.page_size, self.H, self.D)
+
+    def append(self, append_key: torch.Tensor, append_value: torch.Tensor,
+               paged_kv_cache: torch.Tensor) -> None:
+        """`append_paged_kv_cache` for one layer. Requirements (checked): key/value
+        dense `[nnz, H, D]` (or `[nnz, H*D]`) of the plan's dtype on its device,
+        `paged_kv_cache` `[num_pages, 2, page_size, H, D]` with contiguous pages."""
+        if self.nnz == 0:
+            return
+        if append_key.dtype != self.dtype or append_value.dtype != self.dtype \
+                or paged_kv_cache.dtype != self.dtype:
+            raise TypeError("append_key/append_value/paged_kv_cache must have the plan's dtype")
+        if append_key.device != self.device or append_value.device != self.device \
+                or paged_kv_cache.device != self.device:
+            raise ValueError("tensors must live on the plan's device")
+        if tuple(paged_kv_cache.shape[1:]) != self._cache_shape_tail or \
+                not _inner_contiguous(paged_kv_cache):
+            raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
+        if not append_key.is_contiguous() or not append_value.is_contiguous() \
+                or append_key.numel() < self.nnz * self.row or append_value.numel() < self.nnz * self.row:
+            raise ValueError("append_key/append_value must be dense [nnz, H, D]")
+        num_pages = paged_kv_cache.shape[0]
+        if num_pages == 0:
+            return
+        a = self._args
+        a[0] = append_key.data_ptr()
+        a[1] = append_value.data_ptr()
+        a[4] = paged_kv_cache.data_ptr()
+        a[16] = paged_kv_cache.stride(0) if num_pages > 1 else 2 * self.page_size * self.row
+        a[17] = num_pages
+        a[19] = _stream_of(paged_kv_cache)
+        with _on_device_of(paged_kv_cache):
+            _lib.check(self._fn(*a))

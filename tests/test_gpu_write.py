@@ -201,10 +201,22 @@ def test_append_paged_kv_cache_matches_oracle(gpu, kind):
                                      dev.kv_last_block_lens)
     slotted = to_bf16(pool, gpu)
     kvc.reshape_and_cache_layers(dkey, dval, slotted, dev.slot_mapping)
+    planned = to_bf16(pool, gpu)
+    s = w.shape
+    plan = kvc.PagedKVWritePlan(dev.batch_indices, dev.positions, dev.kv_block_indices,
+                                dev.kv_block_indptrs, dev.kv_last_block_lens, s.num_kv_heads,
+                                s.head_dim, s.block_size, torch.bfloat16)
+    for l in range(L):
+        plan.append(dkey[l], dval[l], planned[l])
     torch.cuda.synchronize()
     assert np.array_equal(bits_of(per_layer), want)
     assert np.array_equal(bits_of(fused), want)
     assert np.array_equal(bits_of(slotted), want)
+    assert np.array_equal(bits_of(planned), want)
+    with pytest.raises(TypeError):
+        plan.append(dkey[0].float(), dval[0], planned[0])
+    with pytest.raises(ValueError):
+        plan.append(dkey[0], dval[0], planned[0][:, :, :8])
 
 
 def test_append_paged_skips_tokens_with_bad_indices(gpu):
