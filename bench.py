@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops write,prefill,copy,swap]
 
-Headline (`value`): BASELINE config 2, the Llama-3-8B decode-step KV write
+Headline (`value`): benchmark configuration 2, the Llama-3-8B decode-step KV write
 (256 sequences x 1 new token, 32 layers, 8 KV heads x 128, block_size 16, bf16,
 pool of 65536 blocks = 128 GiB). One step = the K/V write of one decode step
 over all 32 layers through `kvc_reshape_and_cache_layers` (one launch). Inputs
@@ -381,7 +381,7 @@ def main():
         "vs_baseline": None,
         "dtype": "u16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE config 2: Llama-3-8B decode-step KV write, 256 seqs x 1 token, "
+        "config": {"workload": "configuration 2: Llama-3-8B decode-step KV write, 256 seqs x 1 token, "
                                f"{L} layers, 8 KV heads x 128, block_size 16, bf16 lanes, pool "
                                f"{args.pool_blocks} blocks "
                                f"({L * args.pool_blocks * s8.block_bytes / 2**30:.0f} GiB)",

@@ -164,6 +164,29 @@ int kvc_get_batch_indices_positions(const int32_t* append_indptr, const int32_t*
                                     int32_t* batch_indices, int32_t* positions,
                                     void* stream);
 
+/* The whole index preparation of a step in ONE launch, from the per-request
+ * scalars the scheduler sends (proto/worker.proto:40-47: input_len, context_len,
+ * block_ids). Replaces the host-side cumulative sums and list building of
+ * ModelWorker._make_inputs (runtime/worker/llm_worker/model_worker.py:346,
+ * :362-365, :399-423), the two flashinfer index calls (:425-433) and the slot
+ * rule of the scheduler (runtime/src/llm_engine/scheduler.rs:489-511):
+ *   cu_seqlens_q[b+1]  = sum_{i<=b} input_lens[i]           (cu_seqlens_q[0] = 0)
+ *   kv_indptr[b+1]     = sum_{i<=b} num_blocks[i]           (kv_indptr[0] = 0)
+ *   kv_last_page_len[b]= (context_lens[b]-1) % page_size + 1
+ *   for the j-th new token of request b, at out = cu_seqlens_q[b] + j:
+ *     batch_indices[out] = b, positions[out] = context_lens[b] - input_lens[b] + j,
+ *     slot_mapping[out]  = kv_indices[kv_indptr[b] + pos/page_size]*page_size + pos%page_size
+ * kv_indices is the concatenation of the requests' block tables. slot_mapping
+ * may be NULL; a position outside its request's table yields slot -1.
+ * Outputs: cu_seqlens_q, kv_indptr [batch_size+1], kv_last_page_len [batch_size],
+ * batch_indices, positions (int32) and slot_mapping (int64) [nnz]. */
+int kvc_build_write_index(const int32_t* input_lens, const int32_t* context_lens,
+                          const int32_t* num_blocks, const int32_t* kv_indices,
+                          int64_t batch_size, int64_t num_kv_indices, int64_t page_size,
+                          int64_t nnz, int32_t* cu_seqlens_q, int32_t* kv_indptr,
+                          int32_t* kv_last_page_len, int32_t* batch_indices,
+                          int32_t* positions, int64_t* slot_mapping, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Block copy inside the pool (prefix-sharing copy-on-write).
  * Replaces copy_blocks / copy_blocks_kernel

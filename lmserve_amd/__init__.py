@@ -12,13 +12,14 @@ C ABI of include/kvcache.h; nothing here computes on the CPU.
 from . import _lib
 from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_block_maps,
                         reshape_and_cache, reshape_and_cache_layers)
-from .index_prep import InferInput, KVIndexInputs, make_kv_index_inputs, to_device
+from .index_prep import (InferInput, KVIndexInputs, make_kv_index_inputs, to_device,
+                         to_device_one_launch)
 from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
                       allocate_kv_caches, plan_cache)
 from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
                         flatten_block_mappings)
 from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cache_layers,
-                    get_batch_indices_positions, get_seq_lens)
+                    build_write_index, get_batch_indices_positions, get_seq_lens)
 
 __all__ = [
     "copy_blocks", "fill_key_cache", "reshape_and_cache", "reshape_and_cache_layers",
@@ -29,5 +30,6 @@ __all__ = [
     "flatten_block_mappings",
     "BlockAllocator", "CachePlan", "KVWorkerHandle", "LayerSyncHooks", "allocate_kv_caches",
     "plan_cache",
-    "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device",
+    "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device", "to_device_one_launch",
+    "build_write_index",
 ]

@@ -43,6 +43,8 @@ SIGNATURES = {
                                                  _I64, _I64, _I64, c_int, _P]),
     "kvc_get_seq_lens": (c_int, [_P, _P, _I64, _I64, _P, _P]),
     "kvc_get_batch_indices_positions": (c_int, [_P, _P, _I64, _I64, _P, _P, _P]),
+    "kvc_build_write_index": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P,
+                                      _P]),
     "kvc_copy_blocks": (c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _P]),
     "kvc_swap_staging_bytes": (_I64, [_I64, _I64, _I64, c_int, _I64]),
     "kvc_swap_out": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,

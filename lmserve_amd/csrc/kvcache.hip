@@ -308,6 +308,84 @@ __global__ void batch_indices_positions_kernel(const int32_t* append_indptr,
   }
 }
 
+// Whole index preparation of a step in one launch (one workgroup): prefix sums
+// of the per-request new-token counts and block counts, the last-page fill, and
+// for every new token its request, absolute position and slot.
+constexpr int kPrepThreads = 1024;
+
+__global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
+    const int32_t* input_lens, const int32_t* context_lens, const int32_t* num_blocks,
+    const int32_t* kv_indices, int32_t batch_size, int64_t num_kv_indices, int32_t page_size,
+    int64_t nnz, int32_t* cu_seqlens_q, int32_t* kv_indptr, int32_t* kv_last_page_len,
+    int32_t* batch_indices, int32_t* positions, int64_t* slot_mapping) {
+  __shared__ int32_t carry[2];
+  __shared__ int32_t part_q[kPrepThreads];
+  __shared__ int32_t part_b[kPrepThreads];
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    carry[0] = 0;
+    carry[1] = 0;
+    cu_seqlens_q[0] = 0;
+    kv_indptr[0] = 0;
+  }
+  __syncthreads();
+  // chunked inclusive scan (Hillis-Steele inside a chunk of kPrepThreads requests)
+  for (int32_t base = 0; base < batch_size; base += kPrepThreads) {
+    const int32_t b = base + tid;
+    const int32_t q = b < batch_size ? input_lens[b] : 0;
+    const int32_t n = b < batch_size ? num_blocks[b] : 0;
+    part_q[tid] = q;
+    part_b[tid] = n;
+    __syncthreads();
+    for (int off = 1; off < kPrepThreads; off <<= 1) {
+      const int32_t aq = tid >= off ? part_q[tid - off] : 0;
+      const int32_t ab = tid >= off ? part_b[tid - off] : 0;
+      __syncthreads();
+      part_q[tid] += aq;
+      part_b[tid] += ab;
+      __syncthreads();
+    }
+    if (b < batch_size) {
+      cu_seqlens_q[b + 1] = carry[0] + part_q[tid];
+      kv_indptr[b + 1] = carry[1] + part_b[tid];
+      const int32_t ctx = context_lens[b];
+      kv_last_page_len[b] = ctx > 0 ? (ctx - 1) % page_size + 1 : 0;
+    }
+    __syncthreads();
+    if (tid == kPrepThreads - 1) {
+      carry[0] += part_q[tid];
+      carry[1] += part_b[tid];
+    }
+    __syncthreads();
+  }
+  // per token: find its request by bisection over the prefix sums just written
+  // (visible to the whole workgroup after the barrier above); the request's new
+  // tokens occupy positions [context - input, context)
+  const int64_t total = cu_seqlens_q[batch_size];
+  const int64_t limit = total < nnz ? total : nnz;
+  for (int64_t out = tid; out < limit; out += kPrepThreads) {
+    int32_t lo = 0, hi = batch_size;  // invariant: cu[lo] <= out < cu[hi]
+    while (hi - lo > 1) {
+      const int32_t mid = (lo + hi) >> 1;
+      if (cu_seqlens_q[mid] <= out) lo = mid;
+      else hi = mid;
+    }
+    const int32_t b = lo;
+    const int32_t begin = cu_seqlens_q[b];
+    const int32_t n_new = cu_seqlens_q[b + 1] - begin;
+    const int32_t pos = context_lens[b] - n_new + (int32_t)(out - begin);
+    batch_indices[out] = b;
+    positions[out] = pos;
+    if (slot_mapping) {
+      const int64_t it = (int64_t)kv_indptr[b] + pos / page_size;
+      const int64_t table_end = kv_indptr[b + 1] < num_kv_indices ? kv_indptr[b + 1] : num_kv_indices;
+      slot_mapping[out] = (pos >= 0 && it >= 0 && it < table_end)
+                              ? (int64_t)kv_indices[it] * page_size + pos % page_size
+                              : -1;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host helpers
 // ---------------------------------------------------------------------------
@@ -914,6 +992,32 @@ int kvc_get_batch_indices_positions(const int32_t* append_indptr, const int32_t*
     return fail(KVC_ERR_INVALID_ARG, "kvc_get_batch_indices_positions: null pointer");
   hipLaunchKernelGGL(batch_indices_positions_kernel, dim3((unsigned)batch_size), dim3(kThreads), 0,
                      (hipStream_t)stream, append_indptr, seq_lens, nnz, batch_indices, positions);
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+int kvc_build_write_index(const int32_t* input_lens, const int32_t* context_lens,
+                          const int32_t* num_blocks, const int32_t* kv_indices, int64_t batch_size,
+                          int64_t num_kv_indices, int64_t page_size, int64_t nnz,
+                          int32_t* cu_seqlens_q, int32_t* kv_indptr, int32_t* kv_last_page_len,
+                          int32_t* batch_indices, int32_t* positions, int64_t* slot_mapping,
+                          void* stream) {
+  if (batch_size < 0 || nnz < 0 || num_kv_indices < 0 || page_size <= 0 ||
+      batch_size > 0x7fffffffll || page_size > 0x7fffffffll)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: batch_size=%lld nnz=%lld page_size=%lld",
+                (long long)batch_size, (long long)nnz, (long long)page_size);
+  if (!cu_seqlens_q || !kv_indptr)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: null prefix-sum output");
+  if (batch_size > 0 && (!input_lens || !context_lens || !num_blocks || !kv_last_page_len))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: null per-request array");
+  if (nnz > 0 && (!batch_indices || !positions))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: null per-token output");
+  if (slot_mapping && num_kv_indices > 0 && !kv_indices)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: null kv_indices");
+  hipLaunchKernelGGL(build_write_index_kernel, dim3(1), dim3(kPrepThreads), 0, (hipStream_t)stream,
+                     input_lens, context_lens, num_blocks, kv_indices, (int32_t)batch_size,
+                     num_kv_indices, (int32_t)page_size, nnz, cu_seqlens_q, kv_indptr,
+                     kv_last_page_len, batch_indices, positions, slot_mapping);
   KVC_HIP(hipGetLastError());
   return KVC_OK;
 }

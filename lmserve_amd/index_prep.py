@@ -146,3 +146,35 @@ def to_device(host: KVIndexInputs, page_size: int, device="cuda",
         kv_last_block_lens=last,
         slot_mapping=up(host.slot_mapping) if with_slot_mapping else None,
     )
+
+
+def to_device_one_launch(inputs: Sequence[InferInput], page_size: int, device="cuda",
+                         with_slot_mapping: bool = True) -> DeviceKVIndexInputs:
+    """The same device tensors as `to_device(make_kv_index_inputs(...))`, but the
+    host only packs four small arrays (new-token count, context length and
+    block-table length per request, and the concatenated block tables); prefix
+    sums, positions, request indices and slots are computed on the device in a
+    single launch. Requests are ordered as `make_kv_index_inputs` orders them."""
+    from .paged import build_write_index
+
+    order = sorted(range(len(inputs)), key=lambda i: -inputs[i].input_len)
+    reqs = [inputs[i] for i in order]
+    packed = np.empty((3, len(reqs)), dtype=np.int32)
+    tables: List[int] = []
+    prefill_input_len = 0
+    for b, r in enumerate(reqs):
+        packed[0, b] = r.input_len
+        packed[1, b] = r.context_len
+        packed[2, b] = len(r.block_ids)
+        tables += r.block_ids
+        if r.input_len > 1:
+            prefill_input_len += int(r.input_len)
+    nnz = int(packed[0].sum()) if len(reqs) else 0
+    dev_packed = torch.from_numpy(packed).to(device, non_blocking=True)
+    kv_indices = torch.from_numpy(np.asarray(tables, dtype=np.int32)).to(device, non_blocking=True)
+    cu, indptr, last, batch_indices, positions, slots = build_write_index(
+        dev_packed[0], dev_packed[1], dev_packed[2], kv_indices, page_size, nnz, with_slot_mapping)
+    return DeviceKVIndexInputs(position_ids=positions, cu_seqlens_q=cu,
+                               prefill_input_len=prefill_input_len, batch_indices=batch_indices,
+                               positions=positions, kv_block_indices=kv_indices,
+                               kv_block_indptrs=indptr, kv_last_block_lens=last, slot_mapping=slots)

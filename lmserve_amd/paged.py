@@ -248,3 +248,39 @@ class PagedKVWritePlan:
         a[19] = _stream_of(paged_kv_cache)
         with _on_device_of(paged_kv_cache):
             _lib.check(self._fn(*a))
+
+
+def build_write_index(input_lens: torch.Tensor, context_lens: torch.Tensor,
+                      num_blocks: torch.Tensor, kv_indices: torch.Tensor, page_size: int,
+                      nnz: int, with_slot_mapping: bool = True):
+    """All index tensors of a step from the per-request scalars, in one launch.
+
+    input_lens, context_lens, num_blocks: int32 `[B]` on the device (new tokens,
+    context length and block-table length of every request, in batch order);
+    kv_indices: int32 concatenation of the block tables. Returns
+    `(cu_seqlens_q, kv_indptr, kv_last_page_len, batch_indices, positions, slot_mapping)`
+    -- what `ModelWorker._make_inputs` builds on the host and uploads piecewise
+    (model_worker.py:346, :362-365, :399-433), plus the slot mapping.
+    """
+    input_lens = _i32(input_lens, "input_lens")
+    context_lens = _i32(context_lens, "context_lens")
+    num_blocks = _i32(num_blocks, "num_blocks")
+    kv_indices = _i32(kv_indices, "kv_indices")
+    B = input_lens.numel()
+    if context_lens.numel() != B or num_blocks.numel() != B:
+        raise ValueError("input_lens, context_lens and num_blocks must have one entry per request")
+    dev = input_lens.device
+    nnz = int(nnz)
+    cu = torch.empty(B + 1, dtype=torch.int32, device=dev)
+    indptr = torch.empty(B + 1, dtype=torch.int32, device=dev)
+    last = torch.empty(B, dtype=torch.int32, device=dev)
+    batch_indices = torch.empty(nnz, dtype=torch.int32, device=dev)
+    positions = torch.empty(nnz, dtype=torch.int32, device=dev)
+    slots = torch.empty(nnz, dtype=torch.int64, device=dev) if with_slot_mapping else None
+    with _on_device_of(input_lens):
+        _lib.check(_lib.lib().kvc_build_write_index(
+            input_lens.data_ptr(), context_lens.data_ptr(), num_blocks.data_ptr(),
+            kv_indices.data_ptr(), B, kv_indices.numel(), int(page_size), nnz, cu.data_ptr(),
+            indptr.data_ptr(), last.data_ptr(), batch_indices.data_ptr(), positions.data_ptr(),
+            slots.data_ptr() if slots is not None else None, _stream_of(input_lens)))
+    return cu, indptr, last, batch_indices, positions, slots

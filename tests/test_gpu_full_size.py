@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes, checked through properties
+"""The five benchmark configurations at their full sizes, checked through properties
 that do not need a CPU copy of the pool: gather-back of the written rows, a
 census of changed elements over the whole pool, a closed-form block pattern
 for copy and swap, and the swap-out -> swap-in round trip."""

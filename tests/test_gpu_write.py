@@ -99,7 +99,7 @@ def test_fill_key_cache_every_launch_shape(gpu, vpt, nt):
 
 
 def test_config1_llama_1b_write_all_layers(gpu):
-    """BASELINE config 1 at its full size: 16 layers, pool of 1024 blocks, 256
+    """Configuration 1 (Llama-3.2-1B) at its full size: 16 layers, pool of 1024 blocks, 256
     tokens on seeded random distinct free slots; per-layer op and the one-launch
     form must both equal the oracle on the whole 512 MiB pool."""
     s = wl.LLAMA_3_2_1B
