@@ -243,6 +243,66 @@ int kvc_swap_in(void* pool, const void* host_pool,
                 void* staging, int64_t staging_bytes, int mode,
                 void* kernel_stream, void* copy_stream);
 
+/* ---------------------------------------------------------------------------
+ * Rotary position embedding, alone or fused with the K/V write.
+ * (Widening beyond the copy path: the rotation runs immediately before the
+ * write on the same K tensor, runtime/worker/llm_worker/models/llama.py:156-167.)
+ * Replaces rotary_pos_emb / apply_rotary_pos_emb_kernel
+ *   (runtime/worker/llm_worker/ops/rotary_embedding_ops.py:8-35,
+ *    runtime/worker/llm_worker/ops/triton/rotary_embedding.py:5-66):
+ * for token t with p = positions[t], every head, and lane i in [0, rotary_dim/2):
+ *   x = in[i], y = in[rotary_dim/2 + i]
+ *   out[i]                = x*cos[p, i]                - y*sin[p, i]
+ *   out[rotary_dim/2 + i] = y*cos[p, rotary_dim/2 + i] + x*sin[p, rotary_dim/2 + i]
+ * with cos_sin_cache[max_position, 2*rotary_dim] = cos | sin in the tensors'
+ * dtype (runtime/worker/llm_worker/models/layers/rotary_embedding.py:62-70).
+ * Arithmetic is fp32 with one rounding to the storage dtype. Lanes in
+ * [rotary_dim, head_dim) are copied through (the reference leaves them
+ * unwritten). query_out may alias query, key_out may alias key. A position
+ * outside [0, max_position) leaves the token untouched. Strides in elements.
+ *
+ * _and_cache / _and_append_paged additionally store the ROTATED key row and
+ * the value row into the token's cache slot, addressed exactly as
+ * kvc_reshape_and_cache / kvc_append_paged_kv_cache address it (one layer);
+ * key_out may then be NULL. In the page-table form `positions` serves both
+ * the rotation and the page lookup, as the reference passes the same values
+ * for both (runtime/worker/llm_worker/model_worker.py:346, :425-433).
+ * ------------------------------------------------------------------------- */
+typedef enum kvc_dtype { KVC_DTYPE_BF16 = 0, KVC_DTYPE_F16 = 1, KVC_DTYPE_F32 = 2 } kvc_dtype;
+
+int kvc_rotary_pos_emb(const void* query, const void* key, const void* positions, int pos_bytes,
+                       const void* cos_sin_cache, int64_t max_position, int64_t num_tokens,
+                       int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                       int64_t rotary_dim, int64_t q_token_stride, int64_t k_token_stride,
+                       void* query_out, void* key_out, int64_t qo_token_stride,
+                       int64_t ko_token_stride, int dtype, void* stream);
+
+int kvc_rotary_pos_emb_and_cache(const void* query, const void* key, const void* value,
+                                 const void* positions, int pos_bytes, const void* cos_sin_cache,
+                                 int64_t max_position, int64_t num_tokens, int64_t num_heads,
+                                 int64_t num_kv_heads, int64_t head_dim, int64_t rotary_dim,
+                                 int64_t q_token_stride, int64_t k_token_stride,
+                                 int64_t v_token_stride, void* query_out, void* key_out,
+                                 int64_t qo_token_stride, int64_t ko_token_stride,
+                                 void* key_cache, void* value_cache, const void* slot_mapping,
+                                 int slot_bytes, int64_t block_size, int64_t cache_block_stride,
+                                 int64_t cache_slot_stride, int64_t num_cache_blocks, int dtype,
+                                 void* stream);
+
+int kvc_rotary_pos_emb_and_append_paged(const void* query, const void* key, const void* value,
+                                        const int32_t* batch_indices, const int32_t* positions,
+                                        const void* cos_sin_cache, int64_t max_position,
+                                        int64_t nnz, int64_t num_heads, int64_t num_kv_heads,
+                                        int64_t head_dim, int64_t rotary_dim,
+                                        int64_t q_token_stride, int64_t k_token_stride,
+                                        int64_t v_token_stride, void* query_out, void* key_out,
+                                        int64_t qo_token_stride, int64_t ko_token_stride,
+                                        void* paged_kv_cache, const int32_t* kv_indices,
+                                        const int32_t* kv_indptr, int64_t batch_size,
+                                        int64_t num_kv_indices, int64_t page_size,
+                                        int64_t page_stride, int64_t num_pages, int dtype,
+                                        void* stream);
+
 /* Pinned, device-addressable host memory for the host pool; replaces
  * pycuda.driver.pagelocked_empty (runtime/worker/llm_worker/kv_worker.py:123-127).
  * Returns NULL on failure. */

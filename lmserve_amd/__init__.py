@@ -4,6 +4,7 @@
     paged       append_paged_kv_cache(_layers), get_seq_lens, get_batch_indices_positions
     kv_worker   KVWorker (GPU <-> pinned host swap), Device, BlockMapping
     index_prep  host-side block-table / slot-mapping construction
+    rotary      rotary position embedding, alone or fused with the K/V write
     kv_pool     pool sizing, allocator id order, layer-sync handle and model-side hooks
 
 Every operator runs a hand-written HIP kernel from libkvcache.so through the
@@ -18,6 +19,8 @@ from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
                       allocate_kv_caches, plan_cache)
 from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
                         flatten_block_mappings)
+from .rotary import (RotaryEmbedding, make_cos_sin_cache, rotary_pos_emb,
+                     rotary_pos_emb_and_append_paged, rotary_pos_emb_and_cache)
 from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cache_layers,
                     build_write_index, get_batch_indices_positions, get_seq_lens)
 
@@ -28,6 +31,8 @@ __all__ = [
     "get_batch_indices_positions",
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",
     "flatten_block_mappings",
+    "RotaryEmbedding", "make_cos_sin_cache", "rotary_pos_emb", "rotary_pos_emb_and_cache",
+    "rotary_pos_emb_and_append_paged",
     "BlockAllocator", "CachePlan", "KVWorkerHandle", "LayerSyncHooks", "allocate_kv_caches",
     "plan_cache",
     "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device", "to_device_one_launch",

@@ -23,6 +23,10 @@ KVC_ERR_HIP = -5
 KVC_SWAP_STAGED = 0
 KVC_SWAP_DIRECT = 1
 
+KVC_DTYPE_BF16 = 0
+KVC_DTYPE_F16 = 1
+KVC_DTYPE_F32 = 2
+
 _I64 = c_int64
 _P = c_void_p
 
@@ -45,6 +49,15 @@ SIGNATURES = {
     "kvc_get_batch_indices_positions": (c_int, [_P, _P, _I64, _I64, _P, _P, _P]),
     "kvc_build_write_index": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P,
                                       _P]),
+    "kvc_rotary_pos_emb": (c_int, [_P, _P, _P, c_int, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                   _I64, _P, _P, _I64, _I64, c_int, _P]),
+    "kvc_rotary_pos_emb_and_cache": (c_int, [_P, _P, _P, _P, c_int, _P, _I64, _I64, _I64, _I64, _I64,
+                                             _I64, _I64, _I64, _I64, _P, _P, _I64, _I64, _P, _P, _P,
+                                             c_int, _I64, _I64, _I64, _I64, c_int, _P]),
+    "kvc_rotary_pos_emb_and_append_paged": (c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64,
+                                                    _I64, _I64, _I64, _I64, _I64, _P, _P, _I64, _I64,
+                                                    _P, _P, _P, _I64, _I64, _I64, _I64, _I64, c_int,
+                                                    _P]),
     "kvc_copy_blocks": (c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _P]),
     "kvc_swap_staging_bytes": (_I64, [_I64, _I64, _I64, c_int, _I64]),
     "kvc_swap_out": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,

@@ -1,6 +1,6 @@
 """Build libkvcache.so (HIP, gfx950) in-tree with hipcc.
 
-`python -m lmserve_amd.build` compiles `csrc/kvcache.hip` into
+`python -m lmserve_amd.build` compiles `csrc/*.hip` into
 `lmserve_amd/libkvcache.so`. hipcc cross-compiles, so no GPU is needed.
 """
 from __future__ import annotations
@@ -12,7 +12,8 @@ import sys
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
-SOURCE = os.path.join(PKG_DIR, "csrc", "kvcache.hip")
+SOURCES = [os.path.join(PKG_DIR, "csrc", "kvcache.hip"),
+           os.path.join(PKG_DIR, "csrc", "rope_cache.hip")]
 INCLUDE = os.path.join(REPO_ROOT, "include")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcache.so")
 
@@ -36,7 +37,7 @@ def find_hipcc() -> str:
 
 def build(verbose: bool = False) -> str:
     """Compile the library; always recompiles. Returns the path of the .so."""
-    cmd = [find_hipcc(), *HIPCC_FLAGS, "-I", INCLUDE, SOURCE, "-o", LIB_PATH + ".tmp"]
+    cmd = [find_hipcc(), *HIPCC_FLAGS, "-I", INCLUDE, *SOURCES, "-o", LIB_PATH + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -1,0 +1,33 @@
+// Helpers shared by the translation units of libkvcache.
+#ifndef KVC_COMMON_H_
+#define KVC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "kvcache.h"
+
+namespace kvc {
+
+// Records the message for kvc_last_error_string() on this thread and returns `code`.
+int fail(int code, const char* fmt, ...);
+
+inline int log2_exact(int64_t x) {
+  if (x <= 0 || (x & (x - 1))) return -1;
+  int s = 0;
+  while ((int64_t(1) << s) < x) ++s;
+  return s;
+}
+
+}  // namespace kvc
+
+#define KVC_HIP(call)                                                          \
+  do {                                                                         \
+    hipError_t e_ = (call);                                                    \
+    if (e_ != hipSuccess)                                                      \
+      return kvc::fail(KVC_ERR_HIP, "%s failed: %s (%s:%d)", #call,            \
+                       hipGetErrorString(e_), __FILE__, __LINE__);             \
+  } while (0)
+
+#endif  // KVC_COMMON_H_

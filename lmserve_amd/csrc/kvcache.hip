@@ -32,13 +32,13 @@
 #include <cstring>
 #include <vector>
 
+#include "common.h"
 #include "kvcache.h"
 
-namespace {
-
 // ---------------------------------------------------------------------------
-// error plumbing
+// error plumbing (shared with the other translation units through common.h)
 // ---------------------------------------------------------------------------
+namespace kvc {
 thread_local char g_err[512] = "";
 
 int fail(int code, const char* fmt, ...) {
@@ -48,14 +48,10 @@ int fail(int code, const char* fmt, ...) {
   va_end(ap);
   return code;
 }
+}  // namespace kvc
 
-#define KVC_HIP(call)                                                          \
-  do {                                                                         \
-    hipError_t e_ = (call);                                                    \
-    if (e_ != hipSuccess)                                                      \
-      return fail(KVC_ERR_HIP, "%s failed: %s (%s:%d)", #call,                 \
-                  hipGetErrorString(e_), __FILE__, __LINE__);                  \
-  } while (0)
+namespace {
+using kvc::fail;
 
 // ---------------------------------------------------------------------------
 // tuning knobs (kvc_set_tuning); defaults are the measured best on MI355X
@@ -389,12 +385,7 @@ __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
 // ---------------------------------------------------------------------------
 // host helpers
 // ---------------------------------------------------------------------------
-inline int log2_exact(int64_t x) {
-  if (x <= 0 || (x & (x - 1))) return -1;
-  int s = 0;
-  while ((int64_t(1) << s) < x) ++s;
-  return s;
-}
+using kvc::log2_exact;
 
 // widest vector (bytes) that divides every value given (addresses and strides)
 inline int common_vec(std::initializer_list<uint64_t> vals) {
@@ -879,7 +870,7 @@ extern "C" {
 
 int kvc_abi_version(void) { return KVC_ABI_VERSION; }
 
-const char* kvc_last_error_string(void) { return g_err; }
+const char* kvc_last_error_string(void) { return kvc::g_err; }
 
 // Tuning hook for sweeps (not part of the reference surface): returns 0, or
 // KVC_ERR_INVALID_ARG for an unknown key.

@@ -1,0 +1,441 @@
+// Rotary position embedding fused with the K/V write (gfx950).
+//
+// In the reference's attention layer the rotation of Q and K runs as its own
+// launch immediately before the cache write, on the same K tensor. Here one
+// workgroup owns one token: it stages the token's cos/sin row in LDS once
+// (as fp32, shared by every head), rotates Q and K in fp32 with a single
+// rounding to the storage type, and, when a cache is given, stores the rotated
+// K and the V row straight into the token's slot. K is read once and V never
+// takes a separate launch. Without a cache the kernel is the plain rotation.
+//
+// Vectors are 16 bytes (8 bf16/fp16 or 4 fp32 elements); a "pair-vector" is the
+// x half and the y half of the same rotation lanes of one head.
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "common.h"
+#include "kvcache.h"
+
+namespace {
+
+using kvc::fail;
+using kvc::log2_exact;
+
+constexpr int kThreads = 256;
+constexpr int kMaxRotaryDim = 512;  // cos + sin of one position in LDS as fp32: 4 KiB
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---- storage types ---------------------------------------------------------
+struct BF16 {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float load(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+  static __device__ __forceinline__ uint16_t store(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest, ties to even
+    return (uint16_t)(u >> 16);
+  }
+};
+struct F16 {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float load(uint16_t b) { return __half2float(__ushort_as_half(b)); }
+  static __device__ __forceinline__ uint16_t store(float f) { return __half_as_ushort(__float2half_rn(f)); }
+};
+struct F32 {
+  static constexpr int kBytes = 4;
+};
+
+// unpack / pack one 16-byte vector to fp32 lanes
+template <typename T>
+struct Vec {
+  static constexpr int kElems = 16 / T::kBytes;
+  static __device__ __forceinline__ void unpack(u32x4 v, float* out) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[2 * i] = T::load((uint16_t)(v[i] & 0xffffu));
+      out[2 * i + 1] = T::load((uint16_t)(v[i] >> 16));
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* in) {
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      v[i] = (uint32_t)T::store(in[2 * i]) | ((uint32_t)T::store(in[2 * i + 1]) << 16);
+    return v;
+  }
+  static __device__ __forceinline__ float load1(const char* p) { return T::load(*(const uint16_t*)p); }
+  static __device__ __forceinline__ void store1(char* p, float f) { *(uint16_t*)p = T::store(f); }
+};
+template <>
+struct Vec<F32> {
+  static constexpr int kElems = 4;
+  static __device__ __forceinline__ void unpack(u32x4 v, float* out) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = __uint_as_float(v[i]);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* in) {
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __float_as_uint(in[i]);
+    return v;
+  }
+  static __device__ __forceinline__ float load1(const char* p) { return *(const float*)p; }
+  static __device__ __forceinline__ void store1(char* p, float f) { *(float*)p = f; }
+};
+
+struct RopeArgs {
+  const char* query;
+  const char* key;
+  const char* value;       // null without a cache
+  char* query_out;
+  char* key_out;           // may be null when a cache takes the rotated K
+  const void* positions;   // rotation positions; with page-table addressing also the KV positions
+  int pos_bytes;
+  const char* cos_sin_cache;  // [max_position, 2*rotary_dim]: cos | sin
+  int64_t max_position;
+  uint32_t num_heads, num_kv_heads, head_dim, rotary_dim;
+  int64_t q_token_stride, k_token_stride, v_token_stride;     // bytes
+  int64_t qo_token_stride, ko_token_stride;                   // bytes
+  // cache side (key_cache == null: plain rotation)
+  char* key_cache;
+  char* value_cache;
+  const void* slot_mapping;
+  int slot_bytes;
+  const int32_t* batch_indices;  // non-null: page-table addressing
+  const int32_t* kv_indices;
+  const int32_t* kv_indptr;
+  int64_t batch_size, num_kv_indices;
+  int64_t block_size;
+  int bs_shift;
+  int64_t cache_block_stride, cache_slot_stride;  // bytes
+  int64_t num_cache_blocks;
+};
+
+template <typename T, bool VECTOR>
+__global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
+  using VT = Vec<T>;
+  constexpr int EV = VECTOR ? VT::kElems : 1;
+  constexpr int E = T::kBytes;
+  __shared__ float cs[2 * kMaxRotaryDim];  // cos[0, rd) | sin[0, rd)
+
+  const int64_t t = blockIdx.x;
+  const int64_t pos = a.pos_bytes == 8 ? reinterpret_cast<const int64_t*>(a.positions)[t]
+                                       : (int64_t) reinterpret_cast<const int32_t*>(a.positions)[t];
+  if (pos < 0 || pos >= a.max_position) return;  // no cos/sin row: the token is left alone
+  const uint32_t rd = a.rotary_dim;
+  const uint32_t half = rd >> 1;
+  const char* cs_row = a.cos_sin_cache + pos * (int64_t)(2 * rd) * E;
+  for (uint32_t i = threadIdx.x; i < 2 * rd; i += blockDim.x) cs[i] = VT::load1(cs_row + (int64_t)i * E);
+
+  // slot of this token (workgroup-uniform), resolved while the cos/sin row lands
+  char* kc_row = nullptr;
+  char* vc_row = nullptr;
+  if (a.key_cache) {
+    int64_t blk = -1, off = 0;
+    if (a.batch_indices) {
+      const int64_t b = a.batch_indices[t];
+      if (b >= 0 && b < a.batch_size) {
+        const int64_t pg = a.bs_shift >= 0 ? (pos >> a.bs_shift) : pos / a.block_size;
+        off = pos - pg * a.block_size;
+        const int64_t it = (int64_t)a.kv_indptr[b] + pg;
+        if (it >= 0 && it < a.num_kv_indices) blk = a.kv_indices[it];
+      }
+    } else {
+      const int64_t s = a.slot_bytes == 8 ? reinterpret_cast<const int64_t*>(a.slot_mapping)[t]
+                                          : (int64_t) reinterpret_cast<const int32_t*>(a.slot_mapping)[t];
+      if (s >= 0) {
+        blk = a.bs_shift >= 0 ? (s >> a.bs_shift) : s / a.block_size;
+        off = s - blk * a.block_size;
+      }
+    }
+    if (blk >= 0 && blk < a.num_cache_blocks) {
+      const int64_t slot_off = blk * a.cache_block_stride + off * a.cache_slot_stride;
+      kc_row = a.key_cache + slot_off;
+      vc_row = a.value_cache + slot_off;
+    }
+  }
+  __syncthreads();
+
+  const char* q_row = a.query + t * a.q_token_stride;
+  const char* k_row = a.key + t * a.k_token_stride;
+  char* qo_row = a.query_out + t * a.qo_token_stride;
+  char* ko_row = a.key_out ? a.key_out + t * a.ko_token_stride : nullptr;
+  const uint32_t D = a.head_dim;
+  const uint32_t heads = a.num_heads + a.num_kv_heads;
+
+  // 1. rotation: item = (head over Q then K, pair-vector)
+  const uint32_t pv_per_head = half / EV;
+  const uint32_t rot_items = heads * pv_per_head;
+  for (uint32_t item = threadIdx.x; item < rot_items; item += blockDim.x) {
+    const uint32_t h = item / pv_per_head;
+    const uint32_t e0 = (item - h * pv_per_head) * EV;  // first rotation lane of this item
+    const bool is_k = h >= a.num_heads;
+    const uint32_t hh = is_k ? h - a.num_heads : h;
+    const char* in = (is_k ? k_row : q_row) + (int64_t)hh * D * E;
+    float x[EV], y[EV], ox[EV], oy[EV];
+    if constexpr (VECTOR) {
+      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)e0 * E), x);
+      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)(half + e0) * E), y);
+    } else {
+      x[0] = VT::load1(in + (int64_t)e0 * E);
+      y[0] = VT::load1(in + (int64_t)(half + e0) * E);
+    }
+#pragma unroll
+    for (int i = 0; i < EV; ++i) {
+      const float cos_x = cs[e0 + i], cos_y = cs[half + e0 + i];
+      const float sin_x = cs[rd + e0 + i], sin_y = cs[rd + half + e0 + i];
+      ox[i] = x[i] * cos_x - y[i] * sin_x;
+      oy[i] = y[i] * cos_y + x[i] * sin_y;
+    }
+    char* outs[2] = {is_k ? ko_row : qo_row, is_k ? kc_row : nullptr};
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+      if (!outs[o]) continue;
+      char* out = outs[o] + (int64_t)hh * D * E;
+      if constexpr (VECTOR) {
+        *reinterpret_cast<u32x4*>(out + (int64_t)e0 * E) = VT::pack(ox);
+        *reinterpret_cast<u32x4*>(out + (int64_t)(half + e0) * E) = VT::pack(oy);
+      } else {
+        VT::store1(out + (int64_t)e0 * E, ox[0]);
+        VT::store1(out + (int64_t)(half + e0) * E, oy[0]);
+      }
+    }
+  }
+
+  // 2. lanes beyond rotary_dim pass through unchanged (partial rotary)
+  if (rd < D) {
+    const uint32_t tail = (D - rd) / EV;
+    const uint32_t tail_items = heads * tail;
+    for (uint32_t item = threadIdx.x; item < tail_items; item += blockDim.x) {
+      const uint32_t h = item / tail;
+      const uint32_t e0 = rd + (item - h * tail) * EV;
+      const bool is_k = h >= a.num_heads;
+      const uint32_t hh = is_k ? h - a.num_heads : h;
+      const int64_t o = ((int64_t)hh * D + e0) * E;
+      const char* in = (is_k ? k_row : q_row) + o;
+      char* outs[2] = {is_k ? ko_row : qo_row, is_k ? kc_row : nullptr};
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (!outs[k]) continue;
+        if constexpr (VECTOR) *reinterpret_cast<u32x4*>(outs[k] + o) = *reinterpret_cast<const u32x4*>(in);
+        else VT::store1(outs[k] + o, VT::load1(in));
+      }
+    }
+  }
+
+  // 3. the V row goes to the cache as it is
+  if (vc_row) {
+    const char* v_row = a.value + t * a.v_token_stride;
+    const uint32_t v_items = a.num_kv_heads * D / EV;
+    for (uint32_t item = threadIdx.x; item < v_items; item += blockDim.x) {
+      const int64_t o = (int64_t)item * EV * E;
+      if constexpr (VECTOR)
+        __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(v_row + o),
+                                    reinterpret_cast<u32x4*>(vc_row + o));
+      else VT::store1(vc_row + o, VT::load1(v_row + o));
+    }
+  }
+}
+
+template <typename T>
+void launch_rope(const RopeArgs& a, int64_t num_tokens, bool vector, hipStream_t s) {
+  if (vector)
+    hipLaunchKernelGGL((rope_cache_kernel<T, true>), dim3((unsigned)num_tokens), dim3(kThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((rope_cache_kernel<T, false>), dim3((unsigned)num_tokens), dim3(kThreads), 0, s, a);
+}
+
+struct RopeGeom {
+  int64_t num_tokens, num_heads, num_kv_heads, head_dim, rotary_dim, max_position;
+  int64_t q_token_stride, k_token_stride, v_token_stride, qo_token_stride, ko_token_stride;  // elements
+  int dtype;
+};
+
+struct CacheGeom {
+  void* key_cache;
+  void* value_cache;
+  const void* slot_mapping;
+  int slot_bytes;
+  const int32_t* batch_indices;
+  const int32_t* kv_indices;
+  const int32_t* kv_indptr;
+  int64_t batch_size, num_kv_indices;
+  int64_t block_size, cache_block_stride, cache_slot_stride, num_cache_blocks;  // strides in elements
+};
+
+int run_rope(const char* fn, const void* query, const void* key, const void* value,
+             void* query_out, void* key_out, const void* positions, int pos_bytes,
+             const void* cos_sin_cache, const RopeGeom& g, const CacheGeom* c, void* stream) {
+  int E;
+  switch (g.dtype) {
+    case KVC_DTYPE_BF16: case KVC_DTYPE_F16: E = 2; break;
+    case KVC_DTYPE_F32: E = 4; break;
+    default: return fail(KVC_ERR_UNSUPPORTED, "%s: dtype %d (need bf16, f16 or f32)", fn, g.dtype);
+  }
+  if (g.num_tokens < 0 || g.num_heads < 0 || g.num_kv_heads < 0 || g.head_dim <= 0 ||
+      g.rotary_dim < 0 || g.max_position < 0)
+    return fail(KVC_ERR_INVALID_ARG, "%s: negative size", fn);
+  if (g.rotary_dim > g.head_dim || (g.rotary_dim & 1))
+    return fail(KVC_ERR_INVALID_ARG, "%s: rotary_dim %lld must be even and <= head_dim %lld", fn,
+                (long long)g.rotary_dim, (long long)g.head_dim);
+  if (g.rotary_dim > kMaxRotaryDim)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: rotary_dim %lld exceeds %d", fn, (long long)g.rotary_dim,
+                kMaxRotaryDim);
+  if (pos_bytes != 4 && pos_bytes != 8)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: pos_bytes=%d (need 4 or 8)", fn, pos_bytes);
+  if (g.num_tokens > 0x7fffffffll || g.num_heads + g.num_kv_heads > 0xffffll)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: too many tokens or heads", fn);
+  if (g.num_tokens == 0 || g.num_heads + g.num_kv_heads == 0) return KVC_OK;
+  if (!query || !key || !query_out || !positions || !cos_sin_cache)
+    return fail(KVC_ERR_INVALID_ARG, "%s: null pointer", fn);
+  if (!c && !key_out) return fail(KVC_ERR_INVALID_ARG, "%s: no destination for the rotated key", fn);
+  if (g.q_token_stride < g.num_heads * g.head_dim || g.qo_token_stride < g.num_heads * g.head_dim ||
+      g.k_token_stride < g.num_kv_heads * g.head_dim ||
+      (key_out && g.ko_token_stride < g.num_kv_heads * g.head_dim))
+    return fail(KVC_ERR_INVALID_ARG, "%s: token stride smaller than a row", fn);
+
+  RopeArgs a{};
+  a.query = (const char*)query;
+  a.key = (const char*)key;
+  a.value = (const char*)value;
+  a.query_out = (char*)query_out;
+  a.key_out = (char*)key_out;
+  a.positions = positions;
+  a.pos_bytes = pos_bytes;
+  a.cos_sin_cache = (const char*)cos_sin_cache;
+  a.max_position = g.max_position;
+  a.num_heads = (uint32_t)g.num_heads;
+  a.num_kv_heads = (uint32_t)g.num_kv_heads;
+  a.head_dim = (uint32_t)g.head_dim;
+  a.rotary_dim = (uint32_t)g.rotary_dim;
+  a.q_token_stride = g.q_token_stride * E;
+  a.k_token_stride = g.k_token_stride * E;
+  a.v_token_stride = g.v_token_stride * E;
+  a.qo_token_stride = g.qo_token_stride * E;
+  a.ko_token_stride = g.ko_token_stride * E;
+
+  uint64_t align = (uintptr_t)query | (uintptr_t)key | (uintptr_t)query_out | (uintptr_t)key_out |
+                   (uint64_t)a.q_token_stride | (uint64_t)a.k_token_stride |
+                   (uint64_t)a.qo_token_stride | (uint64_t)a.ko_token_stride;
+  if (c) {
+    if (!value || !c->key_cache || !c->value_cache)
+      return fail(KVC_ERR_INVALID_ARG, "%s: null value/cache pointer", fn);
+    if (g.v_token_stride < g.num_kv_heads * g.head_dim)
+      return fail(KVC_ERR_INVALID_ARG, "%s: value token stride smaller than a row", fn);
+    if (c->block_size <= 0 || c->num_cache_blocks < 0 || c->cache_block_stride < 0 ||
+        c->cache_slot_stride < g.num_kv_heads * g.head_dim)
+      return fail(KVC_ERR_INVALID_ARG, "%s: bad cache geometry", fn);
+    if (c->batch_indices) {
+      if (!c->kv_indices || !c->kv_indptr || c->batch_size < 0 || c->num_kv_indices < 0)
+        return fail(KVC_ERR_INVALID_ARG, "%s: bad page-table arguments", fn);
+      if (pos_bytes != 4)
+        return fail(KVC_ERR_UNSUPPORTED, "%s: page-table addressing takes int32 positions", fn);
+    } else {
+      if (!c->slot_mapping) return fail(KVC_ERR_INVALID_ARG, "%s: null slot_mapping", fn);
+      if (c->slot_bytes != 4 && c->slot_bytes != 8)
+        return fail(KVC_ERR_UNSUPPORTED, "%s: slot_bytes=%d (need 4 or 8)", fn, c->slot_bytes);
+    }
+    a.key_cache = (char*)c->key_cache;
+    a.value_cache = (char*)c->value_cache;
+    a.slot_mapping = c->slot_mapping;
+    a.slot_bytes = c->slot_bytes;
+    a.batch_indices = c->batch_indices;
+    a.kv_indices = c->kv_indices;
+    a.kv_indptr = c->kv_indptr;
+    a.batch_size = c->batch_size;
+    a.num_kv_indices = c->num_kv_indices;
+    a.block_size = c->block_size;
+    a.bs_shift = log2_exact(c->block_size);
+    a.cache_block_stride = c->cache_block_stride * E;
+    a.cache_slot_stride = c->cache_slot_stride * E;
+    a.num_cache_blocks = c->num_cache_blocks;
+    align |= (uintptr_t)value | (uintptr_t)c->key_cache | (uintptr_t)c->value_cache |
+             (uint64_t)a.v_token_stride | (uint64_t)a.cache_block_stride |
+             (uint64_t)a.cache_slot_stride;
+  }
+  // 16-byte vectors need aligned rows and halves that hold whole vectors
+  const int ev = 16 / E;
+  const bool vector = (align % 16 == 0) && ((g.rotary_dim / 2) % ev == 0) &&
+                      ((g.head_dim - g.rotary_dim) % ev == 0) && (g.head_dim % ev == 0);
+  hipStream_t s = (hipStream_t)stream;
+  switch (g.dtype) {
+    case KVC_DTYPE_BF16: launch_rope<BF16>(a, g.num_tokens, vector, s); break;
+    case KVC_DTYPE_F16: launch_rope<F16>(a, g.num_tokens, vector, s); break;
+    default: launch_rope<F32>(a, g.num_tokens, vector, s); break;
+  }
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int kvc_rotary_pos_emb(const void* query, const void* key, const void* positions, int pos_bytes,
+                       const void* cos_sin_cache, int64_t max_position, int64_t num_tokens,
+                       int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                       int64_t rotary_dim, int64_t q_token_stride, int64_t k_token_stride,
+                       void* query_out, void* key_out, int64_t qo_token_stride,
+                       int64_t ko_token_stride, int dtype, void* stream) {
+  RopeGeom g{num_tokens, num_heads, num_kv_heads, head_dim, rotary_dim, max_position,
+             q_token_stride, k_token_stride, 0, qo_token_stride, ko_token_stride, dtype};
+  return run_rope("kvc_rotary_pos_emb", query, key, nullptr, query_out, key_out, positions,
+                  pos_bytes, cos_sin_cache, g, nullptr, stream);
+}
+
+int kvc_rotary_pos_emb_and_cache(const void* query, const void* key, const void* value,
+                                 const void* positions, int pos_bytes, const void* cos_sin_cache,
+                                 int64_t max_position, int64_t num_tokens, int64_t num_heads,
+                                 int64_t num_kv_heads, int64_t head_dim, int64_t rotary_dim,
+                                 int64_t q_token_stride, int64_t k_token_stride,
+                                 int64_t v_token_stride, void* query_out, void* key_out,
+                                 int64_t qo_token_stride, int64_t ko_token_stride,
+                                 void* key_cache, void* value_cache, const void* slot_mapping,
+                                 int slot_bytes, int64_t block_size, int64_t cache_block_stride,
+                                 int64_t cache_slot_stride, int64_t num_cache_blocks, int dtype,
+                                 void* stream) {
+  RopeGeom g{num_tokens, num_heads, num_kv_heads, head_dim, rotary_dim, max_position,
+             q_token_stride, k_token_stride, v_token_stride, qo_token_stride, ko_token_stride, dtype};
+  CacheGeom c{key_cache, value_cache, slot_mapping, slot_bytes, nullptr, nullptr, nullptr, 0, 0,
+              block_size, cache_block_stride, cache_slot_stride, num_cache_blocks};
+  return run_rope("kvc_rotary_pos_emb_and_cache", query, key, value, query_out, key_out, positions,
+                  pos_bytes, cos_sin_cache, g, &c, stream);
+}
+
+int kvc_rotary_pos_emb_and_append_paged(const void* query, const void* key, const void* value,
+                                        const int32_t* batch_indices, const int32_t* positions,
+                                        const void* cos_sin_cache, int64_t max_position,
+                                        int64_t nnz, int64_t num_heads, int64_t num_kv_heads,
+                                        int64_t head_dim, int64_t rotary_dim,
+                                        int64_t q_token_stride, int64_t k_token_stride,
+                                        int64_t v_token_stride, void* query_out, void* key_out,
+                                        int64_t qo_token_stride, int64_t ko_token_stride,
+                                        void* paged_kv_cache, const int32_t* kv_indices,
+                                        const int32_t* kv_indptr, int64_t batch_size,
+                                        int64_t num_kv_indices, int64_t page_size,
+                                        int64_t page_stride, int64_t num_pages, int dtype,
+                                        void* stream) {
+  if (nnz > 0 && !batch_indices)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_pos_emb_and_append_paged: null batch_indices");
+  if (num_kv_heads < 0 || head_dim <= 0 || page_size <= 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_pos_emb_and_append_paged: bad H/D/page_size");
+  const int64_t row = num_kv_heads * head_dim;
+  if (page_stride < 2 * page_size * row)
+    return fail(KVC_ERR_INVALID_ARG,
+                "kvc_rotary_pos_emb_and_append_paged: page_stride %lld < 2*page_size*H*D",
+                (long long)page_stride);
+  const int E = dtype == KVC_DTYPE_F32 ? 4 : 2;
+  RopeGeom g{nnz, num_heads, num_kv_heads, head_dim, rotary_dim, max_position,
+             q_token_stride, k_token_stride, v_token_stride, qo_token_stride, ko_token_stride, dtype};
+  char* vc = paged_kv_cache ? (char*)paged_kv_cache + page_size * row * E : nullptr;
+  CacheGeom c{paged_kv_cache, vc, nullptr, 0, batch_indices, kv_indices, kv_indptr, batch_size,
+              num_kv_indices, page_size, page_stride, row, num_pages};
+  return run_rope("kvc_rotary_pos_emb_and_append_paged", query, key, value, query_out, key_out,
+                  positions, 4, cos_sin_cache, g, &c, stream);
+}
+
+}  // extern "C"

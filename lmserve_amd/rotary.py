@@ -1,0 +1,220 @@
+"""Rotary position embedding, alone or fused with the K/V write.
+
+Mirrors runtime/worker/llm_worker/ops/rotary_embedding_ops.py:8-35
+(`rotary_pos_emb`) and the cos/sin table of
+runtime/worker/llm_worker/models/layers/rotary_embedding.py:11-70
+(`RotaryEmbedding`, llama3 frequency scaling included). The fused forms add the
+cache write that follows the rotation in the reference's attention layer
+(runtime/worker/llm_worker/models/llama.py:156-167,
+ runtime/worker/llm_worker/models/layers/attention.py:76-85), so K is read
+once and the write costs no launch of its own.
+
+Arithmetic: fp32 with one rounding to the tensors' dtype.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from .cache_ops import _SLOT_DTYPES, _inner_contiguous, _on_device_of, _require_gpu, _stream_of
+
+_DTYPES = {torch.bfloat16: _lib.KVC_DTYPE_BF16, torch.float16: _lib.KVC_DTYPE_F16,
+           torch.float32: _lib.KVC_DTYPE_F32}
+
+
+def make_cos_sin_cache(rotary_dim: int, max_position_embeddings: int, base: float = 10000.0,
+                       rope_scaling: Optional[dict] = None, dtype: torch.dtype = torch.bfloat16,
+                       device=None) -> torch.Tensor:
+    """`[max_position, 2*rotary_dim]` = cos(emb) | sin(emb), emb = cat(freqs, freqs),
+    freqs[p, i] = p * inv_freq[i]; computed in fp32 and cast to `dtype`
+    (rotary_embedding.py:27-70). `rope_scaling` is the llama3 dict with keys
+    factor, low_freq_factor, high_freq_factor, original_max_position_embeddings."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.int64).float() / rotary_dim))
+    if rope_scaling is not None:
+        factor = rope_scaling["factor"]
+        low_freq_factor = rope_scaling["low_freq_factor"]
+        high_freq_factor = rope_scaling["high_freq_factor"]
+        old_context_len = rope_scaling["original_max_position_embeddings"]
+        low_freq_wavelen = old_context_len / low_freq_factor
+        high_freq_wavelen = old_context_len / high_freq_factor
+        wavelen = 2 * math.pi / inv_freq
+        scaled = torch.where(wavelen > low_freq_wavelen, inv_freq / factor, inv_freq)
+        smooth = (old_context_len / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
+        smoothed = (1 - smooth) * scaled / factor + smooth * scaled
+        is_medium = ~(wavelen < high_freq_wavelen) & ~(wavelen > low_freq_wavelen)
+        inv_freq = torch.where(is_medium, smoothed, scaled)
+    t = torch.arange(max_position_embeddings).float()
+    freqs = torch.einsum("i,j->ij", t, inv_freq.float())
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos_sin = torch.cat((emb.cos().to(dtype), emb.sin().to(dtype)), dim=-1)
+    return cos_sin.to(device) if device is not None else cos_sin
+
+
+def _prep(query, key, positions, cos_sin_cache, head_dim):
+    for t, n in ((query, "query"), (key, "key"), (positions, "positions"),
+                 (cos_sin_cache, "cos_sin_cache")):
+        _require_gpu(t, n)
+    kd = _DTYPES.get(query.dtype)
+    if kd is None:
+        raise TypeError(f"Unsupported dtype: {query.dtype}")
+    if key.dtype != query.dtype or cos_sin_cache.dtype != query.dtype:
+        raise TypeError("query, key and cos_sin_cache must share one dtype")
+    num_tokens = positions.shape[0]
+    q2 = query.reshape(num_tokens, -1)
+    k2 = key.reshape(num_tokens, -1)
+    if q2.stride(-1) != 1:
+        q2 = q2.contiguous()
+    if k2.stride(-1) != 1:
+        k2 = k2.contiguous()
+    if q2.shape[1] % head_dim or k2.shape[1] % head_dim:
+        raise ValueError("query/key width is not a multiple of head_dim")
+    pos_bytes = _SLOT_DTYPES.get(positions.dtype)
+    if pos_bytes is None:
+        raise TypeError("positions must be int32 or int64")
+    if not positions.is_contiguous():
+        positions = positions.contiguous()
+    if cos_sin_cache.dim() != 2 or cos_sin_cache.shape[1] % 2 or not cos_sin_cache.is_contiguous():
+        raise ValueError("cos_sin_cache must be contiguous [max_position, 2*rotary_dim]")
+    return q2, k2, positions, pos_bytes, kd, num_tokens
+
+
+def _tok_stride(t2):
+    return t2.stride(0) if t2.shape[0] > 1 else t2.shape[1]
+
+
+def rotary_pos_emb(query: torch.Tensor, key: torch.Tensor, positions: torch.Tensor,
+                   cos_sin_cache: torch.Tensor, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Rotate `query [T, Hq*D]` and `key [T, Hkv*D]`; returns new tensors of the
+    inputs' shapes (rotary_embedding_ops.py:8-35)."""
+    q2, k2, positions, pos_bytes, kd, T = _prep(query, key, positions, cos_sin_cache, head_dim)
+    q_out = torch.empty_like(q2, memory_format=torch.contiguous_format)
+    k_out = torch.empty_like(k2, memory_format=torch.contiguous_format)
+    if T > 0:
+        with _on_device_of(q2):
+            _lib.check(_lib.lib().kvc_rotary_pos_emb(
+                q2.data_ptr(), k2.data_ptr(), positions.data_ptr(), pos_bytes,
+                cos_sin_cache.data_ptr(), cos_sin_cache.shape[0], T, q2.shape[1] // head_dim,
+                k2.shape[1] // head_dim, head_dim, cos_sin_cache.shape[1] // 2, _tok_stride(q2),
+                _tok_stride(k2), q_out.data_ptr(), k_out.data_ptr(), q_out.shape[1], k_out.shape[1],
+                kd, _stream_of(q2)))
+    return q_out.view(query.shape), k_out.view(key.shape)
+
+
+def rotary_pos_emb_and_cache(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                             positions: torch.Tensor, cos_sin_cache: torch.Tensor, head_dim: int,
+                             kv_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                             return_key: bool = True):
+    """`rotary_pos_emb` plus the slot-mapped write of the rotated key and the
+    value into one layer of the pool, `kv_cache [num_blocks, 2, block_size, H, D]`.
+    Returns `(q_out, k_out)`; `k_out` is None with `return_key=False`."""
+    q2, k2, positions, pos_bytes, kd, T = _prep(query, key, positions, cos_sin_cache, head_dim)
+    for t, n in ((value, "value"), (kv_cache, "kv_cache"), (slot_mapping, "slot_mapping")):
+        _require_gpu(t, n)
+    if value.dtype != query.dtype or kv_cache.dtype != query.dtype:
+        raise TypeError("value and kv_cache must have the query's dtype")
+    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2 or not _inner_contiguous(kv_cache):
+        raise ValueError("kv_cache must be [num_blocks, 2, block_size, H, D] with contiguous blocks")
+    nb, _, bs, H, D = kv_cache.shape
+    v2 = value.reshape(T, -1)
+    if v2.stride(-1) != 1:
+        v2 = v2.contiguous()
+    if D != head_dim or k2.shape[1] != H * D or v2.shape[1] != H * D:
+        raise ValueError("key/value rows do not match the cache's H*D")
+    if slot_mapping.shape[0] != T:
+        raise ValueError("slot_mapping length differs from the number of tokens")
+    slot_bytes = _SLOT_DTYPES.get(slot_mapping.dtype)
+    if slot_bytes is None:
+        slot_mapping, slot_bytes = slot_mapping.to(torch.int64), 8
+    if not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.contiguous()
+    q_out = torch.empty_like(q2, memory_format=torch.contiguous_format)
+    k_out = torch.empty_like(k2, memory_format=torch.contiguous_format) if return_key else None
+    if T > 0 and nb > 0:
+        elem = kv_cache.element_size()
+        row = H * D
+        with _on_device_of(q2):
+            _lib.check(_lib.lib().kvc_rotary_pos_emb_and_cache(
+                q2.data_ptr(), k2.data_ptr(), v2.data_ptr(), positions.data_ptr(), pos_bytes,
+                cos_sin_cache.data_ptr(), cos_sin_cache.shape[0], T, q2.shape[1] // head_dim, H,
+                head_dim, cos_sin_cache.shape[1] // 2, _tok_stride(q2), _tok_stride(k2),
+                _tok_stride(v2), q_out.data_ptr(), k_out.data_ptr() if return_key else None,
+                q_out.shape[1], row, kv_cache.data_ptr(), kv_cache.data_ptr() + bs * row * elem,
+                slot_mapping.data_ptr(), slot_bytes, bs,
+                kv_cache.stride(0) if nb > 1 else 2 * bs * row, row, nb, kd, _stream_of(q2)))
+    return q_out.view(query.shape), (k_out.view(key.shape) if return_key else None)
+
+
+def rotary_pos_emb_and_append_paged(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                    batch_indices: torch.Tensor, positions: torch.Tensor,
+                                    cos_sin_cache: torch.Tensor, head_dim: int,
+                                    paged_kv_cache: torch.Tensor, kv_indices: torch.Tensor,
+                                    kv_indptr: torch.Tensor, kv_last_page_len: torch.Tensor,
+                                    return_key: bool = True):
+    """`rotary_pos_emb` plus `append_paged_kv_cache` of the rotated key and the
+    value in one launch; `positions` (int32) is both the rotation position and
+    the KV position of each token, as in the reference."""
+    q2, k2, positions, pos_bytes, kd, T = _prep(query, key, positions, cos_sin_cache, head_dim)
+    if pos_bytes != 4:
+        raise TypeError("positions must be int32 for page-table addressing")
+    for t, n in ((value, "value"), (paged_kv_cache, "paged_kv_cache")):
+        _require_gpu(t, n)
+    for t, n in ((batch_indices, "batch_indices"), (kv_indices, "kv_indices"),
+                 (kv_indptr, "kv_indptr"), (kv_last_page_len, "kv_last_page_len")):
+        _require_gpu(t, n)
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise TypeError(f"{n} must be contiguous int32")
+    if value.dtype != query.dtype or paged_kv_cache.dtype != query.dtype:
+        raise TypeError("value and paged_kv_cache must have the query's dtype")
+    if paged_kv_cache.dim() != 5 or paged_kv_cache.shape[1] != 2 or \
+            not _inner_contiguous(paged_kv_cache):
+        raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
+    num_pages, _, page_size, H, D = paged_kv_cache.shape
+    v2 = value.reshape(T, -1)
+    if v2.stride(-1) != 1:
+        v2 = v2.contiguous()
+    if D != head_dim or k2.shape[1] != H * D or v2.shape[1] != H * D:
+        raise ValueError("key/value rows do not match the cache's H*D")
+    if batch_indices.numel() != T:
+        raise ValueError("batch_indices and positions differ in length")
+    q_out = torch.empty_like(q2, memory_format=torch.contiguous_format)
+    k_out = torch.empty_like(k2, memory_format=torch.contiguous_format) if return_key else None
+    if T > 0 and num_pages > 0:
+        row = H * D
+        with _on_device_of(q2):
+            _lib.check(_lib.lib().kvc_rotary_pos_emb_and_append_paged(
+                q2.data_ptr(), k2.data_ptr(), v2.data_ptr(), batch_indices.data_ptr(),
+                positions.data_ptr(), cos_sin_cache.data_ptr(), cos_sin_cache.shape[0], T,
+                q2.shape[1] // head_dim, H, head_dim, cos_sin_cache.shape[1] // 2, _tok_stride(q2),
+                _tok_stride(k2), _tok_stride(v2), q_out.data_ptr(),
+                k_out.data_ptr() if return_key else None, q_out.shape[1], row,
+                paged_kv_cache.data_ptr(), kv_indices.data_ptr(), kv_indptr.data_ptr(),
+                kv_indptr.numel() - 1, kv_indices.numel(), page_size,
+                paged_kv_cache.stride(0) if num_pages > 1 else 2 * page_size * row, num_pages, kd,
+                _stream_of(q2)))
+    return q_out.view(query.shape), (k_out.view(key.shape) if return_key else None)
+
+
+class RotaryEmbedding(torch.nn.Module):
+    """`RotaryEmbedding` of the reference (rotary_embedding.py:11-80): builds the
+    cos/sin table from a HF-style config and rotates `(query, key)` in `forward`."""
+
+    def __init__(self, config, base: int = 10000) -> None:
+        super().__init__()
+        base = getattr(config, "rope_theta", base)
+        partial_rotary_factor = getattr(config, "partial_rotary_factor", 1.0)
+        head_dim = getattr(config, "head_dim", None) or \
+            config.hidden_size // config.num_attention_heads
+        self.rotary_dim = int(head_dim * partial_rotary_factor)
+        self.max_position_embeddings = config.max_position_embeddings
+        self.head_dim = head_dim
+        cos_sin = make_cos_sin_cache(self.rotary_dim, self.max_position_embeddings, base,
+                                     getattr(config, "rope_scaling", None),
+                                     getattr(config, "torch_dtype", torch.bfloat16))
+        self.register_buffer("cos_sin_cached", cos_sin, persistent=False)
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor,
+                positions: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        return rotary_pos_emb(query, key, positions, self.cos_sin_cached, self.head_dim)

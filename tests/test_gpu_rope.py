@@ -1,0 +1,198 @@
+"""GPU checks of the rotary embedding, alone and fused with the K/V write.
+
+Floating point: the rotated values must lie within HALF AN ULP of the storage
+dtype (plus fp32 evaluation error) of the float64 formula -- tolerance
+`eps*|exact|*1.01 + 2^-21*(|a|+|b|)` with eps = 2^-8 (bf16), 2^-11 (fp16),
+2^-24 (fp32) and a, b the two products of the lane. The cache side of the
+fused kernel is held bit-exactly to the kernel's own rotated key and to the
+input value rows, and to the copy-path oracle for placement.
+"""
+import numpy as np
+import pytest
+import torch
+
+import lmserve_amd as kvc
+from lmserve_amd import rotary
+from lmserve_amd import workloads as wl
+from oracle import kvc_oracle as orc
+from oracle import rope_oracle as ro
+
+pytestmark = pytest.mark.gpu
+
+EPS = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -24}
+
+
+def _case(gpu, T, Hq, Hkv, D, rd, dtype, max_pos=4096, seed=0, scaling=None):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(T, Hq * D, generator=g).to(dtype)
+    k = torch.randn(T, Hkv * D, generator=g).to(dtype)
+    v = torch.randn(T, Hkv * D, generator=g).to(dtype)
+    pos = torch.randint(0, max_pos, (T,), generator=g, dtype=torch.int32)
+    cs = rotary.make_cos_sin_cache(rd, max_pos, 500000.0, scaling, dtype=dtype)
+    return q, k, v, pos, cs
+
+
+def _check_rotation(got, x, pos, cs, D, dtype, which):
+    """got: rotated tensor from the GPU; x: input; both CPU tensors of dtype."""
+    T = x.shape[0]
+    exact_q, exact_k = ro.rotary_pos_emb_f64(x.double().numpy(), x.double().numpy(), pos.numpy(),
+                                             cs.double().numpy(), D)
+    exact = exact_q
+    rd = cs.shape[1] // 2
+    xh = np.abs(x.double().numpy()).reshape(T, -1, D)
+    prod = np.zeros_like(xh)
+    half = rd // 2
+    prod[:, :, :half] = xh[:, :, :half] + xh[:, :, half:rd]       # |x cos| + |y sin| <= |x| + |y|
+    prod[:, :, half:rd] = prod[:, :, :half]
+    tol = EPS[dtype] * np.abs(exact) * 1.01 + 2.0 ** -21 * prod.reshape(T, -1) + 1e-30
+    err = np.abs(got.double().numpy() - exact)
+    assert (err <= tol).all(), f"{which}: max excess {(err - tol).max()}"
+    # pass-through lanes are bit-exact
+    if rd < D:
+        assert torch.equal(got.reshape(T, -1, D)[:, :, rd:], x.reshape(T, -1, D)[:, :, rd:])
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,rd,dtype", [
+    (256, 32, 8, 128, 128, torch.bfloat16),     # Llama-3-8B decode batch
+    (300, 28, 4, 128, 128, torch.bfloat16),     # Qwen2.5-7B
+    (64, 32, 8, 64, 64, torch.float16),         # Llama-3.2-1B heads
+    (50, 4, 2, 64, 32, torch.bfloat16),         # partial rotary
+    (40, 3, 1, 20, 12, torch.bfloat16),         # odd sizes: scalar path
+    (33, 4, 4, 32, 32, torch.float32),
+    (1, 32, 8, 128, 128, torch.bfloat16),
+])
+def test_rotary_pos_emb_within_half_an_ulp(gpu, T, Hq, Hkv, D, rd, dtype):
+    q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, rd, dtype, seed=T)
+    q_out, k_out = kvc.rotary_pos_emb(q.to(gpu), k.to(gpu), pos.to(gpu), cs.to(gpu), D)
+    assert q_out.shape == q.shape and k_out.shape == k.shape and q_out.dtype == dtype
+    _check_rotation(q_out.cpu(), q, pos, cs, D, dtype, "query")
+    _check_rotation(k_out.cpu(), k, pos, cs, D, dtype, "key")
+    # against the torch fp32 reference: identical up to the last bit in a few lanes
+    fq, fk = ro.rotary_pos_emb_fp32(q, k, pos.long(), cs, D)
+    if dtype != torch.float32:      # with fp32 storage there is no final rounding to hide fma contraction
+        same = (q_out.cpu() == fq).float().mean().item()
+        assert same > 0.99, f"only {same:.4f} of the lanes equal the fp32 reference"
+    else:
+        assert torch.allclose(q_out.cpu(), fq, rtol=0, atol=2e-6)
+    # int64 positions give the same bits
+    q64, k64 = kvc.rotary_pos_emb(q.to(gpu), k.to(gpu), pos.long().to(gpu), cs.to(gpu), D)
+    assert torch.equal(q64, q_out) and torch.equal(k64, k_out)
+
+
+def test_llama3_scaled_table_and_3d_inputs(gpu):
+    scaling = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 8192}
+    T, Hq, Hkv, D = 48, 8, 2, 128
+    q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, D, torch.bfloat16, max_pos=20000, scaling=scaling)
+    q3 = q.view(T, Hq, D).to(gpu)
+    q_out, k_out = kvc.rotary_pos_emb(q3, k.to(gpu), pos.to(gpu), cs.to(gpu), D)
+    assert q_out.shape == (T, Hq, D)
+    _check_rotation(q_out.cpu().view(T, -1), q, pos, cs, D, torch.bfloat16, "query")
+
+
+def test_module_mirrors_the_reference_class(gpu):
+    class Cfg:
+        rope_theta = 500000.0
+        hidden_size = 512
+        num_attention_heads = 8
+        max_position_embeddings = 1024
+        torch_dtype = torch.bfloat16
+        rope_scaling = None
+    mod = kvc.RotaryEmbedding(Cfg()).to(gpu)
+    assert mod.cos_sin_cached.shape == (1024, 128) and mod.head_dim == 64
+    q = torch.randn(5, 8 * 64).bfloat16()
+    k = torch.randn(5, 2 * 64).bfloat16()
+    pos = torch.arange(5, dtype=torch.int32)
+    q_out, k_out = mod(q.to(gpu), k.to(gpu), pos.to(gpu))
+    _check_rotation(q_out.cpu(), q, pos, mod.cos_sin_cached.cpu(), 64, torch.bfloat16, "query")
+    assert torch.equal(q_out[0].cpu(), q[0])          # position 0: cos = 1, sin = 0 exactly
+
+
+@pytest.mark.parametrize("dtype,D,rd", [(torch.bfloat16, 128, 128), (torch.float16, 64, 64),
+                                         (torch.bfloat16, 64, 32), (torch.bfloat16, 20, 12),
+                                         (torch.float32, 32, 32)])
+def test_fused_slot_mapped_write_places_the_rotated_key_bit_exactly(gpu, dtype, D, rd):
+    T, Hq, Hkv, nb, bs = 70, 8, 2, 24, 16
+    q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, rd, dtype, seed=3)
+    rng = np.random.default_rng(4)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    pool = torch.zeros(nb, 2, bs, Hkv, D, dtype=dtype, device=gpu)
+    plain_q, plain_k = kvc.rotary_pos_emb(q.to(gpu), k.to(gpu), pos.to(gpu), cs.to(gpu), D)
+    q_out, k_out = kvc.rotary_pos_emb_and_cache(q.to(gpu), k.to(gpu), v.to(gpu), pos.to(gpu),
+                                                cs.to(gpu), D, pool, torch.from_numpy(slots).to(gpu))
+    assert torch.equal(q_out, plain_q) and torch.equal(k_out, plain_k)
+    # placement: the pool must equal the copy-path oracle fed with the kernel's own rotated key
+    width = {2: np.uint16, 4: np.uint32}[q.element_size()]
+    as_bits = lambda t: t.cpu().contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32).numpy().view(width)
+    want = np.zeros((nb, 2, bs, Hkv, D), dtype=width)
+    orc.reshape_and_cache_np(as_bits(k_out).reshape(T, Hkv, D), as_bits(v).reshape(T, Hkv, D), want, slots)
+    assert np.array_equal(as_bits(pool), want)
+    # without returning the key: same pool, no k_out
+    pool2 = torch.zeros_like(pool)
+    q2, none = kvc.rotary_pos_emb_and_cache(q.to(gpu), k.to(gpu), v.to(gpu), pos.to(gpu), cs.to(gpu),
+                                            D, pool2, torch.from_numpy(slots).to(gpu), return_key=False)
+    assert none is None and torch.equal(q2, plain_q) and torch.equal(pool2, pool)
+
+
+def test_fused_paged_write_equals_rotation_then_append(gpu):
+    s = wl.LLAMA_3_8B
+    rng = np.random.default_rng(9)
+    filled = [0, 37, 5, 64, 200, 16, 15]
+    new = [70, 1, 1, 33, 1, 16, 2]
+    w = wl._write_workload(s, 256, filled, new, rng)
+    idx = kvc.to_device(w.index, s.block_size, gpu)
+    T, Hq, Hkv, D = w.num_tokens, 32, s.num_kv_heads, s.head_dim
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(T, Hq * D, generator=g).bfloat16().to(gpu)
+    k = torch.randn(T, Hkv * D, generator=g).bfloat16().to(gpu)
+    v = torch.randn(T, Hkv * D, generator=g).bfloat16().to(gpu)
+    cs = rotary.make_cos_sin_cache(D, 4096, 500000.0, dtype=torch.bfloat16).to(gpu)
+    # two launches, as the reference runs them
+    pool_a = torch.zeros(256, 2, s.block_size, Hkv, D, dtype=torch.bfloat16, device=gpu)
+    q_a, k_a = kvc.rotary_pos_emb(q, k, idx.positions, cs, D)
+    kvc.append_paged_kv_cache(k_a.view(T, Hkv, D), v.view(T, Hkv, D), idx.batch_indices,
+                              idx.positions, pool_a, idx.kv_block_indices, idx.kv_block_indptrs,
+                              idx.kv_last_block_lens)
+    # one launch
+    pool_b = torch.zeros_like(pool_a)
+    q_b, k_b = kvc.rotary_pos_emb_and_append_paged(q, k, v, idx.batch_indices, idx.positions, cs, D,
+                                                   pool_b, idx.kv_block_indices,
+                                                   idx.kv_block_indptrs, idx.kv_last_block_lens)
+    torch.cuda.synchronize()
+    assert torch.equal(q_a, q_b) and torch.equal(k_a, k_b)
+    assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+    assert int(torch.count_nonzero(pool_b.view(torch.int16))) > 0
+
+
+def test_in_place_rotation_and_guards(gpu):
+    T, Hq, Hkv, D = 20, 4, 2, 64
+    q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, D, torch.bfloat16, max_pos=100)
+    dq, dk, dpos, dcs = q.to(gpu), k.to(gpu), pos.to(gpu), cs.to(gpu)
+    want_q, want_k = kvc.rotary_pos_emb(dq, dk, dpos, dcs, D)
+    # aliasing outputs onto inputs through the C ABI
+    from lmserve_amd import _lib
+    rc = _lib.lib().kvc_rotary_pos_emb(dq.data_ptr(), dk.data_ptr(), dpos.data_ptr(), 4,
+                                       dcs.data_ptr(), 100, T, Hq, Hkv, D, D, Hq * D, Hkv * D,
+                                       dq.data_ptr(), dk.data_ptr(), Hq * D, Hkv * D,
+                                       _lib.KVC_DTYPE_BF16, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.equal(dq, want_q) and torch.equal(dk, want_k)
+    # a position outside the table leaves its token untouched
+    bad = pos.clone()
+    bad[3] = 100
+    bad[7] = -1
+    out_q = torch.full_like(dq, 7.0)
+    out_k = torch.full_like(dk, 7.0)
+    q_in, k_in, dbad = q.to(gpu), k.to(gpu), bad.to(gpu)
+    rc = _lib.lib().kvc_rotary_pos_emb(q_in.data_ptr(), k_in.data_ptr(), dbad.data_ptr(), 4,
+                                       dcs.data_ptr(), 100, T, Hq, Hkv, D, D, Hq * D, Hkv * D,
+                                       out_q.data_ptr(), out_k.data_ptr(), Hq * D, Hkv * D,
+                                       _lib.KVC_DTYPE_BF16, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    keep = [i for i in range(T) if i not in (3, 7)]
+    assert torch.equal(out_q[keep], want_q[keep]) and (out_q[[3, 7]] == 7.0).all()
+    with pytest.raises(TypeError):
+        kvc.rotary_pos_emb(dq.to(torch.int16), dk, dpos, dcs, D)
+    with pytest.raises(ValueError):
+        kvc.rotary_pos_emb(dq, dk, dpos, dcs, 48)
