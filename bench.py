@@ -52,10 +52,11 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=320)
     p.add_argument("--warmup", type=int, default=32)
-    p.add_argument("--ops", default="write,prefill,copy,swap",
+    p.add_argument("--ops", default="write,prefill,copy,swap,rope",
                    help="comma list of extra measurements: write (per-layer / page-table variants "
                         "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
-                        "calib (a plain 1 GiB device copy, for counter calibration); "
+                        "rope (rotation fused with the write vs two launches), "
+                        "calib (a plain elementwise kernel of known size, for counter calibration); "
                         "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=1024,
                    help="blocks per swap direction (config 5 itself is 8192 = 40 GiB pinned)")
@@ -293,7 +294,51 @@ def main():
     bytes_step = sets[0][0].algorithmic_bytes(L)
     value_gbps = bytes_step / (ms_wall * 1e-3) / 1e9
     achieved = bytes_step / (ms_event * 1e-3) / 1e9
-    del sets
+
+    # ------------------------------------------------ rotation + write, per layer (config 2 shape)
+    if "rope" in ops:
+        Hq, Hkv, D, T = 32, s8.num_kv_heads, s8.head_dim, 256
+        cs = kvc.make_cos_sin_cache(D, 8192, 500000.0, dtype=torch.bfloat16).to(dev)
+        R = ROTATE_DECODE
+        qs = [torch.randn(T, Hq * D, device=dev).to(torch.bfloat16) for _ in range(R)]
+        ks = [sets[r][1][0].reshape(T, Hkv * D) for r in range(R)]
+        vs = [sets[r][2][0].reshape(T, Hkv * D) for r in range(R)]
+        idxs = [sets[r][3] for r in range(R)]
+        pool_l = [pool[l] for l in range(L)]
+        E = 2
+        # q read+write, k read + cache write, v read + cache write, cos/sin row, indices
+        rope_bytes = T * (2 * Hq * D * E + 2 * Hkv * D * E + 2 * Hkv * D * E + 2 * D * E + 12)
+
+        def two_launches(i):
+            r = i % R
+            idx = idxs[r]
+            for l in range(L):
+                q_o, k_o = kvc.rotary_pos_emb(qs[r], ks[r], idx.positions, cs, D)
+                kvc.append_paged_kv_cache(k_o, vs[r], idx.batch_indices, idx.positions, pool_l[l],
+                                          idx.kv_block_indices, idx.kv_block_indptrs,
+                                          idx.kv_last_block_lens)
+
+        def fused(i):
+            r = i % R
+            idx = idxs[r]
+            for l in range(L):
+                kvc.rotary_pos_emb_and_append_paged(qs[r], ks[r], vs[r], idx.batch_indices,
+                                                    idx.positions, cs, D, pool_l[l],
+                                                    idx.kv_block_indices, idx.kv_block_indptrs,
+                                                    idx.kv_last_block_lens, return_key=False)
+
+        n = max(R, args.steps // 8 // R * R)
+        for fn, label, extra_b in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
+                                    2 * T * Hkv * D * E),   # rotated key written out and read back
+                                   (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0)):
+            try:
+                ms_w, ms_e = time_region(fn, n, 2, torch, graph_of=R)
+            except Exception as exc:
+                log(f"rope variant skipped: {exc!r}")
+                continue
+            extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes + extra_b, ms_w, ms_e,
+                               calls_per_step=L, launch="hipGraph replay"))
+        del qs, ks, vs, idxs
 
     # ------------------------------------------------ config 4: copy_blocks (same pool)
     if "copy" in ops:
@@ -304,7 +349,7 @@ def main():
                                  max(5, min(args.steps, 20)), 3, torch)
         extra.append(entry(f"cfg4 copy_blocks (4096 pairs x {L} layers, 64 KiB blocks)", nbytes,
                            ms_w, ms_e, launch="eager"))
-    del pool
+    del pool, sets
     torch.cuda.empty_cache()
 
     if "calib" in ops:

@@ -1,12 +1,13 @@
 // Rotary position embedding fused with the K/V write (gfx950).
 //
 // In the reference's attention layer the rotation of Q and K runs as its own
-// launch immediately before the cache write, on the same K tensor. Here one
-// workgroup owns one token: it stages the token's cos/sin row in LDS once
-// (as fp32, shared by every head), rotates Q and K in fp32 with a single
-// rounding to the storage type, and, when a cache is given, stores the rotated
-// K and the V row straight into the token's slot. K is read once and V never
-// takes a separate launch. Without a cache the kernel is the plain rotation.
+// launch immediately before the cache write, on the same K tensor. Here a
+// workgroup owns a run of 16-byte work items of ONE token (so position, cos/sin
+// row and cache slot are workgroup-uniform): it stages the token's cos/sin row
+// in LDS as fp32, rotates Q and K in fp32 with a single rounding to the storage
+// type, and, when a cache is given, stores the rotated K and the V row straight
+// into the token's slot. K is read once and V never takes a separate launch.
+// Without a cache the kernel is the plain rotation.
 //
 // Vectors are 16 bytes (8 bf16/fp16 or 4 fp32 elements); a "pair-vector" is the
 // x half and the y half of the same rotation lanes of one head.
@@ -14,6 +15,7 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 
 #include "common.h"
@@ -113,8 +115,14 @@ struct RopeArgs {
   int bs_shift;
   int64_t cache_block_stride, cache_slot_stride;  // bytes
   int64_t num_cache_blocks;
+  uint32_t groups_per_token;  // workgroups per token
 };
 
+// Work items of one token, in this order: rotation pair-vectors of the Q heads
+// then the K heads, pass-through vectors beyond rotary_dim, V vectors. A
+// workgroup takes blockDim.x consecutive items of one token, one per lane: the
+// lane's global loads are issued first, the cos/sin row is staged in LDS while
+// they are in flight, then the lane computes and stores.
 template <typename T, bool VECTOR>
 __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
   using VT = Vec<T>;
@@ -122,16 +130,71 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
   constexpr int E = T::kBytes;
   __shared__ float cs[2 * kMaxRotaryDim];  // cos[0, rd) | sin[0, rd)
 
-  const int64_t t = blockIdx.x;
+  const uint32_t t = blockIdx.x / a.groups_per_token;
+  const uint32_t group = blockIdx.x - t * a.groups_per_token;
   const int64_t pos = a.pos_bytes == 8 ? reinterpret_cast<const int64_t*>(a.positions)[t]
                                        : (int64_t) reinterpret_cast<const int32_t*>(a.positions)[t];
   if (pos < 0 || pos >= a.max_position) return;  // no cos/sin row: the token is left alone
   const uint32_t rd = a.rotary_dim;
   const uint32_t half = rd >> 1;
+  const uint32_t D = a.head_dim;
+  const uint32_t heads = a.num_heads + a.num_kv_heads;
+  const uint32_t pv_per_head = half / EV;
+  const uint32_t rot_items = heads * pv_per_head;
+  const uint32_t tail_per_head = (D - rd) / EV;
+  const uint32_t tail_items = heads * tail_per_head;
+  const uint32_t v_items = a.key_cache ? a.num_kv_heads * D / EV : 0;
+
+  // ---- this lane's item and its loads ----
+  const uint32_t item = group * blockDim.x + threadIdx.x;
+  enum { kNone, kRotate, kTail, kValue } kind = kNone;
+  bool is_k = false;
+  uint32_t e0 = 0;          // first lane inside the head (rotation / tail)
+  int64_t in_off = 0;       // byte offset of the item inside its source row == inside its out row
+  float x[EV], y[EV];
+  u32x4 raw = {0, 0, 0, 0};
+  float raw1 = 0.f;
+  if (item < rot_items) {
+    kind = kRotate;
+    const uint32_t h = item / pv_per_head;
+    e0 = (item - h * pv_per_head) * EV;
+    is_k = h >= a.num_heads;
+    const uint32_t hh = is_k ? h - a.num_heads : h;
+    in_off = (int64_t)hh * D * E;
+    const char* in = (is_k ? a.key + (int64_t)t * a.k_token_stride
+                           : a.query + (int64_t)t * a.q_token_stride) + in_off;
+    if constexpr (VECTOR) {
+      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)e0 * E), x);
+      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)(half + e0) * E), y);
+    } else {
+      x[0] = VT::load1(in + (int64_t)e0 * E);
+      y[0] = VT::load1(in + (int64_t)(half + e0) * E);
+    }
+  } else if (item < rot_items + tail_items) {
+    kind = kTail;
+    const uint32_t it = item - rot_items;
+    const uint32_t h = it / tail_per_head;
+    e0 = rd + (it - h * tail_per_head) * EV;
+    is_k = h >= a.num_heads;
+    const uint32_t hh = is_k ? h - a.num_heads : h;
+    in_off = ((int64_t)hh * D + e0) * E;
+    const char* in = (is_k ? a.key + (int64_t)t * a.k_token_stride
+                           : a.query + (int64_t)t * a.q_token_stride) + in_off;
+    if constexpr (VECTOR) raw = *reinterpret_cast<const u32x4*>(in);
+    else raw1 = VT::load1(in);
+  } else if (item < rot_items + tail_items + v_items) {
+    kind = kValue;
+    in_off = (int64_t)(item - rot_items - tail_items) * EV * E;
+    const char* in = a.value + (int64_t)t * a.v_token_stride + in_off;
+    if constexpr (VECTOR) raw = *reinterpret_cast<const u32x4*>(in);
+    else raw1 = VT::load1(in);
+  }
+
+  // ---- cos/sin row of this position into LDS (fp32), shared by all heads ----
   const char* cs_row = a.cos_sin_cache + pos * (int64_t)(2 * rd) * E;
   for (uint32_t i = threadIdx.x; i < 2 * rd; i += blockDim.x) cs[i] = VT::load1(cs_row + (int64_t)i * E);
 
-  // slot of this token (workgroup-uniform), resolved while the cos/sin row lands
+  // ---- slot of this token (workgroup-uniform) ----
   char* kc_row = nullptr;
   char* vc_row = nullptr;
   if (a.key_cache) {
@@ -160,30 +223,12 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
   }
   __syncthreads();
 
-  const char* q_row = a.query + t * a.q_token_stride;
-  const char* k_row = a.key + t * a.k_token_stride;
-  char* qo_row = a.query_out + t * a.qo_token_stride;
-  char* ko_row = a.key_out ? a.key_out + t * a.ko_token_stride : nullptr;
-  const uint32_t D = a.head_dim;
-  const uint32_t heads = a.num_heads + a.num_kv_heads;
-
-  // 1. rotation: item = (head over Q then K, pair-vector)
-  const uint32_t pv_per_head = half / EV;
-  const uint32_t rot_items = heads * pv_per_head;
-  for (uint32_t item = threadIdx.x; item < rot_items; item += blockDim.x) {
-    const uint32_t h = item / pv_per_head;
-    const uint32_t e0 = (item - h * pv_per_head) * EV;  // first rotation lane of this item
-    const bool is_k = h >= a.num_heads;
-    const uint32_t hh = is_k ? h - a.num_heads : h;
-    const char* in = (is_k ? k_row : q_row) + (int64_t)hh * D * E;
-    float x[EV], y[EV], ox[EV], oy[EV];
-    if constexpr (VECTOR) {
-      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)e0 * E), x);
-      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)(half + e0) * E), y);
-    } else {
-      x[0] = VT::load1(in + (int64_t)e0 * E);
-      y[0] = VT::load1(in + (int64_t)(half + e0) * E);
-    }
+  // ---- compute and store ----
+  char* qo_row = a.query_out + (int64_t)t * a.qo_token_stride;
+  char* ko_row = a.key_out ? a.key_out + (int64_t)t * a.ko_token_stride : nullptr;
+  char* outs[2] = {is_k ? ko_row : qo_row, is_k ? kc_row : nullptr};
+  if (kind == kRotate) {
+    float ox[EV], oy[EV];
 #pragma unroll
     for (int i = 0; i < EV; ++i) {
       const float cos_x = cs[e0 + i], cos_y = cs[half + e0 + i];
@@ -191,11 +236,10 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
       ox[i] = x[i] * cos_x - y[i] * sin_x;
       oy[i] = y[i] * cos_y + x[i] * sin_y;
     }
-    char* outs[2] = {is_k ? ko_row : qo_row, is_k ? kc_row : nullptr};
 #pragma unroll
     for (int o = 0; o < 2; ++o) {
       if (!outs[o]) continue;
-      char* out = outs[o] + (int64_t)hh * D * E;
+      char* out = outs[o] + in_off;
       if constexpr (VECTOR) {
         *reinterpret_cast<u32x4*>(out + (int64_t)e0 * E) = VT::pack(ox);
         *reinterpret_cast<u32x4*>(out + (int64_t)(half + e0) * E) = VT::pack(oy);
@@ -204,49 +248,27 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
         VT::store1(out + (int64_t)(half + e0) * E, oy[0]);
       }
     }
-  }
-
-  // 2. lanes beyond rotary_dim pass through unchanged (partial rotary)
-  if (rd < D) {
-    const uint32_t tail = (D - rd) / EV;
-    const uint32_t tail_items = heads * tail;
-    for (uint32_t item = threadIdx.x; item < tail_items; item += blockDim.x) {
-      const uint32_t h = item / tail;
-      const uint32_t e0 = rd + (item - h * tail) * EV;
-      const bool is_k = h >= a.num_heads;
-      const uint32_t hh = is_k ? h - a.num_heads : h;
-      const int64_t o = ((int64_t)hh * D + e0) * E;
-      const char* in = (is_k ? k_row : q_row) + o;
-      char* outs[2] = {is_k ? ko_row : qo_row, is_k ? kc_row : nullptr};
+  } else if (kind == kTail) {
+    // lanes beyond rotary_dim pass through unchanged (partial rotary)
 #pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        if (!outs[k]) continue;
-        if constexpr (VECTOR) *reinterpret_cast<u32x4*>(outs[k] + o) = *reinterpret_cast<const u32x4*>(in);
-        else VT::store1(outs[k] + o, VT::load1(in));
-      }
+    for (int o = 0; o < 2; ++o) {
+      if (!outs[o]) continue;
+      if constexpr (VECTOR) *reinterpret_cast<u32x4*>(outs[o] + in_off) = raw;
+      else VT::store1(outs[o] + in_off, raw1);
     }
-  }
-
-  // 3. the V row goes to the cache as it is
-  if (vc_row) {
-    const char* v_row = a.value + t * a.v_token_stride;
-    const uint32_t v_items = a.num_kv_heads * D / EV;
-    for (uint32_t item = threadIdx.x; item < v_items; item += blockDim.x) {
-      const int64_t o = (int64_t)item * EV * E;
-      if constexpr (VECTOR)
-        __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(v_row + o),
-                                    reinterpret_cast<u32x4*>(vc_row + o));
-      else VT::store1(vc_row + o, VT::load1(v_row + o));
-    }
+  } else if (kind == kValue && vc_row) {
+    // the V row goes to the cache as it is
+    if constexpr (VECTOR) __builtin_nontemporal_store(raw, reinterpret_cast<u32x4*>(vc_row + in_off));
+    else VT::store1(vc_row + in_off, raw1);
   }
 }
 
 template <typename T>
-void launch_rope(const RopeArgs& a, int64_t num_tokens, bool vector, hipStream_t s) {
-  if (vector)
-    hipLaunchKernelGGL((rope_cache_kernel<T, true>), dim3((unsigned)num_tokens), dim3(kThreads), 0, s, a);
-  else
-    hipLaunchKernelGGL((rope_cache_kernel<T, false>), dim3((unsigned)num_tokens), dim3(kThreads), 0, s, a);
+void launch_rope(const RopeArgs& a, int64_t num_tokens, bool vector, unsigned threads,
+                 hipStream_t s) {
+  const dim3 grid((unsigned)(num_tokens * a.groups_per_token)), block(threads);
+  if (vector) hipLaunchKernelGGL((rope_cache_kernel<T, true>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((rope_cache_kernel<T, false>), grid, block, 0, s, a);
 }
 
 struct RopeGeom {
@@ -361,11 +383,23 @@ int run_rope(const char* fn, const void* query, const void* key, const void* val
   const int ev = 16 / E;
   const bool vector = (align % 16 == 0) && ((g.rotary_dim / 2) % ev == 0) &&
                       ((g.head_dim - g.rotary_dim) % ev == 0) && (g.head_dim % ev == 0);
+  // one item per lane, two wavefronts per workgroup: a token of the 8B shape
+  // (320 rotation + 128 value vectors) spreads over four workgroups
+  const int64_t ev_used = vector ? ev : 1;
+  const int64_t heads = g.num_heads + g.num_kv_heads;
+  const int64_t items = heads * ((g.rotary_dim / 2) / ev_used) +
+                        heads * ((g.head_dim - g.rotary_dim) / ev_used) +
+                        (c ? g.num_kv_heads * g.head_dim / ev_used : 0);
+  const unsigned threads = 128;
+  a.groups_per_token = (uint32_t)std::max<int64_t>(1, (items + threads - 1) / threads);
+  if (g.num_tokens * (int64_t)a.groups_per_token > 0x7fffffffll)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: launch of %lld workgroups is too large", fn,
+                (long long)(g.num_tokens * (int64_t)a.groups_per_token));
   hipStream_t s = (hipStream_t)stream;
   switch (g.dtype) {
-    case KVC_DTYPE_BF16: launch_rope<BF16>(a, g.num_tokens, vector, s); break;
-    case KVC_DTYPE_F16: launch_rope<F16>(a, g.num_tokens, vector, s); break;
-    default: launch_rope<F32>(a, g.num_tokens, vector, s); break;
+    case KVC_DTYPE_BF16: launch_rope<BF16>(a, g.num_tokens, vector, threads, s); break;
+    case KVC_DTYPE_F16: launch_rope<F16>(a, g.num_tokens, vector, threads, s); break;
+    default: launch_rope<F32>(a, g.num_tokens, vector, threads, s); break;
   }
   KVC_HIP(hipGetLastError());
   return KVC_OK;
