@@ -1,0 +1,204 @@
+// Calls libkvcache through its C ABI from a plain HIP program (no Python, no
+// torch): every operator of the copy path on small seeded inputs, compared
+// byte for byte with the C oracle (oracle/kvc_oracle.c, linked in).
+// Exit status 0 and a final "ABI CHECK PASSED" line on success.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <numeric>
+#include <random>
+#include <vector>
+
+#include "kvcache.h"
+
+extern "C" {
+void oracle_reshape_and_cache(const void*, const void*, void*, const int64_t*, int64_t, int64_t,
+                              int64_t, int64_t, int64_t);
+void oracle_append_paged_kv_cache(const void*, const void*, const int32_t*, const int32_t*, void*,
+                                  const int32_t*, const int32_t*, int64_t, int64_t, int64_t, int64_t,
+                                  int64_t);
+void oracle_copy_blocks(void*, const int64_t*, int64_t, int64_t, int64_t, int64_t, int64_t);
+void oracle_save_blocks_to_host(const void*, void*, const int64_t*, const int64_t*, int64_t, int64_t,
+                                int64_t, int64_t, int64_t, int64_t);
+void oracle_load_blocks_from_host(void*, const void*, const int64_t*, const int64_t*, int64_t,
+                                  int64_t, int64_t, int64_t, int64_t, int64_t);
+}
+
+#define HIP_OK(x)                                                                     \
+  do {                                                                                \
+    hipError_t e_ = (x);                                                              \
+    if (e_ != hipSuccess) {                                                           \
+      std::fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_));                    \
+      return 2;                                                                       \
+    }                                                                                 \
+  } while (0)
+#define KVC_OK_OR_DIE(x)                                                              \
+  do {                                                                                \
+    int rc_ = (x);                                                                    \
+    if (rc_ != KVC_OK) {                                                              \
+      std::fprintf(stderr, "%s -> %d: %s\n", #x, rc_, kvc_last_error_string());       \
+      return 3;                                                                       \
+    }                                                                                 \
+  } while (0)
+
+static int fails = 0;
+static void expect_equal(const char* what, const void* a, const void* b, size_t n) {
+  if (std::memcmp(a, b, n) != 0) {
+    std::fprintf(stderr, "MISMATCH: %s\n", what);
+    ++fails;
+  } else {
+    std::printf("ok: %s\n", what);
+  }
+  std::fflush(stdout);
+}
+
+int main() {
+  const int64_t L = 3, nb = 48, bs = 16, H = 2, D = 64, E = 2;
+  const int64_t row = H * D, blk_elems = 2 * bs * row, blk_bytes = blk_elems * E;
+  const int64_t layer_elems = nb * blk_elems;
+  const size_t pool_bytes = (size_t)(L * layer_elems * E);
+  std::mt19937_64 rng(7);
+  std::vector<uint16_t> pool(L * layer_elems);
+  for (auto& x : pool) x = (uint16_t)rng();
+
+  // --- a mixed step: request 0 appends 20 tokens after 5, request 1 one token after 33
+  std::vector<int32_t> kv_indices = {7, 19, 3, 40, 11, 25};  // tables: [7,19] and [3,40,11]; 25 unused
+  std::vector<int32_t> kv_indptr = {0, 2, 5};
+  std::vector<int32_t> last = {(25 - 1) % 16 + 1, (34 - 1) % 16 + 1};
+  std::vector<int32_t> bi, pos;
+  std::vector<int64_t> slots;
+  for (int p = 5; p < 25; ++p) { bi.push_back(0); pos.push_back(p); slots.push_back((int64_t)kv_indices[p / 16] * 16 + p % 16); }
+  bi.push_back(1); pos.push_back(33); slots.push_back((int64_t)kv_indices[2 + 33 / 16] * 16 + 33 % 16);
+  const int64_t T = (int64_t)bi.size();
+  std::vector<uint16_t> key(L * T * row), value(L * T * row);
+  for (auto& x : key) x = (uint16_t)rng();
+  for (auto& x : value) x = (uint16_t)rng();
+
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+  void *d_pool, *d_key, *d_value, *d_slots, *d_bi, *d_pos, *d_ind, *d_ptr, *d_last, *d_maps;
+  HIP_OK(hipMalloc(&d_pool, pool_bytes));
+  HIP_OK(hipMalloc(&d_key, key.size() * E));
+  HIP_OK(hipMalloc(&d_value, value.size() * E));
+  HIP_OK(hipMalloc(&d_slots, T * 8));
+  HIP_OK(hipMalloc(&d_bi, T * 4));
+  HIP_OK(hipMalloc(&d_pos, T * 4));
+  HIP_OK(hipMalloc(&d_ind, kv_indices.size() * 4));
+  HIP_OK(hipMalloc(&d_ptr, kv_indptr.size() * 4));
+  HIP_OK(hipMalloc(&d_last, last.size() * 4));
+  HIP_OK(hipMemcpy(d_key, key.data(), key.size() * E, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_value, value.data(), value.size() * E, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_slots, slots.data(), T * 8, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_bi, bi.data(), T * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_pos, pos.data(), T * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_ind, kv_indices.data(), kv_indices.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_ptr, kv_indptr.data(), kv_indptr.size() * 4, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_last, last.data(), last.size() * 4, hipMemcpyHostToDevice));
+
+  std::vector<uint16_t> got(pool.size()), want(pool);
+  std::printf("abi version %d\n", kvc_abi_version());
+
+  // 1. slot-mapped write, one launch per layer
+  HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+  for (int64_t l = 0; l < L; ++l) {
+    char* layer = (char*)d_pool + l * layer_elems * E;
+    KVC_OK_OR_DIE(kvc_reshape_and_cache((char*)d_key + l * T * row * E, (char*)d_value + l * T * row * E,
+                                        layer, layer + bs * row * E, d_slots, 8, T, row, row, row, bs,
+                                        blk_elems, row, nb, (int)E, stream));
+    oracle_reshape_and_cache(key.data() + l * T * row, value.data() + l * T * row,
+                             want.data() + l * layer_elems, slots.data(), T, bs, H, D, E);
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+  expect_equal("kvc_reshape_and_cache (per layer) == oracle", got.data(), want.data(), pool_bytes);
+
+  // 2. the same write for all layers in one launch
+  HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+  KVC_OK_OR_DIE(kvc_reshape_and_cache_layers(d_key, d_value, d_pool, (char*)d_pool + bs * row * E,
+                                             d_slots, 8, T, row, row, row, bs, blk_elems, row, nb, L,
+                                             T * row, T * row, layer_elems, (int)E, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+  expect_equal("kvc_reshape_and_cache_layers == oracle", got.data(), want.data(), pool_bytes);
+
+  // 3. page-table addressed write (must land on the same slots)
+  std::vector<uint16_t> want_paged(pool);
+  HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+  for (int64_t l = 0; l < L; ++l) {
+    KVC_OK_OR_DIE(kvc_append_paged_kv_cache(
+        (char*)d_key + l * T * row * E, (char*)d_value + l * T * row * E, (const int32_t*)d_bi,
+        (const int32_t*)d_pos, (char*)d_pool + l * layer_elems * E, (const int32_t*)d_ind,
+        (const int32_t*)d_ptr, (const int32_t*)d_last, T, 2, (int64_t)kv_indices.size(), H, D, bs,
+        row, row, blk_elems, nb, (int)E, stream));
+    oracle_append_paged_kv_cache(key.data() + l * T * row, value.data() + l * T * row, bi.data(),
+                                 pos.data(), want_paged.data() + l * layer_elems, kv_indices.data(),
+                                 kv_indptr.data(), T, H, D, bs, E);
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+  expect_equal("kvc_append_paged_kv_cache == oracle", got.data(), want_paged.data(), pool_bytes);
+  expect_equal("page-table write == slot-mapped write", want_paged.data(), want.data(), pool_bytes);
+
+  // 4. copy_blocks
+  std::vector<int64_t> maps = {7, 0, 7, 1, 19, 30, 5, 5, 40, 47};
+  HIP_OK(hipMalloc(&d_maps, maps.size() * 8));
+  HIP_OK(hipMemcpy(d_maps, maps.data(), maps.size() * 8, hipMemcpyHostToDevice));
+  KVC_OK_OR_DIE(kvc_copy_blocks(d_pool, (const int64_t*)d_maps, (int64_t)maps.size() / 2, L,
+                                layer_elems * E, blk_bytes, nb, stream));
+  oracle_copy_blocks(want.data(), maps.data(), (int64_t)maps.size() / 2, L, layer_elems, blk_elems, E);
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+  expect_equal("kvc_copy_blocks == oracle", got.data(), want.data(), pool_bytes);
+
+  // 5. swap out / in, both modes, through library-pinned host memory
+  const int64_t nhb = 10, n = 6;
+  std::vector<int64_t> out_src = {30, 0, 47, 19, 5, 11}, out_dst = {2, 3, 4, 9, 0, 6};
+  std::vector<int64_t> in_src = {9, 0, 3}, in_dst = {44, 45, 13};
+  const size_t host_bytes = (size_t)(nhb * L * blk_bytes);
+  for (int mode = 0; mode < 2; ++mode) {
+    uint16_t* host = (uint16_t*)kvc_host_alloc_pinned(host_bytes);
+    if (!host) { std::fprintf(stderr, "pinned alloc failed: %s\n", kvc_last_error_string()); return 4; }
+    std::vector<uint16_t> want_host(host_bytes / 2);
+    for (size_t i = 0; i < want_host.size(); ++i) host[i] = want_host[i] = (uint16_t)(0xFFC0 + i % 61);
+    const int64_t staging_bytes = kvc_swap_staging_bytes(n, L, blk_bytes, mode, 2);
+    void* staging;
+    HIP_OK(hipMalloc(&staging, staging_bytes));
+    hipStream_t copy_stream;
+    HIP_OK(hipStreamCreate(&copy_stream));
+    KVC_OK_OR_DIE(kvc_swap_out(d_pool, host, out_src.data(), out_dst.data(), n, L, layer_elems * E,
+                               blk_bytes, nb, nhb, 0, L, staging, staging_bytes, mode, stream, copy_stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    oracle_save_blocks_to_host(want.data(), want_host.data(), out_src.data(), out_dst.data(), n, L, nb,
+                               blk_bytes, 0, L);
+    expect_equal(mode ? "kvc_swap_out (direct) == oracle" : "kvc_swap_out (staged) == oracle", host,
+                 want_host.data(), host_bytes);
+    KVC_OK_OR_DIE(kvc_swap_in(d_pool, host, in_src.data(), in_dst.data(), 3, L, layer_elems * E,
+                              blk_bytes, nb, nhb, 0, L, staging, staging_bytes, mode, stream, copy_stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    oracle_load_blocks_from_host(want.data(), want_host.data(), in_src.data(), in_dst.data(), 3, L, nb,
+                                 blk_bytes, 0, L);
+    HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+    expect_equal(mode ? "kvc_swap_in (direct) == oracle" : "kvc_swap_in (staged) == oracle", got.data(),
+                 want.data(), pool_bytes);
+    // an id outside the host pool is rejected before anything runs
+    std::vector<int64_t> bad = {nhb};
+    const int rc = kvc_swap_out(d_pool, host, out_src.data(), bad.data(), 1, L, layer_elems * E,
+                                blk_bytes, nb, nhb, 0, L, staging, staging_bytes, mode, stream, copy_stream);
+    if (rc != KVC_ERR_OUT_OF_RANGE) { std::fprintf(stderr, "expected KVC_ERR_OUT_OF_RANGE, got %d\n", rc); ++fails; }
+    HIP_OK(hipStreamSynchronize(copy_stream));
+    HIP_OK(hipStreamDestroy(copy_stream));
+    HIP_OK(hipFree(staging));
+    KVC_OK_OR_DIE(kvc_host_free_pinned(host));
+  }
+
+  HIP_OK(hipDeviceSynchronize());
+  if (fails) {
+    std::printf("ABI CHECK FAILED (%d mismatches)\n", fails);
+    return 1;
+  }
+  std::printf("ABI CHECK PASSED\n");
+  return 0;
+}

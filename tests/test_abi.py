@@ -115,3 +115,33 @@ def test_staging_size_arithmetic():
     assert L.kvc_swap_staging_bytes(3, nl, blk, _lib.KVC_SWAP_STAGED, 100) == 256 + 6 * per_block
     assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_DIRECT, 0) == ids
     assert L.kvc_swap_staging_bytes(-1, nl, blk, 0, 0) < 0
+
+
+def test_rope_and_index_build_validate_their_arguments():
+    L = _lib.lib()
+    f = L.kvc_rotary_pos_emb
+    #  q, k, pos, pos_bytes, cs, max_pos, T, Hq, Hkv, D, rd, qs, ks, qo, ko, qos, kos, dtype, stream
+    ok = [256, 256, 256, 4, 256, 100, 4, 8, 2, 64, 64, 512, 128, 256, 256, 512, 128, _lib.KVC_DTYPE_BF16, None]
+
+    def call(**kw):
+        names = ["q", "k", "pos", "pos_bytes", "cs", "max_pos", "T", "Hq", "Hkv", "D", "rd", "qs", "ks",
+                 "qo", "ko", "qos", "kos", "dtype", "stream"]
+        a = list(ok)
+        for k, v in kw.items():
+            a[names.index(k)] = v
+        return f(*a)
+
+    assert call(T=0) == _lib.KVC_OK                         # nothing to do, nothing launched
+    assert call(dtype=7) == _lib.KVC_ERR_UNSUPPORTED
+    assert call(rd=65) == _lib.KVC_ERR_INVALID_ARG          # odd
+    assert call(rd=128) == _lib.KVC_ERR_INVALID_ARG         # beyond head_dim
+    assert call(D=1024, rd=1024, qs=8192, ks=2048, qos=8192, kos=2048) == _lib.KVC_ERR_UNSUPPORTED
+    assert call(pos_bytes=2) == _lib.KVC_ERR_UNSUPPORTED
+    assert call(q=None) == _lib.KVC_ERR_INVALID_ARG
+    assert call(ko=None) == _lib.KVC_ERR_INVALID_ARG        # no cache and no key_out: nowhere to put K
+    assert call(qs=100) == _lib.KVC_ERR_INVALID_ARG         # stride smaller than the row
+    g = L.kvc_build_write_index
+    assert g(None, None, None, None, -1, 0, 16, 0, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
+    assert g(None, None, None, None, 2, 0, 16, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
+    assert g(1, 1, 1, 1, 2, 4, 0, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG   # page_size 0
+    assert L.kvc_set_tuning(b"no_such_knob", 1) == _lib.KVC_ERR_INVALID_ARG
