@@ -175,3 +175,32 @@ def test_disk_tier_round_trip(gpu, tmp_path):
                                                   kvc.Device.Host, kvc.Device.Disk)
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("chunk", [0, 4])
+def test_staged_swap_of_a_layer_range_with_runs_of_consecutive_host_ids(gpu, chunk):
+    """A partial layer range makes each host block a strided row; runs of
+    consecutive host ids then go out as one pitched (2-D) extent."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb = 6, 40, 16
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, "staged", chunk, seed=21)
+    try:
+        rng = np.random.default_rng(22)
+        old = rng.permutation(nb)[:7].astype(np.int64)
+        host_ids = np.asarray([3, 4, 5, 6, 9, 10, 0], dtype=np.int64)   # runs of 4, 2 and 1
+        maps = _mappings(old, host_ids, pieces=1)
+        gpu_np = pool.reshape(L, nb, -1)
+        host_np = w.host_kv_caches.copy()
+        orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids, 1, 4)
+        w.save_kv_blocks_to_host_nowait(maps, layer_begin=1, layer_end=4)
+        w.dtoh_stream.synchronize()
+        assert np.array_equal(w.host_kv_caches, host_np)
+        new = np.setdiff1d(np.arange(nb), old)[:7].astype(np.int64)
+        want = gpu_np.copy()
+        orc.c_load_blocks_from_host(want, host_np, host_ids, new, 2, 5)
+        w.load_kv_blocks_from_host_nowait(_mappings(host_ids, new, pieces=1), layer_begin=2, layer_end=5)
+        w.htod_stream.synchronize()
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), want)
+    finally:
+        w.close()
