@@ -524,13 +524,19 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
   a.items_per_token = (uint32_t)items64;
 
-  // Vectors per lane: a small launch is latency-bound and wants every lane busy
-  // with one vector; a large one wants several loads in flight per lane.
+  // Vectors per lane, from sweeps on MI355X: a small launch is latency-bound and
+  // wants every lane busy with one vector; a launch of some tens of MiB fits the
+  // machine in one resident wave of workgroups and gains from several loads in
+  // flight per lane; beyond that, more and smaller workgroups win again.
   const int64_t launch_bytes = g.num_tokens * g.row_elems * E * 2 * g.num_layers;
   WriteLaunch l{};
   l.vpt = g_tune.write_vpt;
   if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8)
-    l.vpt = launch_bytes >= (int64_t(32) << 20) ? 4 : (launch_bytes >= (int64_t(8) << 20) ? 2 : 1);
+    l.vpt = launch_bytes >= (int64_t(96) << 20)   ? 1   // enough workgroups to fill the machine many
+                                                        // times over: the leanest lane measured best
+            : launch_bytes >= (int64_t(32) << 20) ? 4   // one resident wave of workgroups, 4 loads in flight
+            : launch_bytes >= (int64_t(8) << 20)  ? 2
+                                                  : 1;
   while (l.vpt > 1 && (int64_t)(l.vpt / 2) * kThreads >= items64) l.vpt /= 2;
   const int64_t lanes = (items64 + l.vpt - 1) / l.vpt;
   l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes + 63) / 64 * 64);
