@@ -270,6 +270,8 @@ def main():
     from lmserve_amd import _lib
     from lmserve_amd import workloads as wl
 
+    from lmserve_amd.build import ensure_built
+    ensure_built()  # uses the built library; compiles only if there is none
     _lib.lib()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")

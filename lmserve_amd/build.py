@@ -77,6 +77,15 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+def ensure_built(native_check: bool = False) -> None:
+    """For tests, the smoke check and the benchmark: use what is built, build
+    only what is missing. The operators themselves never build anything."""
+    if not os.path.exists(LIB_PATH):
+        build(verbose=True)
+    if native_check and not os.path.exists(NATIVE_CHECK_BIN):
+        build_native_check(verbose=True)
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
     sys.exit(0)

@@ -10,6 +10,9 @@ if REPO_ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # load what is built; compile only if the library is missing altogether
+    from lmserve_amd.build import ensure_built
+    ensure_built()
 
 
 @pytest.fixture(scope="session")

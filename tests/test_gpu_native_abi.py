@@ -12,7 +12,9 @@ BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "abi_ch
 
 
 def test_c_abi_from_a_plain_hip_program(gpu):
-    assert os.path.exists(BIN), "tests/native/abi_check is not built (run __graft_entry__.build())"
+    from lmserve_amd.build import ensure_built
+    ensure_built(native_check=True)    # builds only if the binary is missing
+    assert os.path.exists(BIN)
     proc = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(proc.stdout)
     print(proc.stderr)
