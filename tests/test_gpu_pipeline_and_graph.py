@@ -208,3 +208,33 @@ def test_graph_replay_of_write_and_copy_matches_eager_every_time(gpu):
                                         want[l], w.index.kv_block_indices, w.index.kv_block_indptrs)
         orc.c_copy_blocks(want, flat)
         assert np.array_equal(bits_of(dpool), want), f"replay {rep} differs from the oracle"
+
+
+def test_dispatcher_registered_ops_run_the_same_kernels(gpu):
+    """torch.ops.kvcache.* (lmserve_amd.torch_ops) mutate their cache argument
+    exactly as the plain functions do."""
+    import lmserve_amd.torch_ops  # noqa: F401  (registers the ops)
+    s = wl.LLAMA_3_2_1B
+    nb, bs = 64, s.block_size
+    w = wl.decode_step(s, num_blocks=nb, batch=16, max_context=40, seed=8)
+    idx = kvc.to_device(w.index, bs, gpu)
+    T = w.num_tokens
+    key, value = bf16_bits((T, s.num_kv_heads, s.head_dim), 1), bf16_bits((T, s.num_kv_heads, s.head_dim), 2)
+    pool = sentinel_pool((2, nb, 2, bs, s.num_kv_heads, s.head_dim), 3)
+    want = pool.copy()
+    orc.c_append_paged_kv_cache(key, value, w.index.batch_indices, w.index.positions, want[0],
+                                w.index.kv_block_indices, w.index.kv_block_indptrs)
+    orc.reshape_and_cache_np(key, value, want[1], w.index.slot_mapping)
+    used = set(w.index.kv_block_indices.tolist())
+    free = [b for b in range(nb) if b not in used]
+    flat = np.asarray([int(w.index.kv_block_indices[0]), free[0]], dtype=np.int64)
+    orc.c_copy_blocks(want, flat)
+    dpool = to_bf16(pool, gpu)
+    dk, dv = to_bf16(key, gpu), to_bf16(value, gpu)
+    torch.ops.kvcache.append_paged_kv_cache(dk, dv, idx.batch_indices, idx.positions, dpool[0],
+                                            idx.kv_block_indices, idx.kv_block_indptrs,
+                                            idx.kv_last_block_lens)
+    torch.ops.kvcache.reshape_and_cache(dk, dv, dpool[1], idx.slot_mapping)
+    torch.ops.kvcache.copy_blocks(dpool, torch.from_numpy(flat).to(gpu))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), want)
