@@ -28,9 +28,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
-#include <vector>
 
 #include "common.h"
 #include "kvcache.h"
@@ -149,11 +147,13 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   const char* value_row = a.value + (int64_t)t * a.value_token_stride;
   const uint32_t first = group * (VPT * blockDim.x) + threadIdx.x;
   V data[VPT];
-  int64_t dst_off[VPT];  // offset inside the slot's row set, < 0 = no item
+  int64_t dst_off[VPT];  // offset from the slot's K (or V) row, < 0 = no item
+  bool to_v[VPT];
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const uint32_t item = first + j * blockDim.x;
     dst_off[j] = -1;
+    to_v[j] = false;
     if (item < a.items_per_token) {
       uint32_t r, vec;
       if (a.vpr_shift >= 0) {
@@ -168,9 +168,8 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
       const char* src = (is_v ? value_row + layer * a.value_layer_stride
                               : key_row + layer * a.key_layer_stride) + (int64_t)vec * VEC;
       data[j] = ld<NTL>(reinterpret_cast<const V*>(src));
-      // bit 0 carries K|V; VEC-aligned offsets leave it free only for VEC >= 2,
-      // so keep the flag in the sign-safe top instead: offsets are far below 2^62
-      dst_off[j] = (layer * a.cache_layer_stride + (int64_t)vec * VEC) | ((int64_t)is_v << 62);
+      dst_off[j] = layer * a.cache_layer_stride + (int64_t)vec * VEC;
+      to_v[j] = is_v;
     }
   }
 
@@ -209,11 +208,8 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   char* vc_row = a.value_cache + slot_off;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    if (dst_off[j] >= 0) {
-      const bool is_v = (dst_off[j] >> 62) & 1;
-      char* dst = (is_v ? vc_row : kc_row) + (dst_off[j] & ~(int64_t(1) << 62));
-      st<NT>(reinterpret_cast<V*>(dst), data[j]);
-    }
+    if (dst_off[j] >= 0)
+      st<NT>(reinterpret_cast<V*>((to_v[j] ? vc_row : kc_row) + dst_off[j]), data[j]);
   }
 }
 
