@@ -49,8 +49,8 @@ def build_native_check(verbose: bool = False) -> str:
     hipcc = find_hipcc()
     steps = [
         ["gcc", "-O2", "-std=c11", "-c", ORACLE_C, "-o", oracle_obj],
-        [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I", INCLUDE, "-c", NATIVE_CHECK_SRC,
-         "-o", main_obj],
+        [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-I", INCLUDE, "-c", NATIVE_CHECK_SRC, "-o", main_obj],
         [hipcc, main_obj, oracle_obj, "-L", PKG_DIR, "-lkvcache",
          "-Wl,-rpath,$ORIGIN/../../lmserve_amd", "-o", NATIVE_CHECK_BIN],
     ]
