@@ -297,6 +297,23 @@ def main():
     value_gbps = bytes_step / (ms_wall * 1e-3) / 1e9
     achieved = bytes_step / (ms_event * 1e-3) / 1e9
 
+    # a plain elementwise kernel moving the same bytes per launch as the headline
+    # (32 MiB read + 32 MiB written), rotated over as many buffers: what a launch
+    # of this size can reach on this machine whatever the kernel
+    same_size = None
+    try:
+        n_el = (bytes_step // 2) // 4
+        srcs = [torch.zeros(n_el, dtype=torch.int32, device=dev) for _ in range(ROTATE_DECODE)]
+        dsts = [torch.empty(n_el, dtype=torch.int32, device=dev) for _ in range(ROTATE_DECODE)]
+        ms_w, ms_e = time_region(lambda i: torch.add(srcs[i % ROTATE_DECODE], 1, out=dsts[i % ROTATE_DECODE]),
+                                 args.steps, args.warmup, torch)
+        same_size = {"kernel": "torch.add(int32, 1, out=...)", "bytes_per_launch": int(n_el * 8),
+                     "us_per_launch": round(ms_e * 1e3, 3),
+                     "gbps": round(n_el * 8 / (ms_e * 1e-3) / 1e9, 1)}
+        del srcs, dsts
+    except Exception as exc:
+        log(f"same-size plain copy skipped: {exc!r}")
+
     # ------------------------------------------------ rotation + write, per layer (config 2 shape)
     if "rope" in ops:
         Hq, Hkv, D, T = 32, s8.num_kv_heads, s8.head_dim, 256
@@ -440,7 +457,8 @@ def main():
                      "traffic": MEASURED_TRAFFIC_CFG2_ONE_LAUNCH
                      if (L == 32 and args.pool_blocks == 65536) else None,
                      "kernel": "write_rows_kernel", "bytes_per_launch": int(bytes_step),
-                     "us_per_launch": round(ms_event * 1e3, 3)},
+                     "us_per_launch": round(ms_event * 1e3, 3),
+                     "plain_kernel_of_same_size": same_size},
         "cpu_baseline": cpu,
         "ops": extra,
     }
