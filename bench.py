@@ -33,6 +33,7 @@ if REPO_ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 ROTATE_DECODE = 16   # 16 x 32 MiB of K/V sources
+PREWARM_S = 0.15     # seconds of untimed launches ahead of every timed region
 ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 
 # HBM bytes per launch of the headline kernel (config 2, all layers in one launch)
@@ -72,7 +73,18 @@ def time_region(fn, steps, warmup, torch, graph_of=0):
     graph_of > 0: the launches of `graph_of` consecutive steps are captured once
     into a hipGraph and the timed region replays it (steps // graph_of) times,
     then runs the remaining steps eagerly -- exactly K steps either way, without
-    the host's per-launch cost between them."""
+    the host's per-launch cost between them.
+
+    Before the W warm-up calls the same fn runs for PREWARM_S of wall time, so
+    that the memory and shader clocks have left their idle state (a cold start
+    reads about 4 % slower on a 13 us launch); those calls are not counted."""
+    t_end = time.perf_counter() + PREWARM_S
+    i = 0
+    while time.perf_counter() < t_end:
+        fn(i)
+        i += 1
+        if i % 64 == 0:
+            torch.cuda.synchronize()
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
@@ -403,6 +415,17 @@ def main():
         out_maps = [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))]
         in_maps = [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))]
         nbytes = n * L5 * s70.block_bytes
+        # the on-device half alone: gather to / scatter from a dense HBM buffer (HBM roofline)
+        ids_out = torch.from_numpy(old).to(dev)
+        ids_in = torch.from_numpy(new).to(dev)
+        dense = torch.empty(n, L5, s70.block_elems, dtype=torch.bfloat16, device=dev)
+        ms_w, ms_e = time_region(lambda i: kvc.gather_blocks(pool5, ids_out, out=dense), 10, 2, torch)
+        extra.append(entry(f"cfg5 gather stage, HBM only ({n} blocks x {L5} layers x 64 KiB -> dense buffer)",
+                           2 * nbytes, ms_w, ms_e, launch="eager"))
+        ms_w, ms_e = time_region(lambda i: kvc.scatter_blocks(pool5, ids_in, dense), 10, 2, torch)
+        extra.append(entry(f"cfg5 scatter stage, HBM only (dense buffer -> {n} blocks x {L5} layers x 64 KiB)",
+                           2 * nbytes, ms_w, ms_e, launch="eager"))
+        del dense
         for mode in ("direct", "staged"):
             worker = kvc.KVWorker(pool5, n, swap_mode=mode)
             try:
@@ -451,7 +474,8 @@ def main():
                                f"({L * args.pool_blocks * s8.block_bytes / 2**30:.0f} GiB)",
                    "entry": "kvc_reshape_and_cache_layers (all layers in one launch)",
                    "launch": "one eager launch per step on torch's current stream",
-                   "rotation": f"{ROTATE_DECODE} K/V source sets and slot sets cycled"},
+                   "rotation": f"{ROTATE_DECODE} K/V source sets and slot sets cycled",
+                   "clock_prewarm_s": PREWARM_S},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_CFG2_ONE_LAUNCH

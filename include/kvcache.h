@@ -56,7 +56,7 @@ const char* kvc_last_error_string(void);
 
 /* Launch-shape knobs for measurement sweeps; process-wide, not thread-safe
  * against concurrent launches. No counterpart in the reference. Keys:
- * "copy_unroll" (1,2,4,8,16), "copy_nt" (0/1), "copy_max_wgs" (0 = one
+ * "copy_unroll" and "gather_unroll" (1,2,4,8,16), "copy_nt" (0/1), "copy_order" (0/1), "copy_max_wgs" (0 = one
  * workgroup per chunk), "write_vpt" (0 = by size, 1, 2, 4, 8), "write_nt" (bit 0: non-temporal stores, bit 1: loads), "write_order" (0/1),
  * "direct_max_wgs". Unknown key: KVC_ERR_INVALID_ARG. */
 int kvc_set_tuning(const char* key, int value);
@@ -302,6 +302,23 @@ int kvc_rotary_pos_emb_and_append_paged(const void* query, const void* key, cons
                                         int64_t num_kv_indices, int64_t page_size,
                                         int64_t page_stride, int64_t num_pages, int dtype,
                                         void* stream);
+
+/* The on-device half of a swap on its own: gather scattered pool blocks into a
+ * dense device buffer laid out like the host pool, [n, layer_end-layer_begin,
+ * block_bytes], or scatter such a buffer back:
+ *   gather : buffer[i, l-layer_begin, :] = pool[l, block_ids[i], :]
+ *   scatter: pool[l, block_ids[i], :]    = buffer[i, l-layer_begin, :]
+ * The same row semantics as kv_worker.py:213-227 / :197-211 of the reference
+ * with the host pool replaced by device memory and host ids 0..n-1; what a
+ * prefill-to-decode hand-off over a device-to-device link would send. block_ids
+ * is an int64 array on the DEVICE; ids outside [0, num_blocks) are skipped. */
+int kvc_gather_blocks(const void* pool, void* buffer, const int64_t* block_ids, int64_t n,
+                      int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                      int64_t num_blocks, int64_t layer_begin, int64_t layer_end, void* stream);
+
+int kvc_scatter_blocks(void* pool, const void* buffer, const int64_t* block_ids, int64_t n,
+                       int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                       int64_t num_blocks, int64_t layer_begin, int64_t layer_end, void* stream);
 
 /* Pinned, device-addressable host memory for the host pool; replaces
  * pycuda.driver.pagelocked_empty (runtime/worker/llm_worker/kv_worker.py:123-127).

@@ -1,6 +1,6 @@
 """MI355X-native paged KV-cache data movement behind LMServe's operator surface.
 
-    cache_ops   copy_blocks, fill_key_cache, reshape_and_cache(_layers)
+    cache_ops   copy_blocks, fill_key_cache, reshape_and_cache(_layers), gather/scatter_blocks
     paged       append_paged_kv_cache(_layers), get_seq_lens, get_batch_indices_positions
     kv_worker   KVWorker (GPU <-> pinned host swap), Device, BlockMapping
     index_prep  host-side block-table / slot-mapping construction
@@ -12,7 +12,7 @@ C ABI of include/kvcache.h; nothing here computes on the CPU.
 """
 from . import _lib
 from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_block_maps,
-                        reshape_and_cache, reshape_and_cache_layers)
+                        gather_blocks, reshape_and_cache, reshape_and_cache_layers, scatter_blocks)
 from .index_prep import (InferInput, KVIndexInputs, make_kv_index_inputs, to_device,
                          to_device_one_launch)
 from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
@@ -26,7 +26,7 @@ from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cac
 
 __all__ = [
     "copy_blocks", "fill_key_cache", "reshape_and_cache", "reshape_and_cache_layers",
-    "flatten_block_maps", "check_block_maps",
+    "flatten_block_maps", "check_block_maps", "gather_blocks", "scatter_blocks",
     "append_paged_kv_cache", "append_paged_kv_cache_layers", "PagedKVWritePlan", "get_seq_lens",
     "get_batch_indices_positions",
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",

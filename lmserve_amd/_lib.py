@@ -59,6 +59,8 @@ SIGNATURES = {
                                                     _P, _P, _P, _I64, _I64, _I64, _I64, _I64, c_int,
                                                     _P]),
     "kvc_copy_blocks": (c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _P]),
+    "kvc_gather_blocks": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
+    "kvc_scatter_blocks": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
     "kvc_swap_staging_bytes": (_I64, [_I64, _I64, _I64, c_int, _I64]),
     "kvc_swap_out": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
                              _I64, c_int, _P, _P]),

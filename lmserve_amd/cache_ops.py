@@ -283,3 +283,56 @@ def reshape_and_cache_layers(
             kv_caches.data_ptr() + bs * row * elem, slot_mapping.data_ptr(), slot_bytes,
             num_tokens, row, row, row, bs, 2 * bs * row, row, nb, L, num_tokens * row,
             num_tokens * row, nb * 2 * bs * row, elem, _stream_of(kv_caches)))
+
+
+def _pool_geometry(kv_caches: torch.Tensor):
+    _require_gpu(kv_caches, "kv_caches")
+    if kv_caches.dim() < 3 or not kv_caches.is_contiguous():
+        raise ValueError("kv_caches must be a contiguous [L, num_blocks, ...] tensor")
+    L, nb = kv_caches.shape[0], kv_caches.shape[1]
+    block_elems = kv_caches[0].numel() // nb if nb else 0
+    elem = kv_caches.element_size()
+    return L, nb, block_elems, block_elems * elem, nb * block_elems * elem
+
+
+def _ids_on_device(block_ids: torch.Tensor, kv_caches: torch.Tensor) -> torch.Tensor:
+    if block_ids.dtype != torch.int64 or block_ids.device != kv_caches.device or block_ids.dim() != 1:
+        raise ValueError("block_ids must be a 1-D int64 tensor on the pool's device")
+    return block_ids if block_ids.is_contiguous() else block_ids.contiguous()
+
+
+def gather_blocks(kv_caches: torch.Tensor, block_ids: torch.Tensor, out: torch.Tensor = None,
+                  layer_begin: int = 0, layer_end: int = None) -> torch.Tensor:
+    """`out[i, l - layer_begin] = kv_caches[l, block_ids[i]]`: scattered pool
+    blocks into a dense device buffer in host-pool layout `[n, layers, block_elems]`
+    (the row order of the reference's host pool, kv_worker.py:123-127)."""
+    L, nb, block_elems, block_bytes, layer_stride = _pool_geometry(kv_caches)
+    block_ids = _ids_on_device(block_ids, kv_caches)
+    layer_end = L if layer_end is None else layer_end
+    n, nl = block_ids.numel(), layer_end - layer_begin
+    if out is None:
+        out = torch.empty(n, max(nl, 0), block_elems, dtype=kv_caches.dtype, device=kv_caches.device)
+    elif out.dtype != kv_caches.dtype or out.device != kv_caches.device or not out.is_contiguous() \
+            or out.numel() != n * nl * block_elems:
+        raise ValueError("out must be a contiguous [n, layers, block_elems] tensor of the pool's dtype")
+    with _on_device_of(kv_caches):
+        _lib.check(_lib.lib().kvc_gather_blocks(
+            kv_caches.data_ptr(), out.data_ptr(), block_ids.data_ptr(), n, L, layer_stride,
+            block_bytes, nb, layer_begin, layer_end, _stream_of(kv_caches)))
+    return out
+
+
+def scatter_blocks(kv_caches: torch.Tensor, block_ids: torch.Tensor, buffer: torch.Tensor,
+                   layer_begin: int = 0, layer_end: int = None) -> None:
+    """`kv_caches[l, block_ids[i]] = buffer[i, l - layer_begin]`: the inverse of `gather_blocks`."""
+    L, nb, block_elems, block_bytes, layer_stride = _pool_geometry(kv_caches)
+    block_ids = _ids_on_device(block_ids, kv_caches)
+    layer_end = L if layer_end is None else layer_end
+    n, nl = block_ids.numel(), layer_end - layer_begin
+    if buffer.dtype != kv_caches.dtype or buffer.device != kv_caches.device \
+            or not buffer.is_contiguous() or buffer.numel() != n * nl * block_elems:
+        raise ValueError("buffer must be a contiguous [n, layers, block_elems] tensor of the pool's dtype")
+    with _on_device_of(kv_caches):
+        _lib.check(_lib.lib().kvc_scatter_blocks(
+            kv_caches.data_ptr(), buffer.data_ptr(), block_ids.data_ptr(), n, L, layer_stride,
+            block_bytes, nb, layer_begin, layer_end, _stream_of(kv_caches)))

@@ -204,3 +204,37 @@ def test_staged_swap_of_a_layer_range_with_runs_of_consecutive_host_ids(gpu, chu
         assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), want)
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("layers", [(0, None), (1, 4)])
+def test_device_gather_and_scatter_match_the_swap_oracle(gpu, layers):
+    """gather_blocks / scatter_blocks are the swap's row semantics with the host
+    pool replaced by a dense device buffer and host ids 0..n-1."""
+    s = wl.LLAMA_3_8B
+    L, nb, n = 5, 48, 13
+    lb, le = layers
+    le = L if le is None else le
+    pool = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), 31)
+    dpool = to_bf16(pool, gpu)
+    rng = np.random.default_rng(32)
+    perm = rng.permutation(nb)
+    ids, fresh = perm[:n].astype(np.int64), perm[n:2 * n].astype(np.int64)
+    gpu_np = pool.reshape(L, nb, -1)
+    want_buf = np.zeros((n, L, gpu_np.shape[2]), dtype=np.uint16)
+    orc.c_save_blocks_to_host(gpu_np, want_buf, ids, np.arange(n), lb, le)
+    buf = kvc.gather_blocks(dpool, torch.from_numpy(ids).to(gpu), layer_begin=lb, layer_end=le)
+    assert buf.shape == (n, le - lb, gpu_np.shape[2])
+    assert np.array_equal(bits_of(buf), want_buf[:, lb:le])
+    assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)          # pool untouched
+    want = gpu_np.copy()
+    orc.c_load_blocks_from_host(want, want_buf, np.arange(n), fresh, lb, le)
+    kvc.scatter_blocks(dpool, torch.from_numpy(fresh).to(gpu), buf, layer_begin=lb, layer_end=le)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), want)
+    # ids outside the pool are skipped, the rest still lands
+    bad = torch.tensor([int(fresh[0]), nb, -1], dtype=torch.int64, device=gpu)
+    out = kvc.gather_blocks(dpool, bad)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(out[0]), want[:, fresh[0]])
+    with pytest.raises(ValueError):
+        kvc.scatter_blocks(dpool, torch.from_numpy(fresh).to(gpu), buf[:, :1].contiguous())
