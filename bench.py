@@ -53,10 +53,11 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=320)
     p.add_argument("--warmup", type=int, default=32)
-    p.add_argument("--ops", default="write,prefill,copy,swap,rope",
+    p.add_argument("--ops", default="write,prefill,copy,swap,rope,shard",
                    help="comma list of extra measurements: write (per-layer / page-table variants "
                         "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
                         "rope (rotation fused with the write vs two launches), "
+                        "shard (one rank's head slice of Llama-3.1-70B at tp=8), "
                         "calib (a plain elementwise kernel of known size, for counter calibration); "
                         "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=1024,
@@ -447,6 +448,46 @@ def main():
             finally:
                 worker.close()
         del pool5
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------ one rank's slice of Llama-3.1-70B at tp=8
+    if "shard" in ops:
+        sh = wl.LLAMA_3_1_70B.shard(8)          # 1 KV head: 256-byte rows, 8 KiB blocks, 80 layers
+        nbs = 65536
+        pool_s, Ls = alloc_pool(torch, sh, nbs, dev)
+        sets_s = write_inputs(torch, kvc, wl.decode_step, sh, Ls, nbs, dev, ROTATE_DECODE, batch=256)
+        es, _ = bench_write_config(torch, kvc, "70B/tp8 shard decode", sets_s, pool_s, Ls, args.steps,
+                                   args.warmup, ["fused_slot:graph", "per_layer_paged:graph"])
+        extra += es
+        maps = [torch.from_numpy(wl.copy_on_write_pairs(nbs, 4096, seed=r)[0]).to(dev) for r in range(2)]
+        nbytes = 2 * 4096 * Ls * sh.block_bytes + 16 * 4096
+        ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool_s, maps[i % 2]), 20, 3, torch)
+        extra.append(entry(f"70B/tp8 shard copy_blocks (4096 pairs x {Ls} layers, 8 KiB blocks)", nbytes,
+                           ms_w, ms_e, launch="eager"))
+        n = min(args.swap_blocks * 4, nbs // 2)
+        old, host_ids, new = wl.swap_round_trip(nbs, n, seed=0)
+        nbytes = n * Ls * sh.block_bytes
+        worker = kvc.KVWorker(pool_s, n, swap_mode="direct")
+        try:
+            for direction, maps_, src, dst in (
+                    ("swap_out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))],
+                     kvc.Device.GPU, kvc.Device.Host),
+                    ("swap_in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))],
+                     kvc.Device.Host, kvc.Device.GPU)):
+                worker.copy_kv_sync(maps_, src, dst)
+                times = []
+                for _ in range(3):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    worker.copy_kv_sync(maps_, src, dst)
+                    times.append(time.perf_counter() - t0)
+                t = sorted(times)[1]
+                extra.append({"name": f"70B/tp8 shard {direction} (direct; {n} blocks x {Ls} layers x 8 KiB)",
+                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                              "bytes_per_call": int(nbytes)})
+        finally:
+            worker.close()
+        del pool_s, sets_s
         torch.cuda.empty_cache()
 
     cpu = None

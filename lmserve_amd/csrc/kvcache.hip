@@ -407,6 +407,21 @@ inline int common_vec(std::initializer_list<uint64_t> vals) {
   return (int)acc;
 }
 
+// Workgroups of kThreads lanes the current device holds at once (2048 lanes per CU).
+int resident_workgroups() {
+  static thread_local int cached_dev = -1, cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 2048;
+  if (dev != cached_dev) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached = cus * (2048 / kThreads);
+    cached_dev = dev;
+  }
+  return cached;
+}
+
 struct WriteLaunch {
   unsigned grid;     // workgroups
   unsigned threads;  // lanes per workgroup
@@ -535,19 +550,27 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
   a.items_per_token = (uint32_t)items64;
 
-  // Vectors per lane, from sweeps on MI355X: a small launch is latency-bound and
-  // wants every lane busy with one vector; a launch of some tens of MiB fits the
-  // machine in one resident wave of workgroups and gains from several loads in
-  // flight per lane; beyond that, more and smaller workgroups win again.
-  const int64_t launch_bytes = g.num_tokens * g.row_elems * E * 2 * g.num_layers;
+  // Vectors per lane, from sweeps on MI355X. One vector per lane (the leanest
+  // lane, the most workgroups) is best whenever the launch is either smaller
+  // than one resident set of workgroups (8 of 256 lanes per CU) or many times
+  // larger. In between, a launch that 2 or 4 vectors per lane shrink to exactly
+  // one resident set runs 3-5 % faster that way (no second round of workgroup
+  // dispatch, several loads in flight per lane): the 64 MiB decode step of an
+  // 8-head model is that case. Rows under 1 KiB never gain: a lane's vectors
+  // then fall in different layers' rows.
   WriteLaunch l{};
   l.vpt = g_tune.write_vpt;
-  if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8)
-    l.vpt = launch_bytes >= (int64_t(96) << 20)   ? 1   // enough workgroups to fill the machine many
-                                                        // times over: the leanest lane measured best
-            : launch_bytes >= (int64_t(32) << 20) ? 4   // one resident wave of workgroups, 4 loads in flight
-            : launch_bytes >= (int64_t(8) << 20)  ? 2
-                                                  : 1;
+  if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8) {
+    l.vpt = 1;
+    const int64_t resident = (int64_t)resident_workgroups();
+    const auto wgs = [&](int v) {
+      return g.num_tokens * ((items64 + (int64_t)v * kThreads - 1) / ((int64_t)v * kThreads));
+    };
+    if (g.row_elems * E >= 1024 && wgs(1) > resident) {
+      if (wgs(2) <= resident) l.vpt = 2;
+      else if (wgs(4) <= resident) l.vpt = 4;
+    }
+  }
   while (l.vpt > 1 && (int64_t)(l.vpt / 2) * kThreads >= items64) l.vpt /= 2;
   const int64_t lanes = (items64 + l.vpt - 1) / l.vpt;
   l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes + 63) / 64 * 64);

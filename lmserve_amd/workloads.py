@@ -43,6 +43,15 @@ class KVShape:
     def block_bytes(self) -> int:
         return self.block_elems * self.elem_bytes
 
+    def shard(self, tp: int) -> "KVShape":
+        """The head slice one rank holds under tensor parallelism of degree `tp`
+        (runtime/worker/llm_worker/models/llama.py:105-106: num_kv_heads // tp_size;
+        block tables and mappings are the same on every rank)."""
+        if tp < 1 or self.num_kv_heads % tp:
+            raise ValueError(f"{self.num_kv_heads} KV heads do not split over {tp} ranks")
+        return KVShape(f"{self.name}/tp{tp}", self.num_layers, self.num_kv_heads // tp,
+                       self.head_dim, self.block_size, self.elem_bytes)
+
 
 LLAMA_3_2_1B = KVShape("llama-3.2-1b", 16, 8, 64)
 LLAMA_3_8B = KVShape("llama-3-8b", 32, 8, 128)
