@@ -53,16 +53,20 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=320)
     p.add_argument("--warmup", type=int, default=32)
-    p.add_argument("--ops", default="write,prefill,copy,swap,rope,shard",
+    p.add_argument("--ops", default="write,prefill,copy,swap,rope,shard,disk",
                    help="comma list of extra measurements: write (per-layer / page-table variants "
                         "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
                         "rope (rotation fused with the write vs two launches), "
                         "shard (one rank's head slice of Llama-3.1-70B at tp=8), "
+                        "disk (host <-> disk tier), "
                         "calib (a plain elementwise kernel of known size, for counter calibration); "
                         "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=1024,
                    help="blocks per swap direction (config 5 itself is 8192 = 40 GiB pinned)")
     p.add_argument("--pool-blocks", type=int, default=65536)
+    p.add_argument("--disk-blocks", type=int, default=256,
+                   help="blocks moved by the disk-tier measurement (5 MiB each)")
+    p.add_argument("--disk-dir", default=None, help="directory of the disk-tier file (default: tmp)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
     return p.parse_args()
@@ -238,6 +242,84 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
         out.append(entry(f"{tag}/{label}", nbytes, ms_w, ms_e, calls_per_step=calls,
                          launch="hipGraph replay" if mode == "graph" else "eager (Python + ctypes per call)"))
     return out, results
+
+
+def bench_disk_tier(kvc, shape_cfg, n, directory):
+    """Whole-block save (to the device, fdatasync included) and load through the
+    native tier, beside the reference's way of doing it: one task per layer on 4
+    threads, one row per entry through a NumPy memory map
+    (runtime/worker/llm_worker/kv_worker.py:229-247, :297-322)."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+
+    import numpy as np
+
+    L, E = shape_cfg.num_layers, shape_cfg.block_elems
+    directory = directory or tempfile.gettempdir()
+    nbytes = n * L * E * 2
+    pinned = kvc.PinnedHostPool((n, L, E), np.uint16)   # the pool the KV worker really holds
+    host = pinned.array
+    host[...] = np.arange(n, dtype=np.uint16)[:, None, None]
+    rng = np.random.default_rng(0)
+    src, dst = rng.permutation(n), rng.permutation(n)
+    out = []
+    path = os.path.join(directory, f"kvc-bench-disk-{os.getpid()}.npy")
+    try:
+        with kvc.DiskTier(path, (n, L, E), np.uint16, direct=True, threads=8) as d:
+            t0 = time.perf_counter()
+            d.save_blocks(host, src, dst)
+            d.sync()
+            t1 = time.perf_counter()
+            d.load_blocks(host, dst, src)
+            t2 = time.perf_counter()
+            direct = d.is_direct
+            staged = d.last_transfer_staged
+        out.append({"name": f"cfg5 rows, Host->Disk ({n} blocks x {L} layers x 64 KiB, native tier, "
+                            f"8 threads, O_DIRECT {'on' if direct else 'refused'}"
+                            f"{', pinned pool staged through aligned buffers' if staged else ''}"
+                            f", fdatasync included)",
+                    "ms_per_call": round((t1 - t0) * 1e3, 1), "disk_gbps": round(nbytes / (t1 - t0) / 1e9, 2),
+                    "bytes_per_call": int(nbytes)})
+        out.append({"name": f"cfg5 rows, Disk->Host ({n} blocks, native tier, "
+                            f"{'from the device' if direct else 'page cache warm'})",
+                    "ms_per_call": round((t2 - t1) * 1e3, 1), "disk_gbps": round(nbytes / (t2 - t1) / 1e9, 2),
+                    "bytes_per_call": int(nbytes)})
+    finally:
+        if os.path.exists(path):
+            os.remove(path)
+    try:
+        mm = np.lib.format.open_memmap(path, mode="w+", dtype=np.uint16, shape=(n, L, E))
+
+        def save_layer(l):
+            for s_, d_ in zip(src, dst):
+                mm[d_][l] = host[s_][l]
+
+        def load_layer(l):
+            for s_, d_ in zip(dst, src):
+                host[d_][l] = mm[s_][l]
+
+        with ThreadPoolExecutor(4) as ex:
+            t0 = time.perf_counter()
+            list(ex.map(save_layer, range(L)))
+            mm.flush()
+            t1 = time.perf_counter()
+            list(ex.map(load_layer, range(L)))
+            t2 = time.perf_counter()
+        del mm
+        out.append({"name": f"cfg5 rows, Host->Disk, port of the reference's memory-map row copies "
+                            f"(4 threads, flush included)",
+                    "ms_per_call": round((t1 - t0) * 1e3, 1), "disk_gbps": round(nbytes / (t1 - t0) / 1e9, 2),
+                    "bytes_per_call": int(nbytes)})
+        out.append({"name": "cfg5 rows, Disk->Host, port of the reference's memory-map row copies "
+                            "(4 threads, page cache warm)",
+                    "ms_per_call": round((t2 - t1) * 1e3, 1), "disk_gbps": round(nbytes / (t2 - t1) / 1e9, 2),
+                    "bytes_per_call": int(nbytes)})
+    finally:
+        if os.path.exists(path):
+            os.remove(path)
+        del host
+        pinned.close()
+    return out
 
 
 def cpu_baseline_write(torch, shape_cfg, L, seconds):
@@ -489,6 +571,13 @@ def main():
             worker.close()
         del pool_s, sets_s
         torch.cuda.empty_cache()
+
+    # ------------------------------------------------ host <-> disk tier (config 5 block rows)
+    if "disk" in ops:
+        try:
+            extra += bench_disk_tier(kvc, wl.LLAMA_3_1_70B, args.disk_blocks, args.disk_dir)
+        except OSError as exc:
+            log(f"disk tier skipped: {exc!r}")
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -40,7 +40,8 @@ typedef enum kvc_status {
   KVC_ERR_UNSUPPORTED = -2,   /* elem_bytes / index width not supported        */
   KVC_ERR_OUT_OF_RANGE = -3,  /* a host-resident block id is outside its pool  */
   KVC_ERR_STAGING = -4,       /* staging buffer too small for the request      */
-  KVC_ERR_HIP = -5            /* a HIP runtime call failed (see error string)  */
+  KVC_ERR_HIP = -5,           /* a HIP runtime call failed (see error string)  */
+  KVC_ERR_IO = -6             /* a file operation of the disk tier failed      */
 } kvc_status;
 
 /* how kvc_swap_out / kvc_swap_in move the bytes over PCIe */
@@ -319,6 +320,58 @@ int kvc_gather_blocks(const void* pool, void* buffer, const int64_t* block_ids, 
 int kvc_scatter_blocks(void* pool, const void* buffer, const int64_t* block_ids, int64_t n,
                        int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
                        int64_t num_blocks, int64_t layer_begin, int64_t layer_end, void* stream);
+
+/*
+ * Host <-> disk tier: whole blocks between the host pool and a block file.
+ * Replaces
+ *   memmap_disk_kv_cache              (runtime/worker/llm_worker/kv_worker.py:48-85)
+ *   _load_layer_kv_blocks_from_disk   (kv_worker.py:229-237)
+ *   _save_layer_kv_blocks_to_disk     (kv_worker.py:239-247)
+ *   load/save_kv_blocks_from/to_disk  (kv_worker.py:297-322, one task per layer on 4 threads)
+ * The file is a NumPy `.npy` array of shape (num_blocks, num_layers, block_elems)
+ * and dtype string `descr` ("<u2" for bf16 lanes carried as uint16, kv_worker.py:17-22).
+ * kvc_disk_open reuses a file whose stored shape and dtype match and removes and
+ * recreates any other, as the reference does; a new file is sparse and starts
+ * its data at byte 4096. With KVC_DISK_DIRECT the transfers bypass the page
+ * cache (O_DIRECT) whenever the data offset and one block's bytes over all
+ * layers are multiples of 4096 and the file system allows it; otherwise they are
+ * ordinary buffered reads and writes. The host side of an O_DIRECT transfer is
+ * handed to the kernel in place when the pool is 4096-aligned ordinary memory;
+ * a pool the kernel cannot pin (EFAULT: memory mapped by the GPU driver, i.e.
+ * kvc_host_alloc_pinned) or an unaligned one goes through a 4 MiB aligned
+ * staging buffer per thread.
+ *   save: disk[dst_disk_ids[i]] = host[src_host_ids[i]]   (all layers of the block)
+ *   load: host[dst_host_ids[i]] = disk[src_disk_ids[i]]
+ * Pairs whose ids are consecutive on both sides travel as one extent; extents
+ * are spread over `threads` threads (<= 0: 8). Synchronous: returns when the
+ * data has been handed to the kernel (kvc_disk_sync forces it to the device).
+ * Ids are HOST int64 arrays, range-checked before any I/O. Destinations must be
+ * distinct. No GPU work; safe to call from any thread, one call per handle at a
+ * time for overlapping blocks.
+ */
+typedef struct kvc_disk kvc_disk;
+
+enum { KVC_DISK_DIRECT = 1 };
+enum {
+  KVC_DISK_INFO_DATA_OFFSET = 0, /* byte offset of block 0 in the file            */
+  KVC_DISK_INFO_DIRECT = 1,      /* 1 if an O_DIRECT descriptor is in use         */
+  KVC_DISK_INFO_CREATED = 2,     /* 1 if kvc_disk_open made a new file            */
+  KVC_DISK_INFO_ROW_BYTES = 3,   /* bytes of one block over all layers            */
+  KVC_DISK_INFO_NUM_BLOCKS = 4,
+  KVC_DISK_INFO_BOUNCED = 5      /* 1 if the last transfer staged the host side   */
+};
+
+int kvc_disk_open(const char* path, const char* descr, int64_t num_blocks, int64_t num_layers,
+                  int64_t block_elems, int elem_bytes, int flags, kvc_disk** out);
+int kvc_disk_close(kvc_disk* disk);
+int kvc_disk_sync(kvc_disk* disk);
+int64_t kvc_disk_info(const kvc_disk* disk, int what);
+int kvc_disk_save_blocks(kvc_disk* disk, const void* host_pool, int64_t num_host_blocks,
+                         const int64_t* src_host_ids, const int64_t* dst_disk_ids, int64_t n,
+                         int threads);
+int kvc_disk_load_blocks(kvc_disk* disk, void* host_pool, int64_t num_host_blocks,
+                         const int64_t* src_disk_ids, const int64_t* dst_host_ids, int64_t n,
+                         int threads);
 
 /* Pinned, device-addressable host memory for the host pool; replaces
  * pycuda.driver.pagelocked_empty (runtime/worker/llm_worker/kv_worker.py:123-127).

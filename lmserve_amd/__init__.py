@@ -5,14 +5,17 @@
     kv_worker   KVWorker (GPU <-> pinned host swap), Device, BlockMapping
     index_prep  host-side block-table / slot-mapping construction
     rotary      rotary position embedding, alone or fused with the K/V write
+    disk_tier   DiskTier (host <-> block file, native positional I/O)
     kv_pool     pool sizing, allocator id order, layer-sync handle and model-side hooks
 
 Every operator runs a hand-written HIP kernel from libkvcache.so through the
-C ABI of include/kvcache.h; nothing here computes on the CPU.
+C ABI of include/kvcache.h; the disk tier is host-side file I/O in the same
+library. Nothing here has a CPU fallback.
 """
 from . import _lib
 from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_block_maps,
                         gather_blocks, reshape_and_cache, reshape_and_cache_layers, scatter_blocks)
+from .disk_tier import DiskTier
 from .index_prep import (InferInput, KVIndexInputs, make_kv_index_inputs, to_device,
                          to_device_one_launch)
 from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
@@ -30,7 +33,7 @@ __all__ = [
     "append_paged_kv_cache", "append_paged_kv_cache_layers", "PagedKVWritePlan", "get_seq_lens",
     "get_batch_indices_positions",
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",
-    "flatten_block_mappings",
+    "flatten_block_mappings", "DiskTier",
     "RotaryEmbedding", "make_cos_sin_cache", "rotary_pos_emb", "rotary_pos_emb_and_cache",
     "rotary_pos_emb_and_append_paged",
     "BlockAllocator", "CachePlan", "KVWorkerHandle", "LayerSyncHooks", "allocate_kv_caches",

@@ -19,6 +19,15 @@ KVC_ERR_UNSUPPORTED = -2
 KVC_ERR_OUT_OF_RANGE = -3
 KVC_ERR_STAGING = -4
 KVC_ERR_HIP = -5
+KVC_ERR_IO = -6
+
+KVC_DISK_DIRECT = 1
+KVC_DISK_INFO_DATA_OFFSET = 0
+KVC_DISK_INFO_DIRECT = 1
+KVC_DISK_INFO_CREATED = 2
+KVC_DISK_INFO_ROW_BYTES = 3
+KVC_DISK_INFO_NUM_BLOCKS = 4
+KVC_DISK_INFO_BOUNCED = 5
 
 KVC_SWAP_STAGED = 0
 KVC_SWAP_DIRECT = 1
@@ -66,6 +75,12 @@ SIGNATURES = {
                              _I64, c_int, _P, _P]),
     "kvc_swap_in": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
                             _I64, c_int, _P, _P]),
+    "kvc_disk_open": (c_int, [c_char_p, c_char_p, _I64, _I64, _I64, c_int, c_int, ctypes.POINTER(_P)]),
+    "kvc_disk_close": (c_int, [_P]),
+    "kvc_disk_sync": (c_int, [_P]),
+    "kvc_disk_info": (_I64, [_P, c_int]),
+    "kvc_disk_save_blocks": (c_int, [_P, _P, _I64, _P, _P, _I64, c_int]),
+    "kvc_disk_load_blocks": (c_int, [_P, _P, _I64, _P, _P, _I64, c_int]),
     "kvc_host_alloc_pinned": (_P, [c_size_t]),
     "kvc_host_free_pinned": (c_int, [_P]),
 }
@@ -110,6 +125,8 @@ def check(rc: int) -> None:
         raise ValueError(msg)
     if rc == KVC_ERR_OUT_OF_RANGE:
         raise IndexError(msg)
+    if rc == KVC_ERR_IO:
+        raise OSError(msg)
     raise KVCacheLibraryError(msg)
 
 

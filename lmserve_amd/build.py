@@ -13,7 +13,8 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
 SOURCES = [os.path.join(PKG_DIR, "csrc", "kvcache.hip"),
-           os.path.join(PKG_DIR, "csrc", "rope_cache.hip")]
+           os.path.join(PKG_DIR, "csrc", "rope_cache.hip"),
+           os.path.join(PKG_DIR, "csrc", "disk_tier.cpp")]
 INCLUDE = os.path.join(REPO_ROOT, "include")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcache.so")
 

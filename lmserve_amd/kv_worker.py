@@ -27,6 +27,7 @@ import numpy as np
 import torch
 
 from . import _lib
+from .disk_tier import DiskTier
 
 
 class Device(enum.IntEnum):
@@ -130,6 +131,9 @@ class KVWorker:
       `post_events[l]` before touching layer l, a load records `pre_events[l]`
       and rings the model's doorbell after layer l. Without it the whole layer
       range moves in one call.
+    disk_direct_io / disk_threads: the disk tier bypasses the page cache when
+      alignment and the file system allow, and spreads block extents over this
+      many threads (the reference copies rows through a memory map on 4).
     """
 
     def __init__(
@@ -141,6 +145,8 @@ class KVWorker:
         swap_mode: str = "direct",
         staging_chunk_blocks: int = 0,
         kv_worker_handle=None,
+        disk_direct_io: bool = True,
+        disk_threads: int = 8,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -169,12 +175,17 @@ class KVWorker:
         self.host_kv_caches = self._host_pool.array
         self.host_kv_caches_tensor = torch.from_numpy(self.host_kv_caches)
 
+        # The block file of the disk tier (kv_worker.py:133-145). Transfers go through the
+        # native tier; `disk_kv_caches` stays available as a read-only map of the same file.
         if self.num_disk_blocks > 0:
             if not disk_kv_cache_file:
                 raise ValueError("disk_kv_cache_file is required when num_disk_blocks > 0")
-            self.disk_kv_caches = memmap_disk_kv_cache(
-                disk_kv_cache_file, (self.num_disk_blocks, num_layers, block_elems), np_dtype)
+            self.disk_tier = DiskTier(disk_kv_cache_file,
+                                      (self.num_disk_blocks, num_layers, block_elems), np_dtype,
+                                      direct=disk_direct_io, threads=disk_threads)
+            self.disk_kv_caches = self.disk_tier.memmap("r")
         else:
+            self.disk_tier = None
             self.disk_kv_caches = None
 
         with torch.cuda.device(self.device):
@@ -282,7 +293,7 @@ class KVWorker:
 
     # ----------------------------------------------------------------- disk legs
     def _require_disk(self) -> None:
-        if self.disk_kv_caches is None:
+        if self.disk_tier is None:
             raise ValueError("no disk KV cache configured (num_disk_blocks == 0)")
 
     def load_kv_blocks_from_disk_sync(self, block_mappings: Sequence[BlockMapping]) -> None:
@@ -291,8 +302,7 @@ class KVWorker:
             return
         self._require_disk()
         src, dst = flatten_block_mappings(block_mappings)
-        for s, d in zip(src.tolist(), dst.tolist()):
-            self.host_kv_caches[d] = self.disk_kv_caches[s]
+        self.disk_tier.load_blocks(self.host_kv_caches, src, dst)
 
     def save_kv_blocks_to_disk_sync(self, block_mappings: Sequence[BlockMapping]) -> None:
         """disk[dst] = host[src] for every layer (kv_worker.py:239-247)."""
@@ -300,8 +310,7 @@ class KVWorker:
             return
         self._require_disk()
         src, dst = flatten_block_mappings(block_mappings)
-        for s, d in zip(src.tolist(), dst.tolist()):
-            self.disk_kv_caches[d] = self.host_kv_caches[s]
+        self.disk_tier.save_blocks(self.host_kv_caches, src, dst)
 
     # ---------------------------------------------------------------- dispatcher
     async def _copy_kv_gpu_to_host(self, block_mappings):
@@ -343,5 +352,9 @@ class KVWorker:
             torch.cuda.synchronize()
         self.host_kv_caches_tensor = None
         self.host_kv_caches = None
+        self.disk_kv_caches = None
+        if self.disk_tier is not None:
+            self.disk_tier.close()
+            self.disk_tier = None
         self._host_pool.close()
         self._staging = {"out": None, "in": None}

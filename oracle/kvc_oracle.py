@@ -109,6 +109,17 @@ def load_blocks_from_host_np(gpu, host, src_ids, dst_ids, layer_begin=0, layer_e
     gpu[layer_begin:layer_end][:, dst] = host[src, layer_begin:layer_end].swapaxes(0, 1)
 
 
+def save_blocks_to_disk_np(host, disk, src_ids, dst_ids) -> None:
+    """kv_worker.py:239-247 over all layers (:311-322): disk[dst, l] = host[src, l];
+    host [nhb, L, E], disk [ndb, L, E]."""
+    disk[np.asarray(dst_ids, dtype=np.int64)] = host[np.asarray(src_ids, dtype=np.int64)]
+
+
+def load_blocks_from_disk_np(host, disk, src_ids, dst_ids) -> None:
+    """kv_worker.py:229-237 over all layers (:297-309): host[dst, l] = disk[src, l]."""
+    host[np.asarray(dst_ids, dtype=np.int64)] = disk[np.asarray(src_ids, dtype=np.int64)]
+
+
 # ----------------------------------------------------------------- pure-Python loops
 
 
@@ -164,6 +175,19 @@ def load_blocks_from_host_loops(gpu, host, src_ids, dst_ids) -> None:
         for s, d in zip(src_ids, dst_ids):
             for k in range(gpu.shape[2]):
                 gpu[l, int(d), k] = host[int(s), l, k]
+
+
+def save_blocks_to_disk_loops(host, disk, src_ids, dst_ids) -> None:
+    """The reference's own order: one pass per layer, one row per entry."""
+    for l in range(host.shape[1]):
+        for s, d in zip(src_ids, dst_ids):
+            disk[int(d)][l] = host[int(s)][l]
+
+
+def load_blocks_from_disk_loops(host, disk, src_ids, dst_ids) -> None:
+    for l in range(host.shape[1]):
+        for s, d in zip(src_ids, dst_ids):
+            host[int(d)][l] = disk[int(s)][l]
 
 
 # ----------------------------------------------------------------------- C via ctypes

@@ -162,7 +162,9 @@ def test_disk_tier_round_trip(gpu, tmp_path):
         w = kvc.KVWorker(dpool, nhb, num_disk_blocks=ndb, disk_kv_cache_file=path)
         w.copy_kv_sync([kvc.BlockMapping.from_pairs([(2, 0), (7, 3)])], kvc.Device.GPU, kvc.Device.Host)
         w.copy_kv_sync([kvc.BlockMapping.from_pairs([(0, 4), (3, 1)])], kvc.Device.Host, kvc.Device.Disk)
-        w.disk_kv_caches.flush()
+        w.disk_tier.sync()
+        # the pinned pool is mapped by the GPU driver: O_DIRECT cannot take it in place
+        assert w.disk_tier.last_transfer_staged == w.disk_tier.is_direct
         w.close()
         w = kvc.KVWorker(dpool, nhb, num_disk_blocks=ndb, disk_kv_cache_file=path)  # reopen
         w.copy_kv_sync([kvc.BlockMapping.from_pairs([(4, 5), (1, 2)])], kvc.Device.Disk, kvc.Device.Host)
