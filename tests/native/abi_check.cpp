@@ -1,8 +1,10 @@
 // Calls libkvcache through its C ABI from a plain HIP program (no Python, no
-// torch): every operator of the copy path on small seeded inputs, compared
-// byte for byte with the C oracle (oracle/kvc_oracle.c, linked in).
+// torch): every operator of the copy path, the one-launch index build and the
+// disk tier on small seeded inputs, compared byte for byte with the C oracle
+// (oracle/kvc_oracle.c, linked in) or with arrays written out by hand.
 // Exit status 0 and a final "ABI CHECK PASSED" line on success.
 #include <hip/hip_runtime.h>
+#include <unistd.h>
 
 #include <cstdint>
 #include <cstdio>
@@ -191,6 +193,105 @@ int main() {
     HIP_OK(hipStreamSynchronize(copy_stream));
     HIP_OK(hipStreamDestroy(copy_stream));
     HIP_OK(hipFree(staging));
+    KVC_OK_OR_DIE(kvc_host_free_pinned(host));
+  }
+
+  // 6. device gather and scatter: the pool's blocks <-> a dense [n, L, blk] buffer.
+  //    The dense buffer has the host pool's row layout, so the swap oracle applies.
+  {
+    std::vector<int64_t> ids = {41, 2, 17, 8}, dense_rows = {0, 1, 2, 3}, back = {20, 21, 22, 23};
+    const int64_t m = (int64_t)ids.size();
+    const size_t dense_bytes = (size_t)(m * L * blk_bytes);
+    void *d_ids, *d_back, *d_dense;
+    HIP_OK(hipMalloc(&d_ids, m * 8));
+    HIP_OK(hipMalloc(&d_back, m * 8));
+    HIP_OK(hipMalloc(&d_dense, dense_bytes));
+    HIP_OK(hipMemcpy(d_ids, ids.data(), m * 8, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_back, back.data(), m * 8, hipMemcpyHostToDevice));
+    HIP_OK(hipMemset(d_dense, 0, dense_bytes));
+    KVC_OK_OR_DIE(kvc_gather_blocks(d_pool, d_dense, (const int64_t*)d_ids, m, L, layer_elems * E, blk_bytes,
+                                    nb, 0, L, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<uint16_t> dense(dense_bytes / 2), want_dense(dense_bytes / 2, 0);
+    HIP_OK(hipMemcpy(dense.data(), d_dense, dense_bytes, hipMemcpyDeviceToHost));
+    oracle_save_blocks_to_host(want.data(), want_dense.data(), ids.data(), dense_rows.data(), m, L, nb,
+                               blk_bytes, 0, L);
+    expect_equal("kvc_gather_blocks == oracle", dense.data(), want_dense.data(), dense_bytes);
+    KVC_OK_OR_DIE(kvc_scatter_blocks(d_pool, d_dense, (const int64_t*)d_back, m, L, layer_elems * E,
+                                     blk_bytes, nb, 0, L, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    oracle_load_blocks_from_host(want.data(), want_dense.data(), dense_rows.data(), back.data(), m, L, nb,
+                                 blk_bytes, 0, L);
+    HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+    expect_equal("kvc_scatter_blocks == oracle", got.data(), want.data(), pool_bytes);
+    HIP_OK(hipFree(d_ids));
+    HIP_OK(hipFree(d_back));
+    HIP_OK(hipFree(d_dense));
+  }
+
+  // 7. the whole index of the step in one launch, against the arrays built by hand above
+  {
+    std::vector<int32_t> input_lens = {20, 1}, context_lens = {25, 34}, nblocks = {2, 3};
+    void *d_il, *d_cl, *d_nb, *d_cu, *d_ptr2, *d_last2, *d_bi2, *d_pos2, *d_slots2;
+    HIP_OK(hipMalloc(&d_il, 8)); HIP_OK(hipMalloc(&d_cl, 8)); HIP_OK(hipMalloc(&d_nb, 8));
+    HIP_OK(hipMalloc(&d_cu, 12)); HIP_OK(hipMalloc(&d_ptr2, 12)); HIP_OK(hipMalloc(&d_last2, 8));
+    HIP_OK(hipMalloc(&d_bi2, T * 4)); HIP_OK(hipMalloc(&d_pos2, T * 4)); HIP_OK(hipMalloc(&d_slots2, T * 8));
+    HIP_OK(hipMemcpy(d_il, input_lens.data(), 8, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_cl, context_lens.data(), 8, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_nb, nblocks.data(), 8, hipMemcpyHostToDevice));
+    KVC_OK_OR_DIE(kvc_build_write_index((const int32_t*)d_il, (const int32_t*)d_cl, (const int32_t*)d_nb,
+                                        (const int32_t*)d_ind, 2, 5, bs, T, (int32_t*)d_cu, (int32_t*)d_ptr2,
+                                        (int32_t*)d_last2, (int32_t*)d_bi2, (int32_t*)d_pos2,
+                                        (int64_t*)d_slots2, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<int32_t> g_ptr(3), g_last(2), g_bi(T), g_pos(T), g_cu(3);
+    std::vector<int64_t> g_slots(T);
+    HIP_OK(hipMemcpy(g_cu.data(), d_cu, 12, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_ptr.data(), d_ptr2, 12, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_last.data(), d_last2, 8, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_bi.data(), d_bi2, T * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_pos.data(), d_pos2, T * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_slots.data(), d_slots2, T * 8, hipMemcpyDeviceToHost));
+    const std::vector<int32_t> want_cu = {0, 20, 21};
+    expect_equal("kvc_build_write_index cu_seqlens_q", g_cu.data(), want_cu.data(), 12);
+    expect_equal("kvc_build_write_index kv_indptr", g_ptr.data(), kv_indptr.data(), 12);
+    expect_equal("kvc_build_write_index kv_last_page_len", g_last.data(), last.data(), 8);
+    expect_equal("kvc_build_write_index batch_indices", g_bi.data(), bi.data(), T * 4);
+    expect_equal("kvc_build_write_index positions", g_pos.data(), pos.data(), T * 4);
+    expect_equal("kvc_build_write_index slot_mapping", g_slots.data(), slots.data(), T * 8);
+    for (void* p : {d_il, d_cl, d_nb, d_cu, d_ptr2, d_last2, d_bi2, d_pos2, d_slots2}) HIP_OK(hipFree(p));
+  }
+
+  // 8. host <-> disk tier behind the pinned pool: disk[dst] = host[src] and back
+  {
+    const int64_t ndb = 5;
+    const size_t row_elems = (size_t)(L * blk_elems);
+    uint16_t* host = (uint16_t*)kvc_host_alloc_pinned(host_bytes);
+    if (!host) { std::fprintf(stderr, "pinned alloc failed: %s\n", kvc_last_error_string()); return 4; }
+    for (size_t i = 0; i < host_bytes / 2; ++i) host[i] = (uint16_t)rng();
+    std::vector<uint16_t> host0(host, host + host_bytes / 2);
+    char path[64];
+    std::snprintf(path, sizeof path, "/tmp/kvc-abi-check-%d.npy", (int)getpid());
+    kvc_disk* disk = nullptr;
+    KVC_OK_OR_DIE(kvc_disk_open(path, "<u2", ndb, L, blk_elems, 2, KVC_DISK_DIRECT, &disk));
+    std::vector<int64_t> s_host = {7, 1, 2}, s_disk = {4, 0, 1}, l_disk = {1, 4}, l_host = {9, 8};
+    KVC_OK_OR_DIE(kvc_disk_save_blocks(disk, host, nhb, s_host.data(), s_disk.data(), 3, 4));
+    KVC_OK_OR_DIE(kvc_disk_sync(disk));
+    KVC_OK_OR_DIE(kvc_disk_load_blocks(disk, host, nhb, l_disk.data(), l_host.data(), 2, 4));
+    std::vector<uint16_t> want_h(host0);
+    std::memcpy(&want_h[9 * row_elems], &host0[2 * row_elems], row_elems * 2);   // disk 1 holds host 2
+    std::memcpy(&want_h[8 * row_elems], &host0[7 * row_elems], row_elems * 2);   // disk 4 holds host 7
+    expect_equal("kvc_disk_save_blocks + kvc_disk_load_blocks round trip", host, want_h.data(), host_bytes);
+    std::printf("disk tier: O_DIRECT %s, host side %s\n",
+                kvc_disk_info(disk, KVC_DISK_INFO_DIRECT) ? "on" : "off",
+                kvc_disk_info(disk, KVC_DISK_INFO_BOUNCED) ? "staged" : "in place");
+    std::vector<int64_t> bad = {ndb};
+    if (kvc_disk_save_blocks(disk, host, nhb, s_host.data(), bad.data(), 1, 1) != KVC_ERR_OUT_OF_RANGE) {
+      std::fprintf(stderr, "expected KVC_ERR_OUT_OF_RANGE from the disk tier\n");
+      ++fails;
+    }
+    KVC_OK_OR_DIE(kvc_disk_close(disk));
+    std::remove(path);
     KVC_OK_OR_DIE(kvc_host_free_pinned(host));
   }
 
