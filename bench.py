@@ -441,7 +441,22 @@ def main():
                                                     idx.kv_block_indices, idx.kv_block_indptrs,
                                                     idx.kv_last_block_lens, return_key=False)
 
+        plans = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
+                                          ix.kv_block_indptrs, ix.kv_last_block_lens, cs, Hq, Hkv, D,
+                                          s8.block_size) for ix in idxs]
+        q_buf = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=dev)
+
+        def fused_plan(i):
+            r = i % R
+            for l in range(L):
+                plans[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
+
         n = max(R, args.steps // 8 // R * R)
+        for fn, label in ((fused, "rotary_pos_emb_and_append_paged (1 launch per layer)"),
+                          (fused_plan, "PagedRotaryWritePlan.run (1 launch per layer)")):
+            ms_w, ms_e = time_region(fn, n, 2, torch)
+            extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes, ms_w, ms_e,
+                               calls_per_step=L, launch="eager (Python + ctypes per call)"))
         for fn, label, extra_b in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
                                     2 * T * Hkv * D * E),   # rotated key written out and read back
                                    (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0)):

@@ -22,7 +22,7 @@ from .kv_pool import (BlockAllocator, CachePlan, KVWorkerHandle, LayerSyncHooks,
                       allocate_kv_caches, plan_cache)
 from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
                         flatten_block_mappings)
-from .rotary import (RotaryEmbedding, make_cos_sin_cache, rotary_pos_emb,
+from .rotary import (PagedRotaryWritePlan, RotaryEmbedding, make_cos_sin_cache, rotary_pos_emb,
                      rotary_pos_emb_and_append_paged, rotary_pos_emb_and_cache)
 from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cache_layers,
                     build_write_index, get_batch_indices_positions, get_seq_lens)
@@ -35,7 +35,7 @@ __all__ = [
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",
     "flatten_block_mappings", "DiskTier",
     "RotaryEmbedding", "make_cos_sin_cache", "rotary_pos_emb", "rotary_pos_emb_and_cache",
-    "rotary_pos_emb_and_append_paged",
+    "rotary_pos_emb_and_append_paged", "PagedRotaryWritePlan",
     "BlockAllocator", "CachePlan", "KVWorkerHandle", "LayerSyncHooks", "allocate_kv_caches",
     "plan_cache",
     "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device", "to_device_one_launch",

@@ -197,6 +197,105 @@ def rotary_pos_emb_and_append_paged(query: torch.Tensor, key: torch.Tensor, valu
     return q_out.view(query.shape), (k_out.view(key.shape) if return_key else None)
 
 
+class PagedRotaryWritePlan:
+    """`rotary_pos_emb_and_append_paged` with its per-step arguments checked ONCE.
+
+    The rotation and the append run once per layer with the same positions,
+    index tensors and cos/sin table (models/llama.py:156-167 and
+    models/layers/attention.py:76-85 inside the layer loop of llama.py:236-242).
+    A plan built per step (where the reference builds `InputParams`,
+    model_worker.py:435-446) leaves the layer loop with a handful of pointer
+    reads and the library call; `query_out` / `key_out` may be caller-owned
+    buffers reused across layers, so that nothing is allocated either.
+
+    The plan keeps references to its tensors for as long as it lives.
+    """
+
+    def __init__(self, batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len,
+                 cos_sin_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                 page_size: int):
+        for t, n in ((batch_indices, "batch_indices"), (positions, "positions"),
+                     (kv_indices, "kv_indices"), (kv_indptr, "kv_indptr"),
+                     (kv_last_page_len, "kv_last_page_len")):
+            _require_gpu(t, n)
+            if t.dtype != torch.int32 or not t.is_contiguous():
+                raise TypeError(f"{n} must be contiguous int32")
+        _require_gpu(cos_sin_cache, "cos_sin_cache")
+        self.kd = _DTYPES.get(cos_sin_cache.dtype)
+        if self.kd is None:
+            raise TypeError(f"Unsupported dtype: {cos_sin_cache.dtype}")
+        if cos_sin_cache.dim() != 2 or cos_sin_cache.shape[1] % 2 or not cos_sin_cache.is_contiguous():
+            raise ValueError("cos_sin_cache must be contiguous [max_position, 2*rotary_dim]")
+        if batch_indices.numel() != positions.numel():
+            raise ValueError("batch_indices and positions differ in length")
+        self._keep = (batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len, cos_sin_cache)
+        self.device, self.dtype = cos_sin_cache.device, cos_sin_cache.dtype
+        self.Hq, self.H, self.D, self.page_size = int(num_heads), int(num_kv_heads), int(head_dim), int(page_size)
+        self.nnz = positions.numel()
+        self.q_row, self.kv_row = self.Hq * self.D, self.H * self.D
+        self._fn = _lib.lib().kvc_rotary_pos_emb_and_append_paged
+        # [q, k, v, bi, pos, cs, max_pos, nnz, Hq, H, D, rd, q_stride, k_stride, v_stride, q_out, k_out,
+        #  qo_stride, ko_stride, cache, indices, indptr, B, n_idx, page_size, page_stride, num_pages,
+        #  dtype, stream]
+        self._args = [0, 0, 0, batch_indices.data_ptr(), positions.data_ptr(), cos_sin_cache.data_ptr(),
+                      cos_sin_cache.shape[0], self.nnz, self.Hq, self.H, self.D,
+                      cos_sin_cache.shape[1] // 2, 0, 0, 0, 0, None, self.q_row, self.kv_row, 0,
+                      kv_indices.data_ptr(), kv_indptr.data_ptr(), kv_indptr.numel() - 1,
+                      kv_indices.numel(), self.page_size, 0, 0, self.kd, 0]
+        self._cache_shape_tail = (2, self.page_size, self.H, self.D)
+
+    def _rows(self, t: torch.Tensor, width: int, name: str) -> int:
+        """Token stride (elements) of a `[nnz, width]` / `[nnz, heads, D]` tensor with dense rows."""
+        if t.dtype != self.dtype or t.device != self.device:
+            raise TypeError(f"{name} must have the plan's dtype and device")
+        if t.shape[0] != self.nnz or t.numel() != self.nnz * width:
+            raise ValueError(f"{name} must hold [nnz, {width}] elements")
+        if t.stride(-1) != 1 or (t.dim() == 3 and t.stride(1) != t.shape[2]):
+            raise ValueError(f"{name} rows must be dense")
+        return t.stride(0) if self.nnz > 1 else width
+
+    def run(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+            paged_kv_cache: torch.Tensor, query_out: torch.Tensor = None,
+            key_out: torch.Tensor = None, return_key: bool = False):
+        """One layer: rotates `query` and `key`, writes the rotated key and `value`
+        into the pages. Returns `(query_out, key_out)`; `key_out` is None unless a
+        buffer is given or `return_key` is set. Token-strided inputs (slices of a
+        fused QKV projection) are read in place."""
+        if query_out is None:
+            query_out = torch.empty((self.nnz, self.q_row), dtype=self.dtype, device=self.device)
+        if key_out is None and return_key:
+            key_out = torch.empty((self.nnz, self.kv_row), dtype=self.dtype, device=self.device)
+        if self.nnz == 0:
+            return query_out, key_out
+        if paged_kv_cache.dtype != self.dtype or paged_kv_cache.device != self.device:
+            raise TypeError("paged_kv_cache must have the plan's dtype and device")
+        if tuple(paged_kv_cache.shape[1:]) != self._cache_shape_tail or \
+                not _inner_contiguous(paged_kv_cache):
+            raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
+        num_pages = paged_kv_cache.shape[0]
+        a = self._args
+        a[12] = self._rows(query, self.q_row, "query")
+        a[13] = self._rows(key, self.kv_row, "key")
+        a[14] = self._rows(value, self.kv_row, "value")
+        a[17] = self._rows(query_out, self.q_row, "query_out")
+        a[0], a[1], a[2] = query.data_ptr(), key.data_ptr(), value.data_ptr()
+        a[15] = query_out.data_ptr()
+        if key_out is not None:
+            a[18] = self._rows(key_out, self.kv_row, "key_out")
+            a[16] = key_out.data_ptr()
+        else:
+            a[16] = None
+        if num_pages == 0:
+            raise ValueError("paged_kv_cache has no pages")
+        a[19] = paged_kv_cache.data_ptr()
+        a[25] = paged_kv_cache.stride(0) if num_pages > 1 else 2 * self.page_size * self.kv_row
+        a[26] = num_pages
+        a[28] = _stream_of(paged_kv_cache)
+        with _on_device_of(paged_kv_cache):
+            _lib.check(self._fn(*a))
+        return query_out, key_out
+
+
 class RotaryEmbedding(torch.nn.Module):
     """`RotaryEmbedding` of the reference (rotary_embedding.py:11-80): builds the
     cos/sin table from a HF-style config and rotates `(query, key)` in `forward`."""

@@ -164,6 +164,49 @@ def test_fused_paged_write_equals_rotation_then_append(gpu):
     assert int(torch.count_nonzero(pool_b.view(torch.int16))) > 0
 
 
+def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
+    """The per-step plan gives the same bits as the full wrapper, reading q/k/v in
+    place from one [T, (Hq + 2 Hkv) D] projection output and writing into buffers
+    the caller reuses across layers."""
+    s = wl.LLAMA_3_8B
+    rng = np.random.default_rng(19)
+    w = wl._write_workload(s, 128, [3, 40, 0, 17], [1, 9, 30, 1], rng)
+    idx = kvc.to_device(w.index, s.block_size, gpu)
+    T, Hq, Hkv, D = w.num_tokens, 32, s.num_kv_heads, s.head_dim
+    cs = rotary.make_cos_sin_cache(D, 1024, 500000.0, dtype=torch.bfloat16).to(gpu)
+    plan = kvc.PagedRotaryWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices,
+                                    idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D,
+                                    s.block_size)
+    q_buf = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=gpu)
+    k_buf = torch.empty(T, Hkv * D, dtype=torch.bfloat16, device=gpu)
+    g = torch.Generator().manual_seed(23)
+    for layer in range(3):
+        qkv = torch.randn(T, (Hq + 2 * Hkv) * D, generator=g).bfloat16().to(gpu)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)       # token-strided views
+        pool_a = torch.zeros(128, 2, s.block_size, Hkv, D, dtype=torch.bfloat16, device=gpu)
+        pool_b = torch.zeros_like(pool_a)
+        q_a, k_a = kvc.rotary_pos_emb_and_append_paged(q, k, v, idx.batch_indices, idx.positions, cs,
+                                                       D, pool_a, idx.kv_block_indices,
+                                                       idx.kv_block_indptrs, idx.kv_last_block_lens)
+        q_b, k_b = plan.run(q, k.view(T, Hkv, D), v, pool_b, query_out=q_buf, key_out=k_buf)
+        torch.cuda.synchronize()
+        assert q_b.data_ptr() == q_buf.data_ptr() and k_b.data_ptr() == k_buf.data_ptr()
+        assert torch.equal(q_a.view(T, -1), q_b) and torch.equal(k_a.view(T, -1), k_b), layer
+        assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16)), layer
+        q_c, k_c = plan.run(q, k, v, pool_b)                           # allocates q_out, no key_out
+        torch.cuda.synchronize()
+        assert k_c is None and torch.equal(q_c, q_b)
+    with pytest.raises(TypeError):
+        plan.run(q.float(), k, v, pool_b)
+    with pytest.raises(ValueError):
+        plan.run(q[:-1], k, v, pool_b)
+    with pytest.raises(ValueError):
+        plan.run(q, k, v, pool_b[:, :, :8])
+    with pytest.raises(TypeError):
+        kvc.PagedRotaryWritePlan(idx.batch_indices.long(), idx.positions, idx.kv_block_indices,
+                                 idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D, 16)
+
+
 def test_in_place_rotation_and_guards(gpu):
     T, Hq, Hkv, D = 20, 4, 2, 64
     q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, D, torch.bfloat16, max_pos=100)
