@@ -1,6 +1,7 @@
 """MI355X-native paged KV-cache data movement behind LMServe's operator surface.
 
-    cache_ops   copy_blocks, fill_key_cache, reshape_and_cache(_layers), gather/scatter_blocks
+    cache_ops   copy_blocks, fill_key_cache, reshape_and_cache(_layers), gather/scatter_blocks,
+                swap_out / swap_in (functional form of the GPU <-> host swap)
     paged       append_paged_kv_cache(_layers), get_seq_lens, get_batch_indices_positions
     kv_worker   KVWorker (GPU <-> pinned host swap), Device, BlockMapping
     index_prep  host-side block-table / slot-mapping construction
@@ -14,7 +15,8 @@ library. Nothing here has a CPU fallback.
 """
 from . import _lib
 from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_block_maps,
-                        gather_blocks, reshape_and_cache, reshape_and_cache_layers, scatter_blocks)
+                        gather_blocks, reshape_and_cache, reshape_and_cache_layers, scatter_blocks,
+                        swap_in, swap_out)
 from .disk_tier import DiskTier
 from .index_prep import (InferInput, KVIndexInputs, make_kv_index_inputs, to_device,
                          to_device_one_launch)
@@ -30,6 +32,7 @@ from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cac
 __all__ = [
     "copy_blocks", "fill_key_cache", "reshape_and_cache", "reshape_and_cache_layers",
     "flatten_block_maps", "check_block_maps", "gather_blocks", "scatter_blocks",
+    "swap_out", "swap_in",
     "append_paged_kv_cache", "append_paged_kv_cache_layers", "PagedKVWritePlan", "get_seq_lens",
     "get_batch_indices_positions",
     "KVWorker", "Device", "BlockMapping", "BlockMappingEntry", "PinnedHostPool",

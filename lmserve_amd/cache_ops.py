@@ -336,3 +336,56 @@ def scatter_blocks(kv_caches: torch.Tensor, block_ids: torch.Tensor, buffer: tor
         _lib.check(_lib.lib().kvc_scatter_blocks(
             kv_caches.data_ptr(), buffer.data_ptr(), block_ids.data_ptr(), n, L, layer_stride,
             block_bytes, nb, layer_begin, layer_end, _stream_of(kv_caches)))
+
+
+def _host_ids(ids, name: str):
+    import numpy as np
+
+    if isinstance(ids, torch.Tensor):
+        if ids.is_cuda:
+            raise ValueError(f"{name} must be host-resident (they are range-checked before the launch)")
+        ids = ids.numpy()
+    return np.ascontiguousarray(np.asarray(ids, dtype=np.int64).reshape(-1))
+
+
+def _swap_direct(out: bool, kv_caches: torch.Tensor, host_pool: torch.Tensor, src_ids, dst_ids,
+                 layer_begin: int, layer_end) -> None:
+    L, nb, block_elems, block_bytes, layer_stride = _pool_geometry(kv_caches)
+    if host_pool.is_cuda or not host_pool.is_pinned():
+        raise ValueError("host_pool must be a pinned host tensor (the kernel addresses it over PCIe)")
+    if host_pool.dtype.itemsize != kv_caches.dtype.itemsize or not host_pool.is_contiguous() \
+            or host_pool.dim() != 3 or host_pool.shape[1] != L or host_pool.shape[2] != block_elems:
+        raise ValueError("host_pool must be a contiguous [num_host_blocks, L, block_elems] tensor "
+                         "with the pool's element width")
+    src, dst = _host_ids(src_ids, "src_ids"), _host_ids(dst_ids, "dst_ids")
+    if src.shape != dst.shape:
+        raise ValueError("source and destination id lists differ in length")
+    n = int(src.shape[0])
+    layer_end = L if layer_end is None else layer_end
+    if n == 0 or layer_end <= layer_begin:
+        return
+    lib = _lib.lib()
+    need = lib.kvc_swap_staging_bytes(n, layer_end - layer_begin, block_bytes, _lib.KVC_SWAP_DIRECT, 0)
+    with _on_device_of(kv_caches):
+        ids_dev = torch.empty(int(need), dtype=torch.uint8, device=kv_caches.device)
+        stream = _stream_of(kv_caches)
+        fn = lib.kvc_swap_out if out else lib.kvc_swap_in
+        _lib.check(fn(kv_caches.data_ptr(), host_pool.data_ptr(), src.ctypes.data, dst.ctypes.data, n,
+                      L, layer_stride, block_bytes, nb, host_pool.shape[0], layer_begin, layer_end,
+                      ids_dev.data_ptr(), ids_dev.numel(), _lib.KVC_SWAP_DIRECT, stream, stream))
+
+
+def swap_out(kv_caches: torch.Tensor, host_pool: torch.Tensor, src_ids, dst_ids,
+             layer_begin: int = 0, layer_end: int = None) -> None:
+    """`host_pool[dst_ids[i], l] = kv_caches[l, src_ids[i]]` on the current stream
+    (kv_worker.py:213-227 for every layer of the range): one kernel that stores
+    into the pinned host pool. Asynchronous; the ids are host-resident lists,
+    int64 tensors or arrays."""
+    _swap_direct(True, kv_caches, host_pool, src_ids, dst_ids, layer_begin, layer_end)
+
+
+def swap_in(kv_caches: torch.Tensor, host_pool: torch.Tensor, src_ids, dst_ids,
+            layer_begin: int = 0, layer_end: int = None) -> None:
+    """`kv_caches[l, dst_ids[i]] = host_pool[src_ids[i], l]` on the current stream
+    (kv_worker.py:197-211 for every layer of the range)."""
+    _swap_direct(False, kv_caches, host_pool, src_ids, dst_ids, layer_begin, layer_end)

@@ -238,3 +238,36 @@ def test_dispatcher_registered_ops_run_the_same_kernels(gpu):
     torch.ops.kvcache.copy_blocks(dpool, torch.from_numpy(flat).to(gpu))
     torch.cuda.synchronize()
     assert np.array_equal(bits_of(dpool), want)
+
+    # swap through the functional operators: a torch-pinned host pool and one from the library
+    old, host_ids, new = wl.swap_round_trip(nb, 10, seed=4)
+    block_elems = 2 * bs * s.num_kv_heads * s.head_dim
+    lib_pool = kvc.PinnedHostPool((12, 2, block_elems), np.uint16)
+    try:
+        for host_t in (torch.zeros(12, 2, block_elems, dtype=torch.int16).pin_memory(),
+                       torch.from_numpy(lib_pool.array.view(np.int16))):
+            host_t.zero_()
+            dpool2 = to_bf16(want, gpu)
+            want_host = np.zeros((12, 2, block_elems), dtype=np.uint16)
+            gpu_np = want.reshape(2, nb, -1).copy()
+            orc.c_save_blocks_to_host(gpu_np, want_host, old, host_ids)
+            orc.c_load_blocks_from_host(gpu_np, want_host, host_ids, new)
+            torch.ops.kvcache.swap_out(dpool2, host_t, torch.from_numpy(old), torch.from_numpy(host_ids))
+            torch.ops.kvcache.swap_in(dpool2, host_t, torch.from_numpy(host_ids), torch.from_numpy(new))
+            torch.cuda.synchronize()
+            assert np.array_equal(host_t.numpy().view(np.uint16), want_host)
+            assert np.array_equal(bits_of(dpool2).reshape(2, nb, -1), gpu_np)
+        # a layer range, lists as ids, and the guards
+        host_t.zero_()
+        kvc.swap_out(dpool2, host_t, old.tolist(), host_ids.tolist(), layer_begin=1)
+        torch.cuda.synchronize()
+        assert not host_t[:, 0].any() and np.array_equal(host_t.numpy().view(np.uint16)[:, 1], want_host[:, 1])
+        with pytest.raises(IndexError):
+            kvc.swap_out(dpool2, host_t, [0], [12])
+        with pytest.raises(ValueError):
+            kvc.swap_in(dpool2, torch.zeros(12, 2, block_elems, dtype=torch.int16), [0], [0])   # pageable
+        with pytest.raises(ValueError):
+            kvc.swap_in(dpool2, host_t, torch.tensor([0], device=gpu), [0])
+        del host_t
+    finally:
+        lib_pool.close()
