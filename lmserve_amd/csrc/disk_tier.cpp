@@ -26,6 +26,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <string>
 #include <thread>
 #include <vector>
@@ -48,8 +49,9 @@ struct kvc_disk {
   // Host pool whose pages O_DIRECT could not take in place (EFAULT): memory the
   // GPU driver maps for pinning is such memory. Its transfers go through an
   // aligned bounce buffer per thread from then on.
-  const void* bounce_pool = nullptr;
-  bool last_bounced = false;
+  // Atomics: save and load calls may run on one handle from two threads.
+  std::atomic<const void*> bounce_pool{nullptr};
+  std::atomic<bool> last_bounced{false};
   std::string path;
 };
 
@@ -216,7 +218,7 @@ int run_io(const char* fn, kvc_disk* d, bool to_disk, char* host_pool, int64_t n
   // in place when it is aligned and the kernel can pin its pages, else staged.
   const bool direct = d->fd_direct >= 0 && d->aligned;
   const bool in_place = direct && (reinterpret_cast<uintptr_t>(host_pool) % kAlign) == 0 &&
-                        d->bounce_pool != host_pool;
+                        d->bounce_pool.load(std::memory_order_relaxed) != host_pool;
   const int fd = direct ? d->fd_direct : d->fd;
   const int nthreads = (int)std::max<int64_t>(1, std::min<int64_t>({(int64_t)(threads > 0 ? threads : 8),
                                                                    (int64_t)ext.size(), 64}));
@@ -259,8 +261,8 @@ int run_io(const char* fn, kvc_disk* d, bool to_disk, char* host_pool, int64_t n
     work();
     for (auto& t : pool) t.join();
   }
-  if (faulted.load()) d->bounce_pool = host_pool;
-  d->last_bounced = direct && !(in_place && !faulted.load());
+  if (faulted.load()) d->bounce_pool.store(host_pool, std::memory_order_relaxed);
+  d->last_bounced.store(direct && !(in_place && !faulted.load()), std::memory_order_relaxed);
   if (const int err = first_errno.load())
     return fail(KVC_ERR_IO, "%s: %s of %s failed: %s", fn, to_disk ? "write" : "read", d->path.c_str(),
                 strerror(err));
@@ -283,7 +285,8 @@ int kvc_disk_open(const char* path, const char* descr, int64_t num_blocks, int64
   const int64_t row_bytes = num_layers * block_elems * elem_bytes;
   const int64_t payload = num_blocks * row_bytes;
 
-  kvc_disk d;
+  std::unique_ptr<kvc_disk> holder(new kvc_disk);
+  kvc_disk& d = *holder;
   d.path = path;
   d.num_blocks = num_blocks;
   d.row_bytes = row_bytes;
@@ -326,7 +329,7 @@ int kvc_disk_open(const char* path, const char* descr, int64_t num_blocks, int64
   }
   d.aligned = d.data_offset % kAlign == 0 && row_bytes % kAlign == 0;
   if ((flags & KVC_DISK_DIRECT) && d.aligned) d.fd_direct = open(path, O_RDWR | O_DIRECT | O_CLOEXEC);
-  *out = new kvc_disk(d);
+  *out = holder.release();
   return KVC_OK;
 }
 
@@ -353,7 +356,7 @@ int64_t kvc_disk_info(const kvc_disk* d, int what) {
     case KVC_DISK_INFO_CREATED: return d->created ? 1 : 0;
     case KVC_DISK_INFO_ROW_BYTES: return d->row_bytes;
     case KVC_DISK_INFO_NUM_BLOCKS: return d->num_blocks;
-    case KVC_DISK_INFO_BOUNCED: return d->last_bounced ? 1 : 0;
+    case KVC_DISK_INFO_BOUNCED: return d->last_bounced.load(std::memory_order_relaxed) ? 1 : 0;
     default: return -1;
   }
 }

@@ -145,6 +145,42 @@ def test_long_runs_are_split_across_threads(tmp_path):
     assert np.array_equal(back[::-1], host)
 
 
+def test_save_and_load_may_run_concurrently_on_disjoint_blocks(tmp_path):
+    """The KV worker's dispatcher can have a Host->Disk and a Disk->Host copy in
+    flight at once (both legs run in threads)."""
+    import threading
+    rng = np.random.default_rng(11)
+    host = _aligned((32, 2, 8192), np.uint16)
+    _fill(host, rng)
+    with DiskTier(str(tmp_path / "c.npy"), (32, 2, 8192), np.uint16, threads=4) as d:
+        d.save_blocks(host, np.arange(16), np.arange(16))              # disk 0..15 = host 0..15
+        want = host.copy()
+        want[16:24] = host[0:8]
+        errors = []
+
+        def saver():
+            try:
+                for _ in range(10):
+                    d.save_blocks(host, np.arange(24, 32), np.arange(16, 24))   # disk 16..23 = host 24..31
+            except Exception as exc:   # pragma: no cover
+                errors.append(exc)
+
+        def loader():
+            try:
+                for _ in range(10):
+                    d.load_blocks(host, np.arange(0, 8), np.arange(16, 24))     # host 16..23 = disk 0..7
+            except Exception as exc:   # pragma: no cover
+                errors.append(exc)
+
+        ts = [threading.Thread(target=saver), threading.Thread(target=loader)]
+        [t.start() for t in ts]
+        [t.join() for t in ts]
+        assert not errors
+        assert np.array_equal(host, want)
+    disk = np.load(str(tmp_path / "c.npy"), mmap_mode="r")
+    assert np.array_equal(disk[16:24], want[24:32]) and np.array_equal(disk[:16], want[:16])
+
+
 def test_a_numpy_made_file_is_reused_in_place(tmp_path):
     """The reference creates the file with np.lib.format.open_memmap (kv_worker.py:78-82):
     data starts at byte 128 there, so the tier uses buffered I/O on it."""
