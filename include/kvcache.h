@@ -117,8 +117,9 @@ int kvc_reshape_and_cache_layers(const void* key, const void* value,
  * Index arrays are int32 on the device. kv_last_page_len is accepted for
  * signature parity and not read (flashinfer does not read it either).
  * page_stride is the distance between pages in elements (2*page_size*H*D when
- * contiguous). b outside [0, batch_size), a page-table index outside
- * [0, num_kv_indices) or a page outside [0, num_pages) skips the token.
+ * contiguous). b outside [0, batch_size), a page-table index outside the
+ * request's own table [kv_indptr[b], kv_indptr[b+1]) or outside
+ * [0, num_kv_indices), or a page outside [0, num_pages) skips the token.
  * The _layers form adds the layer loop exactly as kvc_reshape_and_cache_layers.
  * ------------------------------------------------------------------------- */
 int kvc_append_paged_kv_cache(const void* append_key, const void* append_value,

@@ -189,8 +189,9 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
       pg = p / a.block_size;
       off = p - pg * a.block_size;
     }
+    // the page must lie inside this request's own table (and inside the array)
     const int64_t it = (int64_t)a.kv_indptr[b] + pg;
-    if (it < 0 || it >= a.num_kv_indices) return;
+    if (it < 0 || it >= (int64_t)a.kv_indptr[b + 1] || it >= a.num_kv_indices) return;
     blk = a.kv_indices[it];
   } else {
     const int64_t s = (a.slot_bytes == 8)

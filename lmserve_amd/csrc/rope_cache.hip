@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
         const int64_t pg = a.bs_shift >= 0 ? (pos >> a.bs_shift) : pos / a.block_size;
         off = pos - pg * a.block_size;
         const int64_t it = (int64_t)a.kv_indptr[b] + pg;
-        if (it >= 0 && it < a.num_kv_indices) blk = a.kv_indices[it];
+        if (it >= 0 && it < (int64_t)a.kv_indptr[b + 1] && it < a.num_kv_indices) blk = a.kv_indices[it];
       }
     } else {
       const int64_t s = a.slot_bytes == 8 ? reinterpret_cast<const int64_t*>(a.slot_mapping)[t]

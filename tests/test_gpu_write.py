@@ -231,7 +231,11 @@ def test_append_paged_skips_tokens_with_bad_indices(gpu):
     bi[2] = -1          # no such request
     bi[5] = 8           # beyond the batch
     pos[6] = 1 << 20    # beyond the page table
-    keep = np.asarray([0, 1, 3, 4, 7])
+    # beyond its own request's table, yet inside the array: would land in the next request's page
+    own_pages = int(idx.kv_block_indptrs[bi[4] + 1] - idx.kv_block_indptrs[bi[4]])
+    assert bi[4] + 1 < 8
+    pos[4] = own_pages * bs + 3
+    keep = np.asarray([0, 1, 3, 7])
     want = pool.copy()
     orc.c_append_paged_kv_cache(np.ascontiguousarray(key[keep]), np.ascontiguousarray(value[keep]),
                                 bi[keep], pos[keep], want, idx.kv_block_indices,
