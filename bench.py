@@ -500,6 +500,47 @@ def main():
                                    max(ROTATE_PREFILL, args.steps // 2), max(3, args.warmup // 2),
                                    ["fused_slot:graph", "fused_paged:graph", "per_layer_paged:graph"])
         extra += e3
+        if "rope" in ops:
+            # rotation + write per layer at the prefill chunk (28 query heads, 4 KV heads x 128)
+            Hq3, Hkv3, D3 = 28, sq.num_kv_heads, sq.head_dim
+            T3 = sets3[0][0].num_tokens
+            R3 = len(sets3)
+            cs3 = kvc.make_cos_sin_cache(D3, 65536, 1000000.0, dtype=torch.bfloat16).to(dev)
+            q3 = [torch.randn(T3, Hq3 * D3, device=dev).to(torch.bfloat16) for _ in range(R3)]
+            k3 = [sets3[r][1][0].reshape(T3, Hkv3 * D3) for r in range(R3)]
+            v3 = [sets3[r][2][0].reshape(T3, Hkv3 * D3) for r in range(R3)]
+            plans3 = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
+                                               ix.kv_block_indptrs, ix.kv_last_block_lens, cs3, Hq3,
+                                               Hkv3, D3, sq.block_size) for _, _, _, ix in sets3]
+            qo3 = torch.empty(T3, Hq3 * D3, dtype=torch.bfloat16, device=dev)
+            pool3_l = [pool3[l] for l in range(L3)]
+            bytes3 = T3 * (2 * Hq3 * D3 * 2 + 4 * Hkv3 * D3 * 2 + 2 * D3 * 2 + 12)
+
+            def fused3(i):
+                r = i % R3
+                for l in range(L3):
+                    plans3[r].run(q3[r], k3[r], v3[r], pool3_l[l], query_out=qo3)
+
+            def two3(i):
+                r = i % R3
+                ix = sets3[r][3]
+                for l in range(L3):
+                    q_o, k_o = kvc.rotary_pos_emb(q3[r], k3[r], ix.positions, cs3, D3)
+                    kvc.append_paged_kv_cache(k_o, v3[r], ix.batch_indices, ix.positions, pool3_l[l],
+                                              ix.kv_block_indices, ix.kv_block_indptrs,
+                                              ix.kv_last_block_lens)
+
+            for fn, label, extra_b in ((two3, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
+                                        2 * T3 * Hkv3 * D3 * 2),
+                                       (fused3, "PagedRotaryWritePlan.run (1 launch per layer)", 0)):
+                try:
+                    ms_w, ms_e = time_region(fn, R3, 1, torch, graph_of=R3)
+                except Exception as exc:
+                    log(f"prefill rope variant skipped: {exc!r}")
+                    continue
+                extra.append(entry(f"cfg3 chunked prefill + rotation/{label}", bytes3 + extra_b, ms_w, ms_e,
+                                   calls_per_step=L3, launch="hipGraph replay"))
+            del q3, k3, v3, plans3, qo3
         del sets3, pool3
         torch.cuda.empty_cache()
 

@@ -20,6 +20,13 @@ inline int log2_exact(int64_t x) {
   return s;
 }
 
+// Launch shape of the rotation kernel, set through kvc_set_tuning
+// ("rope_threads": 64/128/256 lanes per workgroup, 0 = by size).
+struct RopeTuning {
+  int threads = 0;
+};
+extern RopeTuning g_rope_tune;
+
 }  // namespace kvc
 
 #define KVC_HIP(call)                                                          \

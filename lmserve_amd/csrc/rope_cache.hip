@@ -21,6 +21,10 @@
 #include "common.h"
 #include "kvcache.h"
 
+namespace kvc {
+RopeTuning g_rope_tune;
+}
+
 namespace {
 
 using kvc::fail;
@@ -35,17 +39,25 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 struct BF16 {
   static constexpr int kBytes = 2;
   static __device__ __forceinline__ float load(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+  // Round to nearest, ties to even, through the native conversion: gfx950 has a
+  // packed f32 -> bf16 convert instruction, which the compiler selects for this.
   static __device__ __forceinline__ uint16_t store(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest, ties to even
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+  }
+  static __device__ __forceinline__ uint32_t store2(float lo, float hi) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
   }
 };
 struct F16 {
   static constexpr int kBytes = 2;
   static __device__ __forceinline__ float load(uint16_t b) { return __half2float(__ushort_as_half(b)); }
   static __device__ __forceinline__ uint16_t store(float f) { return __half_as_ushort(__float2half_rn(f)); }
+  static __device__ __forceinline__ uint32_t store2(float lo, float hi) {
+    return (uint32_t)store(lo) | ((uint32_t)store(hi) << 16);
+  }
 };
 struct F32 {
   static constexpr int kBytes = 4;
@@ -66,7 +78,7 @@ struct Vec {
     u32x4 v;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      v[i] = (uint32_t)T::store(in[2 * i]) | ((uint32_t)T::store(in[2 * i + 1]) << 16);
+      v[i] = T::store2(in[2 * i], in[2 * i + 1]);
     return v;
   }
   static __device__ __forceinline__ float load1(const char* p) { return T::load(*(const uint16_t*)p); }
@@ -116,14 +128,18 @@ struct RopeArgs {
   int64_t cache_block_stride, cache_slot_stride;  // bytes
   int64_t num_cache_blocks;
   uint32_t groups_per_token;  // workgroups per token
+  int pv_shift;               // log2(pair-vectors per head) or -1
+  int cs_vector;              // cos/sin rows are 16-byte aligned runs of whole vectors
 };
 
 // Work items of one token, in this order: rotation pair-vectors of the Q heads
 // then the K heads, pass-through vectors beyond rotary_dim, V vectors. A
-// workgroup takes blockDim.x consecutive items of one token, one per lane: the
-// lane's global loads are issued first, the cos/sin row is staged in LDS while
-// they are in flight, then the lane computes and stores.
-template <typename T, bool VECTOR>
+// workgroup takes IPL * blockDim.x consecutive items of one token, IPL per lane
+// (item = first + j * blockDim.x, so the lanes of a wavefront stay on
+// consecutive vectors): all of the lane's global loads are issued first, the
+// cos/sin row is staged in LDS while they are in flight, then the lane computes
+// and stores.
+template <typename T, bool VECTOR, int IPL>
 __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
   using VT = Vec<T>;
   constexpr int EV = VECTOR ? VT::kElems : 1;
@@ -145,56 +161,71 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
   const uint32_t tail_items = heads * tail_per_head;
   const uint32_t v_items = a.key_cache ? a.num_kv_heads * D / EV : 0;
 
-  // ---- this lane's item and its loads ----
-  const uint32_t item = group * blockDim.x + threadIdx.x;
-  enum { kNone, kRotate, kTail, kValue } kind = kNone;
-  bool is_k = false;
-  uint32_t e0 = 0;          // first lane inside the head (rotation / tail)
-  int64_t in_off = 0;       // byte offset of the item inside its source row == inside its out row
-  float x[EV], y[EV];
-  u32x4 raw = {0, 0, 0, 0};
-  float raw1 = 0.f;
-  if (item < rot_items) {
-    kind = kRotate;
-    const uint32_t h = item / pv_per_head;
-    e0 = (item - h * pv_per_head) * EV;
-    is_k = h >= a.num_heads;
-    const uint32_t hh = is_k ? h - a.num_heads : h;
-    in_off = (int64_t)hh * D * E;
-    const char* in = (is_k ? a.key + (int64_t)t * a.k_token_stride
-                           : a.query + (int64_t)t * a.q_token_stride) + in_off;
-    if constexpr (VECTOR) {
-      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)e0 * E), x);
-      VT::unpack(*reinterpret_cast<const u32x4*>(in + (int64_t)(half + e0) * E), y);
-    } else {
-      x[0] = VT::load1(in + (int64_t)e0 * E);
-      y[0] = VT::load1(in + (int64_t)(half + e0) * E);
+  // ---- this lane's items and their loads ----
+  enum : int { kNone, kRotate, kTail, kValue };
+  int kind[IPL];
+  bool is_k[IPL];
+  uint32_t e0[IPL];     // first lane inside the head (rotation / tail)
+  int64_t in_off[IPL];  // byte offset of the item inside its source row == inside its out row
+  u32x4 rx[IPL], ry[IPL];  // 16-byte path: x half and y half (or the one pass-through vector)
+  float sx[IPL], sy[IPL];  // element path
+  const uint32_t first = group * (IPL * blockDim.x) + threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < IPL; ++j) {
+    const uint32_t item = first + j * blockDim.x;
+    kind[j] = kNone;
+    is_k[j] = false;
+    e0[j] = 0;
+    in_off[j] = 0;
+    sx[j] = sy[j] = 0.f;
+    if (item < rot_items) {
+      kind[j] = kRotate;
+      const uint32_t h = a.pv_shift >= 0 ? item >> a.pv_shift : item / pv_per_head;
+      e0[j] = (item - h * pv_per_head) * EV;
+      is_k[j] = h >= a.num_heads;
+      const uint32_t hh = is_k[j] ? h - a.num_heads : h;
+      in_off[j] = (int64_t)hh * D * E;
+      const char* in = (is_k[j] ? a.key + (int64_t)t * a.k_token_stride
+                                : a.query + (int64_t)t * a.q_token_stride) + in_off[j];
+      if constexpr (VECTOR) {
+        rx[j] = *reinterpret_cast<const u32x4*>(in + (int64_t)e0[j] * E);
+        ry[j] = *reinterpret_cast<const u32x4*>(in + (int64_t)(half + e0[j]) * E);
+      } else {
+        sx[j] = VT::load1(in + (int64_t)e0[j] * E);
+        sy[j] = VT::load1(in + (int64_t)(half + e0[j]) * E);
+      }
+    } else if (item < rot_items + tail_items) {
+      kind[j] = kTail;
+      const uint32_t it = item - rot_items;
+      const uint32_t h = it / tail_per_head;
+      e0[j] = rd + (it - h * tail_per_head) * EV;
+      is_k[j] = h >= a.num_heads;
+      const uint32_t hh = is_k[j] ? h - a.num_heads : h;
+      in_off[j] = ((int64_t)hh * D + e0[j]) * E;
+      const char* in = (is_k[j] ? a.key + (int64_t)t * a.k_token_stride
+                                : a.query + (int64_t)t * a.q_token_stride) + in_off[j];
+      if constexpr (VECTOR) rx[j] = *reinterpret_cast<const u32x4*>(in);
+      else sx[j] = VT::load1(in);
+    } else if (item < rot_items + tail_items + v_items) {
+      kind[j] = kValue;
+      in_off[j] = (int64_t)(item - rot_items - tail_items) * EV * E;
+      const char* in = a.value + (int64_t)t * a.v_token_stride + in_off[j];
+      if constexpr (VECTOR) rx[j] = *reinterpret_cast<const u32x4*>(in);
+      else sx[j] = VT::load1(in);
     }
-  } else if (item < rot_items + tail_items) {
-    kind = kTail;
-    const uint32_t it = item - rot_items;
-    const uint32_t h = it / tail_per_head;
-    e0 = rd + (it - h * tail_per_head) * EV;
-    is_k = h >= a.num_heads;
-    const uint32_t hh = is_k ? h - a.num_heads : h;
-    in_off = ((int64_t)hh * D + e0) * E;
-    const char* in = (is_k ? a.key + (int64_t)t * a.k_token_stride
-                           : a.query + (int64_t)t * a.q_token_stride) + in_off;
-    if constexpr (VECTOR) raw = *reinterpret_cast<const u32x4*>(in);
-    else raw1 = VT::load1(in);
-  } else if (item < rot_items + tail_items + v_items) {
-    kind = kValue;
-    in_off = (int64_t)(item - rot_items - tail_items) * EV * E;
-    const char* in = a.value + (int64_t)t * a.v_token_stride + in_off;
-    if constexpr (VECTOR) raw = *reinterpret_cast<const u32x4*>(in);
-    else raw1 = VT::load1(in);
   }
 
-  // ---- cos/sin row of this position into LDS (fp32), shared by all heads ----
+  // ---- cos/sin row of this position: issue the loads (first vector of each lane) ----
   const char* cs_row = a.cos_sin_cache + pos * (int64_t)(2 * rd) * E;
-  for (uint32_t i = threadIdx.x; i < 2 * rd; i += blockDim.x) cs[i] = VT::load1(cs_row + (int64_t)i * E);
+  constexpr int CV = VT::kElems;  // whole 16-byte vectors when the row is aligned and a multiple of them
+  const uint32_t cs_vecs = 2 * rd / CV;
+  u32x4 cs_first = {0, 0, 0, 0};
+  if (a.cs_vector && threadIdx.x < cs_vecs)
+    cs_first = *reinterpret_cast<const u32x4*>(cs_row + (int64_t)threadIdx.x * 16);
 
   // ---- slot of this token (workgroup-uniform) ----
+  // Placed after every vector load has been issued and before the first wait on
+  // them: the chain of dependent scalar loads runs while they are in flight.
   char* kc_row = nullptr;
   char* vc_row = nullptr;
   if (a.key_cache) {
@@ -221,54 +252,92 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
       vc_row = a.value_cache + slot_off;
     }
   }
+  // ---- cos/sin row into LDS as fp32, shared by all heads ----
+  if (a.cs_vector) {
+    for (uint32_t i = threadIdx.x; i < cs_vecs; i += blockDim.x) {
+      float f[CV];
+      VT::unpack(i == threadIdx.x ? cs_first : *reinterpret_cast<const u32x4*>(cs_row + (int64_t)i * 16), f);
+#pragma unroll
+      for (int e = 0; e < CV; ++e) cs[i * CV + e] = f[e];
+    }
+  } else {
+    for (uint32_t i = threadIdx.x; i < 2 * rd; i += blockDim.x) cs[i] = VT::load1(cs_row + (int64_t)i * E);
+  }
   __syncthreads();
 
   // ---- compute and store ----
   char* qo_row = a.query_out + (int64_t)t * a.qo_token_stride;
   char* ko_row = a.key_out ? a.key_out + (int64_t)t * a.ko_token_stride : nullptr;
-  char* outs[2] = {is_k ? ko_row : qo_row, is_k ? kc_row : nullptr};
-  if (kind == kRotate) {
-    float ox[EV], oy[EV];
 #pragma unroll
-    for (int i = 0; i < EV; ++i) {
-      const float cos_x = cs[e0 + i], cos_y = cs[half + e0 + i];
-      const float sin_x = cs[rd + e0 + i], sin_y = cs[rd + half + e0 + i];
-      ox[i] = x[i] * cos_x - y[i] * sin_x;
-      oy[i] = y[i] * cos_y + x[i] * sin_y;
-    }
-#pragma unroll
-    for (int o = 0; o < 2; ++o) {
-      if (!outs[o]) continue;
-      char* out = outs[o] + in_off;
+  for (int j = 0; j < IPL; ++j) {
+    // outs[0]: the rotated tensor handed back (read again by attention right away);
+    // outs[1]: the cache row of a K item (not read again by this step: non-temporal)
+    char* outs[2] = {is_k[j] ? ko_row : qo_row, is_k[j] ? kc_row : nullptr};
+    if (kind[j] == kRotate) {
+      float x[EV], y[EV], ox[EV], oy[EV];
       if constexpr (VECTOR) {
-        *reinterpret_cast<u32x4*>(out + (int64_t)e0 * E) = VT::pack(ox);
-        *reinterpret_cast<u32x4*>(out + (int64_t)(half + e0) * E) = VT::pack(oy);
+        VT::unpack(rx[j], x);
+        VT::unpack(ry[j], y);
       } else {
-        VT::store1(out + (int64_t)e0 * E, ox[0]);
-        VT::store1(out + (int64_t)(half + e0) * E, oy[0]);
+        x[0] = sx[j];
+        y[0] = sy[j];
       }
-    }
-  } else if (kind == kTail) {
-    // lanes beyond rotary_dim pass through unchanged (partial rotary)
 #pragma unroll
-    for (int o = 0; o < 2; ++o) {
-      if (!outs[o]) continue;
-      if constexpr (VECTOR) *reinterpret_cast<u32x4*>(outs[o] + in_off) = raw;
-      else VT::store1(outs[o] + in_off, raw1);
+      for (int i = 0; i < EV; ++i) {
+        const float cos_x = cs[e0[j] + i], cos_y = cs[half + e0[j] + i];
+        const float sin_x = cs[rd + e0[j] + i], sin_y = cs[rd + half + e0[j] + i];
+        ox[i] = x[i] * cos_x - y[i] * sin_x;
+        oy[i] = y[i] * cos_y + x[i] * sin_y;
+      }
+#pragma unroll
+      for (int o = 0; o < 2; ++o) {
+        if (!outs[o]) continue;
+        char* out = outs[o] + in_off[j];
+        if constexpr (VECTOR) {
+          u32x4* px = reinterpret_cast<u32x4*>(out + (int64_t)e0[j] * E);
+          u32x4* py = reinterpret_cast<u32x4*>(out + (int64_t)(half + e0[j]) * E);
+          if (o == 1) {
+            __builtin_nontemporal_store(VT::pack(ox), px);
+            __builtin_nontemporal_store(VT::pack(oy), py);
+          } else {
+            *px = VT::pack(ox);
+            *py = VT::pack(oy);
+          }
+        } else {
+          VT::store1(out + (int64_t)e0[j] * E, ox[0]);
+          VT::store1(out + (int64_t)(half + e0[j]) * E, oy[0]);
+        }
+      }
+    } else if (kind[j] == kTail) {
+      // lanes beyond rotary_dim pass through unchanged (partial rotary)
+#pragma unroll
+      for (int o = 0; o < 2; ++o) {
+        if (!outs[o]) continue;
+        if constexpr (VECTOR) *reinterpret_cast<u32x4*>(outs[o] + in_off[j]) = rx[j];
+        else VT::store1(outs[o] + in_off[j], sx[j]);
+      }
+    } else if (kind[j] == kValue && vc_row) {
+      // the V row goes to the cache as it is
+      if constexpr (VECTOR) __builtin_nontemporal_store(rx[j], reinterpret_cast<u32x4*>(vc_row + in_off[j]));
+      else VT::store1(vc_row + in_off[j], sx[j]);
     }
-  } else if (kind == kValue && vc_row) {
-    // the V row goes to the cache as it is
-    if constexpr (VECTOR) __builtin_nontemporal_store(raw, reinterpret_cast<u32x4*>(vc_row + in_off));
-    else VT::store1(vc_row + in_off, raw1);
   }
+}
+
+// One item per lane is what runs: 2 and 4 items per lane were measured from
+// 6 MiB to 324 MiB per launch and never gained (the launch is either latency-bound
+// or already has enough workgroups in flight).
+template <typename T, bool VECTOR>
+void launch_rope_ipl(const RopeArgs& a, dim3 grid, dim3 block, hipStream_t s) {
+  hipLaunchKernelGGL((rope_cache_kernel<T, VECTOR, 1>), grid, block, 0, s, a);
 }
 
 template <typename T>
 void launch_rope(const RopeArgs& a, int64_t num_tokens, bool vector, unsigned threads,
                  hipStream_t s) {
   const dim3 grid((unsigned)(num_tokens * a.groups_per_token)), block(threads);
-  if (vector) hipLaunchKernelGGL((rope_cache_kernel<T, true>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((rope_cache_kernel<T, false>), grid, block, 0, s, a);
+  if (vector) launch_rope_ipl<T, true>(a, grid, block, s);
+  else launch_rope_ipl<T, false>(a, grid, block, s);
 }
 
 struct RopeGeom {
@@ -383,14 +452,18 @@ int run_rope(const char* fn, const void* query, const void* key, const void* val
   const int ev = 16 / E;
   const bool vector = (align % 16 == 0) && ((g.rotary_dim / 2) % ev == 0) &&
                       ((g.head_dim - g.rotary_dim) % ev == 0) && (g.head_dim % ev == 0);
-  // one item per lane, two wavefronts per workgroup: a token of the 8B shape
-  // (320 rotation + 128 value vectors) spreads over four workgroups
   const int64_t ev_used = vector ? ev : 1;
   const int64_t heads = g.num_heads + g.num_kv_heads;
   const int64_t items = heads * ((g.rotary_dim / 2) / ev_used) +
                         heads * ((g.head_dim - g.rotary_dim) / ev_used) +
                         (c ? g.num_kv_heads * g.head_dim / ev_used : 0);
-  const unsigned threads = 128;
+  a.pv_shift = log2_exact((g.rotary_dim / 2) / ev_used);
+  a.cs_vector = ((uintptr_t)a.cos_sin_cache % 16 == 0) && ((2 * g.rotary_dim * E) % 16 == 0) ? 1 : 0;
+  // Two wavefronts per workgroup: a decode token of the 8B shape (320 rotation +
+  // 128 value vectors) spreads over four workgroups. 64 and 256 lanes measured
+  // within +-5 % of this from 6 MiB to 324 MiB per launch.
+  unsigned threads = (unsigned)kvc::g_rope_tune.threads;
+  if (threads != 64 && threads != 128 && threads != 256) threads = 128;
   a.groups_per_token = (uint32_t)std::max<int64_t>(1, (items + threads - 1) / threads);
   if (g.num_tokens * (int64_t)a.groups_per_token > 0x7fffffffll)
     return fail(KVC_ERR_UNSUPPORTED, "%s: launch of %lld workgroups is too large", fn,
