@@ -207,6 +207,36 @@ def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
                                  idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D, 16)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_special_values_through_the_identity_rotation(gpu, dtype):
+    """Position 0 has cos = 1, sin = 0: the rotation is x*1 - y*0. Every finite
+    value, signed zero, subnormal and infinity of the storage type must come back
+    with the same bits; a NaN must come back a NaN. (Pins the rounding step: the
+    float -> storage conversion may not flush subnormals or disturb exact values.)"""
+    D, H = 64, 2
+    # every 16-bit pattern once, in the x half and (another order) in the y half
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    T = (1 << 16) // (H * D // 2)
+    x = bits.reshape(T, H, D // 2)
+    y = np.roll(bits, 12345).reshape(T, H, D // 2)
+    fin = np.isfinite(torch.from_numpy(y.view(np.int16).copy()).view(dtype).float().numpy())
+    y = np.where(fin, y, 0).astype(np.uint16)             # 0 * inf would be a NaN: keep y finite
+    q_bits = np.concatenate([x, y], axis=2).reshape(T, H * D)
+    q = torch.from_numpy(q_bits.view(np.int16).copy()).view(dtype)
+    cs = rotary.make_cos_sin_cache(D, 4, 10000.0, dtype=dtype)
+    pos = torch.zeros(T, dtype=torch.int32)
+    q_out, k_out = kvc.rotary_pos_emb(q.to(gpu), q[:, :D].contiguous().to(gpu), pos.to(gpu), cs.to(gpu), D)
+    torch.cuda.synchronize()
+    got = q_out.cpu().view(torch.int16).numpy().view(np.uint16).reshape(T, H, D)
+    xf = q.float().numpy().reshape(T, H, D)[:, :, :D // 2]
+    nan = np.isnan(xf)
+    # y*1 + x*0 is NaN where x is not finite, so only the x half is compared for all patterns
+    assert np.array_equal(got[:, :, :D // 2][~nan], x[~nan])
+    assert np.isnan(q_out.cpu().float().numpy().reshape(T, H, D)[:, :, :D // 2][nan]).all()
+    yf_ok = np.isfinite(xf)
+    assert np.array_equal(got[:, :, D // 2:][yf_ok], y[yf_ok])
+
+
 def test_in_place_rotation_and_guards(gpu):
     T, Hq, Hkv, D = 20, 4, 2, 64
     q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, D, torch.bfloat16, max_pos=100)
