@@ -37,11 +37,11 @@ PREWARM_S = 0.15     # seconds of untimed launches ahead of every timed region
 ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 
 # HBM bytes per launch of the headline kernel (config 2, all layers in one launch)
-# from two rocprofv3 --pmc runs: FETCH_SIZE 16438.8 KiB x 2.0000 + WRITE_SIZE
-# 32816.5 KiB x 1.0000, the factors being what the same counters read for a
+# from two rocprofv3 --pmc runs: FETCH_SIZE 16438.9 KiB x 2.0000 + WRITE_SIZE
+# 32805.3 KiB x 1.0000, the factors being what the same counters read for a
 # plain elementwise kernel of known size (1 GiB read, 1 GiB written); summary in
 # profiles/hbm_traffic_fetch_size_write_size.txt. Only valid for the default workload.
-MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67270030
+MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67258665
 
 
 def log(*a):
