@@ -145,3 +145,32 @@ def test_rope_and_index_build_validate_their_arguments():
     assert g(None, None, None, None, 2, 0, 16, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
     assert g(1, 1, 1, 1, 2, 4, 0, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG   # page_size 0
     assert L.kvc_set_tuning(b"no_such_knob", 1) == _lib.KVC_ERR_INVALID_ARG
+
+
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """include/kvcache.h compiles as C99 with no extensions, and a C translation
+    unit that only knows the header links against libkvcache.so and runs the
+    entry points that need no GPU."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "kvcache.h"\n'
+        "int main(void) {\n"
+        "  if (kvc_abi_version() != KVC_ABI_VERSION) return 1;\n"
+        "  if (kvc_copy_blocks(0, 0, -1, 1, 1, 1, 1, 0) != KVC_ERR_INVALID_ARG) return 2;\n"
+        '  if (!strstr(kvc_last_error_string(), "negative")) return 3;\n'
+        "  if (kvc_swap_staging_bytes(3, 80, 65536, KVC_SWAP_DIRECT, 0) != 256) return 4;\n"
+        "  if (kvc_disk_close(0) != KVC_OK) return 5;\n"
+        '  puts("c ok");\n  return 0;\n}\n')
+    exe = tmp_path / "use"
+    lib_dir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Werror", "-I", os.path.join(REPO, "include"),
+                    str(src), "-L", lib_dir, "-lkvcache", f"-Wl,-rpath,{lib_dir}", "-o", str(exe)],
+                   check=True, capture_output=True, text=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and "c ok" in out.stdout, out.stdout + out.stderr
