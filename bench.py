@@ -59,6 +59,7 @@ def parse_args():
                         "rope (rotation fused with the write vs two launches), "
                         "shard (one rank's head slice of Llama-3.1-70B at tp=8), "
                         "disk (host <-> disk tier), "
+                        "sweep (write / copy_blocks / plain kernel over launch sizes; not in the default), "
                         "calib (a plain elementwise kernel of known size, for counter calibration); "
                         "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=1024,
@@ -242,6 +243,46 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
         out.append(entry(f"{tag}/{label}", nbytes, ms_w, ms_e, calls_per_step=calls,
                          launch="hipGraph replay" if mode == "graph" else "eager (Python + ctypes per call)"))
     return out, results
+
+
+def bench_size_sweep(torch, kvc, wl, pool, L, num_blocks, dev):
+    """One-launch write of T tokens x L layers, copy_blocks of P pairs x L layers and
+    a plain elementwise kernel of the same byte count, over launch sizes from
+    16 MiB to 2 GiB: where the fixed cost of a launch ends and bandwidth begins.
+    Sources rotate over at least 512 MiB so no launch finds its lines cached."""
+    s8 = wl.LLAMA_3_8B
+    out = []
+    for T in (64, 128, 256, 512, 1024, 2048, 4096, 8192):
+        one_way = T * 2 * s8.row_bytes * L
+        R = int(max(2, min(16, (512 << 20) // one_way)))
+        sets = []
+        for r in range(R):
+            slots = torch.from_numpy(wl.random_free_slots(s8, num_blocks, T, seed=r)).to(dev)
+            k = torch.randn(L, T, s8.num_kv_heads, s8.head_dim, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            sets.append((k, torch.randn_like(k), slots))
+        n_el = one_way // 4
+        srcs = [torch.zeros(n_el, dtype=torch.int32, device=dev) for _ in range(R)]
+        dsts = [torch.empty(n_el, dtype=torch.int32, device=dev) for _ in range(R)]
+        steps = max(R, min(64, (8 << 30) // (2 * one_way)) // R * R)
+        ms_w, ms_e = time_region(lambda i: kvc.reshape_and_cache_layers(sets[i % R][0], sets[i % R][1], pool,
+                                                                          sets[i % R][2]),
+                                 steps, 2, torch, graph_of=R)
+        ms_w2, ms_e2 = time_region(lambda i: torch.add(srcs[i % R], 1, out=dsts[i % R]), steps, 2, torch,
+                                   graph_of=R)
+        nbytes = 2 * one_way + 8 * T
+        out.append(entry(f"sweep/write, {T} random rows x {L} layers in one launch", nbytes, ms_w, ms_e,
+                         launch="hipGraph replay", plain_kernel_same_bytes_us=round(ms_e2 * 1e3, 3),
+                         plain_kernel_same_bytes_gbps=round(2 * one_way / (ms_e2 * 1e-3) / 1e9, 1)))
+        del sets, srcs, dsts
+        torch.cuda.empty_cache()
+    for P in (16, 64, 256, 1024, 4096):
+        maps = [torch.from_numpy(wl.copy_on_write_pairs(num_blocks, P, seed=r)[0]).to(dev) for r in range(4)]
+        nbytes = 2 * P * L * s8.block_bytes + 16 * P
+        steps = max(4, min(64, (16 << 30) // nbytes) // 4 * 4)
+        ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool, maps[i % 4]), steps, 2, torch, graph_of=4)
+        out.append(entry(f"sweep/copy_blocks, {P} pairs x {L} layers", nbytes, ms_w, ms_e,
+                         launch="hipGraph replay"))
+    return out
 
 
 def bench_disk_tier(kvc, shape_cfg, n, directory):
@@ -478,6 +519,9 @@ def main():
                                  max(5, min(args.steps, 20)), 3, torch)
         extra.append(entry(f"cfg4 copy_blocks (4096 pairs x {L} layers, 64 KiB blocks)", nbytes,
                            ms_w, ms_e, launch="eager"))
+    # ------------------------------------------------ launch-size sweep (8B shape, same pool)
+    if "sweep" in ops:
+        extra += bench_size_sweep(torch, kvc, wl, pool, L, args.pool_blocks, dev)
     del pool, sets
     torch.cuda.empty_cache()
 
