@@ -207,6 +207,59 @@ def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
                                  idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D, 16)
 
 
+def test_graph_replay_of_the_fused_step_matches_eager_every_time(gpu):
+    """A captured layer loop of `PagedRotaryWritePlan.run` (static q/k/v and output
+    buffers) is replayed with fresh inputs and eager work between replays; every
+    replay must give the bits of the eager call."""
+    s = wl.LLAMA_3_8B
+    L, nb, bs, Hq, Hkv, D = 3, 96, s.block_size, 32, s.num_kv_heads, s.head_dim
+    rng = np.random.default_rng(31)
+    w = wl._write_workload(s, nb, [7, 30, 0], [1, 1, 20], rng)
+    idx = kvc.to_device(w.index, bs, gpu)
+    T = w.num_tokens
+    cs = rotary.make_cos_sin_cache(D, 512, 500000.0, dtype=torch.bfloat16).to(gpu)
+    plan = kvc.PagedRotaryWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices,
+                                    idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D, bs)
+    sq = torch.zeros(L, T, Hq * D, dtype=torch.bfloat16, device=gpu)
+    sk = torch.zeros(L, T, Hkv * D, dtype=torch.bfloat16, device=gpu)
+    sv = torch.zeros_like(sk)
+    q_out = torch.zeros_like(sq)
+    pool = torch.zeros(L, nb, 2, bs, Hkv, D, dtype=torch.bfloat16, device=gpu)
+
+    def step():
+        for l in range(L):
+            plan.run(sq[l], sk[l], sv[l], pool[l], query_out=q_out[l])
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    g = torch.Generator().manual_seed(41)
+    for rep in range(4):
+        q = torch.randn(L, T, Hq * D, generator=g).bfloat16().to(gpu)
+        k = torch.randn(L, T, Hkv * D, generator=g).bfloat16().to(gpu)
+        v = torch.randn(L, T, Hkv * D, generator=g).bfloat16().to(gpu)
+        want_pool = torch.zeros_like(pool)
+        want_q = torch.empty_like(q)
+        for l in range(L):                                         # eager work between replays
+            want_q[l], _ = kvc.rotary_pos_emb_and_append_paged(
+                q[l], k[l], v[l], idx.batch_indices, idx.positions, cs, D, want_pool[l],
+                idx.kv_block_indices, idx.kv_block_indptrs, idx.kv_last_block_lens, return_key=False)
+        sq.copy_(q), sk.copy_(k), sv.copy_(v)
+        pool.zero_()
+        q_out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(q_out, want_q), rep
+        assert torch.equal(pool.view(torch.int16), want_pool.view(torch.int16)), rep
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_special_values_through_the_identity_rotation(gpu, dtype):
     """Position 0 has cos = 1, sin = 0: the rotation is x*1 - y*0. Every finite
