@@ -36,36 +36,6 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or install ROCm under /opt/rocm)")
 
 
-NATIVE_CHECK_SRC = os.path.join(REPO_ROOT, "tests", "native", "abi_check.cpp")
-NATIVE_CHECK_BIN = os.path.join(REPO_ROOT, "tests", "native", "abi_check")
-ORACLE_C = os.path.join(REPO_ROOT, "oracle", "kvc_oracle.c")
-
-
-def build_native_check(verbose: bool = False) -> str:
-    """Compile tests/native/abi_check.cpp: a plain HIP program that drives the
-    C ABI without Python and checks it against the C oracle (linked in as an
-    object of its own; the library itself never sees the oracle)."""
-    oracle_obj = NATIVE_CHECK_BIN + "_oracle.o"
-    main_obj = NATIVE_CHECK_BIN + "_main.o"
-    hipcc = find_hipcc()
-    steps = [
-        ["gcc", "-O2", "-std=c11", "-c", ORACLE_C, "-o", oracle_obj],
-        [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-I", INCLUDE, "-c", NATIVE_CHECK_SRC, "-o", main_obj],
-        [hipcc, main_obj, oracle_obj, "-L", PKG_DIR, "-lkvcache",
-         "-Wl,-rpath,$ORIGIN/../../lmserve_amd", "-o", NATIVE_CHECK_BIN],
-    ]
-    for cmd in steps:
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        proc = subprocess.run(cmd, capture_output=True, text=True)
-        if proc.returncode != 0:
-            raise RuntimeError("native check build failed:\n" + proc.stdout + proc.stderr)
-    os.remove(oracle_obj)
-    os.remove(main_obj)
-    return NATIVE_CHECK_BIN
-
-
 def build(verbose: bool = False) -> str:
     """Compile the library; always recompiles. Returns the path of the .so."""
     cmd = [find_hipcc(), *HIPCC_FLAGS, "-I", INCLUDE, *SOURCES, "-o", LIB_PATH + ".tmp"]
@@ -78,13 +48,11 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
-def ensure_built(native_check: bool = False) -> None:
+def ensure_built() -> None:
     """For tests, the smoke check and the benchmark: use what is built, build
     only what is missing. The operators themselves never build anything."""
     if not os.path.exists(LIB_PATH):
         build(verbose=True)
-    if native_check and not os.path.exists(NATIVE_CHECK_BIN):
-        build_native_check(verbose=True)
 
 
 if __name__ == "__main__":
