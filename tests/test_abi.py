@@ -174,3 +174,26 @@ def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
                    check=True, capture_output=True, text=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
     assert out.returncode == 0 and "c ok" in out.stdout, out.stdout + out.stderr
+
+
+def test_operators_fail_loudly_without_the_library(monkeypatch, tmp_path):
+    """No CPU fallback: with the shared library absent every entry into the
+    binding raises, and so do the operators that sit on it."""
+    import torch
+
+    import lmserve_amd as kvc
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libkvcache.so"))
+    with pytest.raises(_lib.KVCacheLibraryError, match="no CPU fallback"):
+        _lib.lib()
+    with pytest.raises(_lib.KVCacheLibraryError):
+        kvc.DiskTier(str(tmp_path / "x.npy"), (2, 1, 8), np.uint16)
+    # the device operators refuse CPU tensors before they even reach the library
+    pool = torch.zeros(1, 4, 2, 2, 1, 4, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        kvc.copy_blocks(pool, {0: [1]})
+    with pytest.raises(ValueError):
+        kvc.reshape_and_cache(torch.zeros(1, 1, 4, dtype=torch.bfloat16),
+                              torch.zeros(1, 1, 4, dtype=torch.bfloat16), pool[0],
+                              torch.zeros(1, dtype=torch.int64))
