@@ -395,6 +395,8 @@ def cpu_baseline_write(torch, shape_cfg, L, seconds):
 
 
 def main():
+    import numpy as np
+
     args = parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this path has no cross-GPU step "
@@ -626,6 +628,27 @@ def main():
                     extra.append({"name": f"cfg5 {direction} ({mode}; {n} blocks x {L5} layers x 64 KiB)",
                                   "ms_per_call": round(t * 1e3, 2),
                                   "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                  "bytes_per_call": int(nbytes)})
+                if mode == "direct":
+                    # both directions at once on the worker's two streams (PCIe is full duplex):
+                    # write-through of one set of blocks while another set is fetched
+                    host_in = np.arange(n // 2, n, dtype=np.int64)
+                    both_out = [kvc.BlockMapping.from_pairs(zip(old[:n // 2].tolist(), range(n // 2)))]
+                    both_in = [kvc.BlockMapping.from_pairs(zip(host_in.tolist(), new[n // 2:].tolist()))]
+                    times = []
+                    for _ in range(4):
+                        torch.cuda.synchronize()
+                        t0 = time.perf_counter()
+                        worker.save_kv_blocks_to_host_nowait(both_out)
+                        worker.load_kv_blocks_from_host_nowait(both_in)
+                        worker.dtoh_stream.synchronize()
+                        worker.htod_stream.synchronize()
+                        times.append(time.perf_counter() - t0)
+                    t = sorted(times[1:])[1]
+                    extra.append({"name": f"cfg5 swap_out and swap_in at once (direct; {n // 2} blocks each way)",
+                                  "ms_per_call": round(t * 1e3, 2),
+                                  "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                  "pcie_gbps_note": "sum of both directions",
                                   "bytes_per_call": int(nbytes)})
             finally:
                 worker.close()
