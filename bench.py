@@ -662,6 +662,19 @@ def main():
                                   "pcie_gbps": round(nbytes / t / 1e9, 2),
                                   "bytes_per_call": int(nbytes)})
                 if mode == "direct":
+                    # one call per layer, as the layer-pipelined protocol issues them
+                    times = []
+                    for _ in range(3):
+                        torch.cuda.synchronize()
+                        t0 = time.perf_counter()
+                        for l in range(L5):
+                            worker.save_kv_blocks_to_host_nowait(out_maps, layer_begin=l, layer_end=l + 1)
+                        worker.dtoh_stream.synchronize()
+                        times.append(time.perf_counter() - t0)
+                    t = sorted(times)[1]
+                    extra.append({"name": f"cfg5 swap_out layer by layer (direct; {L5} calls of {n} blocks x 1 layer)",
+                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                  "bytes_per_call": int(nbytes)})
                     # both directions at once on the worker's two streams (PCIe is full duplex):
                     # write-through of one set of blocks while another set is fetched
                     host_in = np.arange(n // 2, n, dtype=np.int64)
