@@ -395,6 +395,62 @@ def cpu_baseline_write(torch, shape_cfg, L, seconds):
                       f"({pool.numel() * 2 / 2**30:.1f} GiB), {el:.1f} s"}
 
 
+def cpu_baseline_others(torch, wl, seconds_each):
+    """torch-CPU statements of the other operations on bounded samples: the
+    prefill-chunk write (config 3 shape), copy_blocks (config 4 shape) and the
+    swap in both directions (config 5 rows), pools scaled to fit host RAM."""
+    from oracle import torch_cpu
+
+    def timed(fn, nbytes, what):
+        fn()  # warm-up
+        n, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            n += 1
+            el = time.perf_counter() - t0
+            if el >= seconds_each or n >= 5000:
+                break
+        return {"name": what, "value": round(nbytes * n / el / 1e9, 2), "unit": "GB/s",
+                "us_per_call": round(el / n * 1e6, 1), "calls": n, "seconds": round(el, 1)}
+
+    out = []
+    # config 3: 2048 tokens x 28 layers, Qwen2.5-7B rows
+    sq = wl.QWEN_2_5_7B
+    nb = 2048
+    w = wl.chunked_prefill(sq, num_blocks=nb, num_seqs=4, chunk_tokens=2048, min_context=16,
+                           max_context=4096, seed=0)
+    slots = torch.from_numpy(w.index.slot_mapping)
+    pool = torch.zeros(sq.num_layers, nb, 2, sq.block_size, sq.num_kv_heads, sq.head_dim, dtype=torch.bfloat16)
+    key = torch.randn(sq.num_layers, w.num_tokens, sq.num_kv_heads, sq.head_dim).to(torch.bfloat16)
+    value = torch.randn_like(key)
+    out.append(timed(lambda: torch_cpu.reshape_and_cache_layers_cpu(key, value, pool, slots),
+                     w.algorithmic_bytes(sq.num_layers),
+                     f"config 3 write, 2048 tokens x {sq.num_layers} layers, pool scaled to {nb} blocks/layer"))
+    del pool, key, value
+    # config 4: copy_blocks, 512 pairs x 32 layers x 64 KiB on a 4096-block pool
+    s8 = wl.LLAMA_3_8B
+    nb, P = 4096, 512
+    pool = torch.zeros(s8.num_layers, nb, s8.block_elems, dtype=torch.bfloat16)
+    flat, _ = wl.copy_on_write_pairs(nb, P, seed=0)
+    src, dst = torch.from_numpy(flat[0::2].copy()), torch.from_numpy(flat[1::2].copy())
+    out.append(timed(lambda: torch_cpu.copy_blocks_cpu(pool, src, dst), 2 * P * s8.num_layers * s8.block_bytes,
+                     f"config 4 copy_blocks, {P} pairs x {s8.num_layers} layers x 64 KiB, pool scaled to {nb} blocks/layer"))
+    del pool
+    # config 5: swap rows, 128 blocks x 80 layers x 64 KiB each way
+    s70 = wl.LLAMA_3_1_70B
+    nb, n = 512, 128
+    pool = torch.zeros(s70.num_layers, nb, s70.block_elems, dtype=torch.bfloat16)
+    host = torch.zeros(n, s70.num_layers, s70.block_elems, dtype=torch.bfloat16)
+    old, host_ids, new = wl.swap_round_trip(nb, n, seed=0)
+    old_t, host_t, new_t = (torch.from_numpy(a) for a in (old, host_ids, new))
+    nbytes = 2 * n * s70.num_layers * s70.block_bytes     # read + written
+    out.append(timed(lambda: torch_cpu.swap_out_cpu(pool, host, old_t, host_t), nbytes,
+                     f"config 5 swap-out rows, {n} blocks x {s70.num_layers} layers x 64 KiB (host memory both sides)"))
+    out.append(timed(lambda: torch_cpu.swap_in_cpu(pool, host, host_t, new_t), nbytes,
+                     f"config 5 swap-in rows, {n} blocks x {s70.num_layers} layers x 64 KiB (host memory both sides)"))
+    return out
+
+
 def main():
     import numpy as np
 
@@ -750,6 +806,8 @@ def main():
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline_write(torch, s8, L, args.cpu_seconds)
+        if ops:
+            cpu["other_ops"] = cpu_baseline_others(torch, wl, max(1.0, args.cpu_seconds / 4))
 
     line = {
         "metric": "achieved HBM GB/s, KV write (Llama-3-8B decode step)",
