@@ -622,6 +622,10 @@ def main():
         ms_w, ms_e = time_region(lambda i: torch.add(a, 1, out=b), 10, 2, torch)
         extra.append(entry("calibration: plain elementwise kernel, 1 GiB read + 1 GiB written "
                            "(torch.add(int32, 1))", 2 << 30, ms_w, ms_e, launch="eager"))
+        # write-only ceiling of the machine: a plain fill of 1 GiB
+        ms_w, ms_e = time_region(lambda i: b.fill_(3), 10, 2, torch)
+        extra.append(entry("calibration: plain fill, 1 GiB written (Tensor.fill_)", 1 << 30, ms_w, ms_e,
+                           launch="eager"))
         del a, b
         torch.cuda.empty_cache()
 
