@@ -1,7 +1,9 @@
 /*
  * kvcache.h -- C ABI of libkvcache, the MI355X (gfx950) paged KV-cache
- * data-movement library: slot-mapped K/V write, block copy, and block
- * gather/scatter between the HBM pool and a pinned host pool.
+ * data-movement library: slot-mapped and page-table K/V write (alone or fused
+ * with the rotary embedding), block copy, block gather/scatter between the HBM
+ * pool and a pinned host pool, the index preparation of a step, and the
+ * host <-> disk tier of the block cache.
  *
  * Conventions shared by every entry point
  *   - plain pointers and sizes only; `stream` arguments are hipStream_t passed
@@ -9,7 +11,9 @@
  *   - returns KVC_OK (0) or a negative kvc_status; never throws; the text of the
  *     last failure on the calling thread is kvc_last_error_string();
  *   - asynchronous on the given stream(s) unless the name ends in _sync;
- *   - never allocates or frees device memory; the caller owns every buffer;
+ *   - never allocates or frees device memory; the caller owns every buffer
+ *     (host-side helpers own small pinned bounce buffers, events and, in the
+ *     disk tier, per-thread staging);
  *   - every offset is computed in 64 bits (one layer of a 65536-block Llama-3-8B
  *     pool already holds 2^31 elements);
  *   - block ids / slots outside [0, capacity) are skipped by the kernels
