@@ -336,8 +336,9 @@ int kvc_scatter_blocks(void* pool, const void* buffer, const int64_t* block_ids,
  * The file is a NumPy `.npy` array of shape (num_blocks, num_layers, block_elems)
  * and dtype string `descr` ("<u2" for bf16 lanes carried as uint16, kv_worker.py:17-22).
  * kvc_disk_open reuses a file whose stored shape and dtype match and removes and
- * recreates any other, as the reference does; a new file is sparse and starts
- * its data at byte 4096. With KVC_DISK_DIRECT the transfers bypass the page
+ * recreates any other, as the reference does; a new file is sparse (unless
+ * KVC_DISK_PREALLOCATE asks for its blocks to be reserved) and starts its data
+ * at byte 4096. With KVC_DISK_DIRECT the transfers bypass the page
  * cache (O_DIRECT) whenever the data offset and one block's bytes over all
  * layers are multiples of 4096 and the file system allows it; otherwise they are
  * ordinary buffered reads and writes. The host side of an O_DIRECT transfer is
@@ -356,7 +357,10 @@ int kvc_scatter_blocks(void* pool, const void* buffer, const int64_t* block_ids,
  */
 typedef struct kvc_disk kvc_disk;
 
-enum { KVC_DISK_DIRECT = 1 };
+enum {
+  KVC_DISK_DIRECT = 1,      /* bypass the page cache where alignment allows            */
+  KVC_DISK_PREALLOCATE = 2 /* a new file reserves all its blocks at once (posix_fallocate) */
+};
 enum {
   KVC_DISK_INFO_DATA_OFFSET = 0, /* byte offset of block 0 in the file            */
   KVC_DISK_INFO_DIRECT = 1,      /* 1 if an O_DIRECT descriptor is in use         */

@@ -22,6 +22,7 @@ KVC_ERR_HIP = -5
 KVC_ERR_IO = -6
 
 KVC_DISK_DIRECT = 1
+KVC_DISK_PREALLOCATE = 2
 KVC_DISK_INFO_DATA_OFFSET = 0
 KVC_DISK_INFO_DIRECT = 1
 KVC_DISK_INFO_CREATED = 2

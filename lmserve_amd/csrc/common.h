@@ -27,6 +27,9 @@ struct RopeTuning {
 };
 extern RopeTuning g_rope_tune;
 
+// MiB of aligned staging per thread in the disk tier ("disk_bounce_mib").
+extern int g_disk_bounce_mib;
+
 }  // namespace kvc
 
 #define KVC_HIP(call)                                                          \

@@ -17,6 +17,7 @@
 // extent is aligned for O_DIRECT, which keeps tens of GiB of KV blocks out of
 // the page cache. No GPU work in this file.
 #include <fcntl.h>
+#include <sys/mman.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
@@ -27,14 +28,17 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <thread>
+#include <utility>
 #include <vector>
 
 #include "kvcache.h"
 
 namespace kvc {
 int fail(int code, const char* fmt, ...);
+int g_disk_bounce_mib = 4;  // per-thread staging of an O_DIRECT transfer (kvc_set_tuning "disk_bounce_mib")
 }
 using kvc::fail;
 
@@ -53,13 +57,47 @@ struct kvc_disk {
   std::atomic<const void*> bounce_pool{nullptr};
   std::atomic<bool> last_bounced{false};
   std::string path;
+
+  // Staging buffers of O_DIRECT transfers, kept with the handle so a call does
+  // not fault fresh pages in every time: 2 MiB-aligned and advised as huge pages
+  // (large physically contiguous segments make large block requests), touched
+  // once when made.
+  std::mutex stage_lock;
+  std::vector<std::pair<char*, int64_t>> stages;
+
+  char* take_stage(int64_t bytes) {
+    {
+      std::lock_guard<std::mutex> g(stage_lock);
+      for (size_t i = 0; i < stages.size(); ++i) {
+        if (stages[i].second == bytes) {
+          char* p = stages[i].first;
+          stages.erase(stages.begin() + (long)i);
+          return p;
+        }
+      }
+    }
+    void* mem = nullptr;
+    const size_t huge = size_t(2) << 20;
+    const size_t size = ((size_t)bytes + huge - 1) / huge * huge;
+    if (posix_memalign(&mem, huge, size) != 0) return nullptr;
+    (void)madvise(mem, size, MADV_HUGEPAGE);
+    memset(mem, 0, size);
+    return static_cast<char*>(mem);
+  }
+  void give_stage(char* p, int64_t bytes) {
+    std::lock_guard<std::mutex> g(stage_lock);
+    if (stages.size() < 64) stages.emplace_back(p, bytes);
+    else free(p);
+  }
+  ~kvc_disk() {
+    for (auto& st : stages) free(st.first);
+  }
 };
 
 namespace {
 
 constexpr int64_t kAlign = 4096;
 constexpr int64_t kMaxExtent = int64_t(64) << 20;  // split longer runs so threads share them
-constexpr int64_t kBounceBytes = int64_t(4) << 20;  // per-thread staging for O_DIRECT
 
 // "{'descr': '<u2', 'fortran_order': False, 'shape': (8192, 80, 32768), }" padded
 // with spaces and a final newline to `total` bytes including the 10-byte preamble
@@ -162,9 +200,10 @@ int read_all(int fd, char* p, int64_t n, int64_t off) {
 
 // One extent through an aligned staging buffer: the file side stays O_DIRECT, the
 // host side is an ordinary memcpy.
-int bounce_io(int fd, bool to_disk, char* host, int64_t len, int64_t off, char* stage) {
+int bounce_io(int fd, bool to_disk, char* host, int64_t len, int64_t off, char* stage,
+              int64_t stage_bytes) {
   while (len > 0) {
-    const int64_t n = std::min(len, kBounceBytes);
+    const int64_t n = std::min(len, stage_bytes);
     int err;
     if (to_disk) {
       memcpy(stage, host, (size_t)n);
@@ -222,6 +261,7 @@ int run_io(const char* fn, kvc_disk* d, bool to_disk, char* host_pool, int64_t n
   const int fd = direct ? d->fd_direct : d->fd;
   const int nthreads = (int)std::max<int64_t>(1, std::min<int64_t>({(int64_t)(threads > 0 ? threads : 8),
                                                                    (int64_t)ext.size(), 64}));
+  const int64_t stage_bytes = (int64_t)std::max(1, std::min(kvc::g_disk_bounce_mib, 256)) << 20;
   std::atomic<size_t> next{0};
   std::atomic<int> first_errno{0};
   std::atomic<bool> faulted{false};
@@ -239,10 +279,8 @@ int run_io(const char* fn, kvc_disk* d, bool to_disk, char* host_pool, int64_t n
         err = to_disk ? write_all(fd, h, len, off) : read_all(fd, h, len, off);
       if (direct && err == EFAULT) {
         if (in_place) faulted.store(true, std::memory_order_relaxed);
-        void* mem = stage;
-        if (!mem && posix_memalign(&mem, (size_t)kAlign, (size_t)kBounceBytes) != 0) mem = nullptr;
-        stage = static_cast<char*>(mem);
-        err = stage ? bounce_io(fd, to_disk, h, len, off, stage) : ENOMEM;
+        if (!stage) stage = d->take_stage(stage_bytes);
+        err = stage ? bounce_io(fd, to_disk, h, len, off, stage, stage_bytes) : ENOMEM;
       }
       if (err) {
         int expected = 0;
@@ -250,7 +288,7 @@ int run_io(const char* fn, kvc_disk* d, bool to_disk, char* host_pool, int64_t n
         break;
       }
     }
-    free(stage);
+    if (stage) d->give_stage(stage, stage_bytes);
   };
   if (nthreads == 1) {
     work();
@@ -318,6 +356,9 @@ int kvc_disk_open(const char* path, const char* descr, int64_t num_blocks, int64
     const std::string h = npy_header(descr, num_blocks, num_layers, block_elems, (size_t)kAlign);
     int err = write_all(fd, h.data(), (int64_t)h.size(), 0);
     if (!err && ftruncate(fd, (off_t)(kAlign + payload)) != 0) err = errno;  // sparse, like open_memmap
+    // reserve the blocks now: later writes then meet no allocation in the file
+    // system and cannot run out of space half-way
+    if (!err && (flags & KVC_DISK_PREALLOCATE)) err = posix_fallocate(fd, 0, (off_t)(kAlign + payload));
     if (err) {
       close(fd);
       unlink(path);

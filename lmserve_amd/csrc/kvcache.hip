@@ -929,6 +929,7 @@ int kvc_set_tuning(const char* key, int value) {
   else if (!strcmp(key, "write_order")) g_tune.write_order = value;
   else if (!strcmp(key, "direct_max_wgs")) g_tune.direct_max_wgs = value;
   else if (!strcmp(key, "rope_threads")) kvc::g_rope_tune.threads = value;
+  else if (!strcmp(key, "disk_bounce_mib")) kvc::g_disk_bounce_mib = value;
   else return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: unknown key '%s'", key);
   return KVC_OK;
 }

@@ -24,10 +24,13 @@ class DiskTier:
 
     shape: `(num_disk_blocks, num_layers, block_elems)`; dtype: the NumPy dtype
     of the host pool (bf16 lanes are carried as uint16, kv_worker.py:17-22).
+    preallocate: a new file reserves all its blocks when it is made (the
+    reference's memory map is sparse); first writes then run at the device's
+    rate and cannot fail for lack of space.
     """
 
     def __init__(self, path: str, shape: Tuple[int, int, int], dtype, direct: bool = True,
-                 threads: int = 8):
+                 threads: int = 8, preallocate: bool = False):
         if len(shape) != 3:
             raise ValueError("disk KV cache shape must be (num_disk_blocks, num_layers, block_elems)")
         self.path = str(path)
@@ -37,7 +40,9 @@ class DiskTier:
         handle = ctypes.c_void_p()
         _lib.check(_lib.lib().kvc_disk_open(
             self.path.encode(), self.dtype.str.encode(), self.shape[0], self.shape[1], self.shape[2],
-            self.dtype.itemsize, _lib.KVC_DISK_DIRECT if direct else 0, ctypes.byref(handle)))
+            self.dtype.itemsize,
+            (_lib.KVC_DISK_DIRECT if direct else 0) | (_lib.KVC_DISK_PREALLOCATE if preallocate else 0),
+            ctypes.byref(handle)))
         self._h: Optional[ctypes.c_void_p] = handle
 
     # ------------------------------------------------------------------ facts

@@ -181,6 +181,42 @@ def test_save_and_load_may_run_concurrently_on_disjoint_blocks(tmp_path):
     assert np.array_equal(disk[16:24], want[24:32]) and np.array_equal(disk[:16], want[:16])
 
 
+def test_preallocation_reserves_the_blocks_of_a_new_file(tmp_path):
+    sparse, full = str(tmp_path / "sparse.npy"), str(tmp_path / "full.npy")
+    shape = (64, 2, 8192)                                   # 2 MiB of payload
+    with DiskTier(sparse, shape, np.uint16) as a, DiskTier(full, shape, np.uint16, preallocate=True) as b:
+        assert a.created and b.created
+    payload = 64 * 2 * 8192 * 2
+    assert os.stat(full).st_blocks * 512 >= payload         # reserved on disk
+    assert os.stat(sparse).st_blocks * 512 < payload        # holes, like the reference's memory map
+    assert os.path.getsize(full) == os.path.getsize(sparse) == 4096 + payload
+    assert not np.asarray(np.load(full, mmap_mode="r")).any()
+
+
+def test_staging_buffers_are_reused_across_calls(tmp_path):
+    """Staged transfers (here: an unaligned pool) keep their aligned buffers with
+    the handle; many calls in a row give the same bytes as the closed form."""
+    rng = np.random.default_rng(13)
+    backing = np.zeros(12 * 2 * 4096 + 8, dtype=np.uint16)
+    host = backing[1:1 + 12 * 2 * 4096].reshape(12, 2, 4096)
+    _fill(host, rng)
+    want_disk = np.zeros((10, 2, 4096), dtype=np.uint16)
+    path = str(tmp_path / "reuse.npy")
+    with DiskTier(path, (10, 2, 4096), np.uint16, threads=3) as d:
+        for step in range(8):
+            src = rng.permutation(12)[:5]
+            dst = rng.permutation(10)[:5]
+            d.save_blocks(host, src, dst)
+            orc.save_blocks_to_disk_np(host, want_disk, src, dst)
+            back = rng.permutation(12)[:4]
+            frm = rng.permutation(10)[:4]
+            want_host = host.copy()
+            orc.load_blocks_from_disk_np(want_host, want_disk, frm, back)
+            d.load_blocks(host, frm, back)
+            assert np.array_equal(host, want_host), step
+    assert np.array_equal(np.load(path, mmap_mode="r"), want_disk)
+
+
 def test_a_numpy_made_file_is_reused_in_place(tmp_path):
     """The reference creates the file with np.lib.format.open_memmap (kv_worker.py:78-82):
     data starts at byte 128 there, so the tier uses buffered I/O on it."""
