@@ -133,7 +133,8 @@ class KVWorker:
       range moves in one call.
     disk_direct_io / disk_threads: the disk tier bypasses the page cache when
       alignment and the file system allow, and spreads block extents over this
-      many threads (the reference copies rows through a memory map on 4).
+      many threads (the reference copies rows through a memory map on 4);
+      `disk_preallocate` reserves a new file's blocks when it is made.
     """
 
     def __init__(
@@ -147,6 +148,7 @@ class KVWorker:
         kv_worker_handle=None,
         disk_direct_io: bool = True,
         disk_threads: int = 8,
+        disk_preallocate: bool = False,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -182,7 +184,8 @@ class KVWorker:
                 raise ValueError("disk_kv_cache_file is required when num_disk_blocks > 0")
             self.disk_tier = DiskTier(disk_kv_cache_file,
                                       (self.num_disk_blocks, num_layers, block_elems), np_dtype,
-                                      direct=disk_direct_io, threads=disk_threads)
+                                      direct=disk_direct_io, threads=disk_threads,
+                                      preallocate=disk_preallocate)
             self.disk_kv_caches = self.disk_tier.memmap("r")
         else:
             self.disk_tier = None
