@@ -64,6 +64,7 @@ struct Tuning {
   int write_vpt = 0;        // vectors per lane in write_rows, 0 = by size
   int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
+  int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
   int direct_max_wgs = 64;  // grid cap of the direct swap kernel: PCIe saturates with a few
                             // dozen workgroups, the rest of the GPU stays free for the model
 };
@@ -551,30 +552,40 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
   a.items_per_token = (uint32_t)items64;
 
-  // Vectors per lane, from sweeps on MI355X. One vector per lane (the leanest
-  // lane, the most workgroups) is best whenever the launch is either smaller
-  // than one resident set of workgroups (8 of 256 lanes per CU) or many times
-  // larger. In between, a launch that 2 or 4 vectors per lane shrink to exactly
-  // one resident set runs 3-5 % faster that way (no second round of workgroup
-  // dispatch, several loads in flight per lane): the 64 MiB decode step of an
+  // Launch shape, from sweeps on MI355X. 256-lane workgroups with one vector per
+  // lane (the leanest lane, the most workgroups) are best whenever the launch is
+  // either smaller than one resident set of workgroups (2048 lanes per CU) or
+  // many times larger. In between, a launch that 2 or 4 vectors per lane shrink
+  // to exactly one resident set runs 3-5 % faster that way (no second round of
+  // workgroup dispatch, several loads in flight per lane), and another 3 % faster
+  // with that set made of 128-lane workgroups: the 64 MiB decode step of an
   // 8-head model is that case. Rows under 1 KiB never gain: a lane's vectors
   // then fall in different layers' rows.
   WriteLaunch l{};
+  const auto wgs = [&](int64_t lanes_per_wg, int v) {
+    return g.num_tokens * ((items64 + (int64_t)v * lanes_per_wg - 1) / ((int64_t)v * lanes_per_wg));
+  };
+  const bool fixed_wg = g_tune.write_threads == 64 || g_tune.write_threads == 128 || g_tune.write_threads == 256;
+  int64_t wg = fixed_wg ? g_tune.write_threads : kThreads;
   l.vpt = g_tune.write_vpt;
   if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8) {
     l.vpt = 1;
-    const int64_t resident = (int64_t)resident_workgroups();
-    const auto wgs = [&](int v) {
-      return g.num_tokens * ((items64 + (int64_t)v * kThreads - 1) / ((int64_t)v * kThreads));
-    };
-    if (g.row_elems * E >= 1024 && wgs(1) > resident) {
-      if (wgs(2) <= resident) l.vpt = 2;
-      else if (wgs(4) <= resident) l.vpt = 4;
+    const int64_t resident256 = (int64_t)resident_workgroups();
+    if (g.row_elems * E >= 1024 && wgs(kThreads, 1) > resident256) {
+      const int64_t shaped = fixed_wg ? wg : 128;
+      const int64_t resident = resident256 * (kThreads / shaped);
+      if (wgs(shaped, 2) <= resident) {
+        l.vpt = 2;
+        wg = shaped;
+      } else if (wgs(shaped, 4) <= resident) {
+        l.vpt = 4;
+        wg = shaped;
+      }
     }
   }
-  while (l.vpt > 1 && (int64_t)(l.vpt / 2) * kThreads >= items64) l.vpt /= 2;
+  while (l.vpt > 1 && (int64_t)(l.vpt / 2) * wg >= items64) l.vpt /= 2;
   const int64_t lanes = (items64 + l.vpt - 1) / l.vpt;
-  l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes + 63) / 64 * 64);
+  l.threads = (unsigned)std::min<int64_t>(wg, (lanes + 63) / 64 * 64);
   l.nt = (g_tune.write_nt & 1) != 0;
   l.ntl = (g_tune.write_nt & 2) != 0;
   const int64_t groups = (items64 + (int64_t)l.vpt * l.threads - 1) / ((int64_t)l.vpt * l.threads);
@@ -927,6 +938,7 @@ int kvc_set_tuning(const char* key, int value) {
   else if (!strcmp(key, "write_vpt")) g_tune.write_vpt = value;
   else if (!strcmp(key, "write_nt")) g_tune.write_nt = value;
   else if (!strcmp(key, "write_order")) g_tune.write_order = value;
+  else if (!strcmp(key, "write_threads")) g_tune.write_threads = value;
   else if (!strcmp(key, "direct_max_wgs")) g_tune.direct_max_wgs = value;
   else if (!strcmp(key, "rope_threads")) kvc::g_rope_tune.threads = value;
   else if (!strcmp(key, "disk_bounce_mib")) kvc::g_disk_bounce_mib = value;
