@@ -61,9 +61,18 @@ const char* kvc_last_error_string(void);
 
 /* Launch-shape knobs for measurement sweeps; process-wide, not thread-safe
  * against concurrent launches. No counterpart in the reference. Keys:
- * "copy_unroll" and "gather_unroll" (1,2,4,8,16), "copy_nt" (0/1), "copy_order" (0/1), "copy_max_wgs" (0 = one
- * workgroup per chunk), "write_vpt" (0 = by size, 1, 2, 4, 8), "write_nt" (bit 0: non-temporal stores, bit 1: loads), "write_order" (0/1),
- * "direct_max_wgs". Unknown key: KVC_ERR_INVALID_ARG. */
+ *   "copy_unroll", "gather_unroll"   16-byte vectors per lane in the tile kernel (1, 2, 4, 8, 16)
+ *   "copy_nt"                         non-temporal loads and stores in the tile kernel (0/1)
+ *   "copy_order"                      1 = walk all blocks of a layer before the next layer
+ *   "copy_max_wgs"                    grid cap of the tile kernel (0 = one workgroup per chunk)
+ *   "direct_max_wgs"                  grid cap of the direct swap kernel
+ *   "write_vpt"                       vectors per lane in the write kernel (0 = by size, 1, 2, 4, 8)
+ *   "write_threads"                   lanes per workgroup in the write kernel (0 = by size, 64, 128, 256)
+ *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads
+ *   "write_order"                     1 = a token's workgroups are neighbours in the grid
+ *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
+ *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier
+ * Unknown key: KVC_ERR_INVALID_ARG. */
 int kvc_set_tuning(const char* key, int value);
 
 /* ---------------------------------------------------------------------------
