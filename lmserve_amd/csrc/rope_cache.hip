@@ -459,11 +459,13 @@ int run_rope(const char* fn, const void* query, const void* key, const void* val
                         (c ? g.num_kv_heads * g.head_dim / ev_used : 0);
   a.pv_shift = log2_exact((g.rotary_dim / 2) / ev_used);
   a.cs_vector = ((uintptr_t)a.cos_sin_cache % 16 == 0) && ((2 * g.rotary_dim * E) % 16 == 0) ? 1 : 0;
-  // Two wavefronts per workgroup: a decode token of the 8B shape (320 rotation +
-  // 128 value vectors) spreads over four workgroups. 64 and 256 lanes measured
-  // within +-5 % of this from 6 MiB to 324 MiB per launch.
+  // Lanes per workgroup, from graph-timed sweeps (64 to 8192 tokens): the plain
+  // rotation runs the same with 64 or 128 lanes and slower with 256; with the
+  // cache write fused in, one wavefront per workgroup is 3-9 % faster than two
+  // (the barrier then costs nothing, and a workgroup whose slot chain is late
+  // holds back fewer lanes).
   unsigned threads = (unsigned)kvc::g_rope_tune.threads;
-  if (threads != 64 && threads != 128 && threads != 256) threads = 128;
+  if (threads != 64 && threads != 128 && threads != 256) threads = c ? 64 : 128;
   a.groups_per_token = (uint32_t)std::max<int64_t>(1, (items + threads - 1) / threads);
   if (g.num_tokens * (int64_t)a.groups_per_token > 0x7fffffffll)
     return fail(KVC_ERR_UNSUPPORTED, "%s: launch of %lld workgroups is too large", fn,
