@@ -55,7 +55,7 @@ using kvc::fail;
 // tuning knobs (kvc_set_tuning); defaults are the measured best on MI355X
 // ---------------------------------------------------------------------------
 struct Tuning {
-  int copy_unroll = 4;      // 16-byte vectors in flight per lane in copy_tiles
+  int copy_unroll = 0;      // 16-byte vectors in flight per lane in copy_tiles, 0 = by size
   int gather_unroll = 1;    // the same for pool -> dense buffer (dense writes measured best
                             // with 4 KiB per workgroup: 6.27 vs 5.68 TB/s at 4 vectors)
   int copy_nt = 1;          // non-temporal loads/stores in copy_tiles
@@ -623,6 +623,23 @@ void launch_tiles_nt(const TileArgs& a, unsigned grid, hipStream_t s, bool nt) {
 
 template <int VEC>
 int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt, int64_t n) {
+  if (unroll <= 0) {
+    // By size, from sweeps of copy_blocks (1 to 4096 pairs x 32 layers x 64 KiB):
+    // a launch that fits a quarter of the resident workgroups runs best as few,
+    // deep workgroups (the smallest depth that gets it there; up to a whole tile
+    // per workgroup while that stays within half the resident set): 6-8 % faster
+    // than 4 vectors per lane from 32 to 128 MiB. Larger launches stream best
+    // with 2 vectors per lane.
+    const int64_t resident = resident_workgroups();
+    const auto chunks = [&](int u) {
+      const int64_t c = (int64_t)kThreads * VEC * u;
+      return n * (int64_t)a.num_layers * ((a.tile_bytes + c - 1) / c);
+    };
+    unroll = 0;
+    for (int u = 1; u <= 16 && !unroll; u *= 2)
+      if (chunks(u) <= resident / 4) unroll = u;
+    if (!unroll) unroll = chunks(16) <= resident / 2 ? 16 : 2;
+  }
   // do not carry more vectors per lane than the tile can fill
   while (unroll > 1 && (int64_t)kThreads * VEC * (unroll / 2) >= a.tile_bytes) unroll /= 2;
   const int64_t chunk = (int64_t)kThreads * VEC * unroll;
@@ -651,7 +668,7 @@ int launch_tiles(const TileArgs& a, int64_t n, int max_wgs, hipStream_t s, int u
                               (uint64_t)a.dst_layer_stride, (uint64_t)a.dst_block_stride,
                               (uint64_t)a.tile_bytes});
   if (unroll <= 0) unroll = g_tune.copy_unroll;
-  if (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8 && unroll != 16) unroll = 4;
+  if (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8 && unroll != 16) unroll = 0;  // by size
   const bool nt = g_tune.copy_nt != 0;
   switch (vec) {
     case 16: return launch_tiles_vec<16>(a, unroll, max_wgs, s, nt, n);
