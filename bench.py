@@ -38,10 +38,10 @@ ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 
 # HBM bytes per launch of the headline kernel (config 2, all layers in one launch)
 # from two rocprofv3 --pmc runs: FETCH_SIZE 16438.9 KiB x 2.0000 + WRITE_SIZE
-# 32822.5 KiB x 1.0000, the factors being what the same counters read for a
+# 32810.8 KiB x 1.0000, the factors being what the same counters read for a
 # plain elementwise kernel of known size (1 GiB read, 1 GiB written); summary in
 # profiles/hbm_traffic_fetch_size_write_size.txt. Only valid for the default workload.
-MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67276317
+MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67264347
 
 
 def log(*a):
