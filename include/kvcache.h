@@ -62,7 +62,7 @@ const char* kvc_last_error_string(void);
 /* Launch-shape knobs for measurement sweeps; process-wide, not thread-safe
  * against concurrent launches. No counterpart in the reference. Keys:
  *   "copy_unroll", "gather_unroll"   16-byte vectors per lane in the tile kernel (1, 2, 4, 8, 16;
- *                                     copy_unroll 0 = by launch size)
+ *                                     0 = by launch size)
  *   "copy_nt"                         non-temporal loads and stores in the tile kernel (0/1)
  *   "copy_order"                      1 = walk all blocks of a layer before the next layer
  *   "copy_max_wgs"                    grid cap of the tile kernel (0 = one workgroup per chunk)

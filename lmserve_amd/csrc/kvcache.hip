@@ -56,8 +56,8 @@ using kvc::fail;
 // ---------------------------------------------------------------------------
 struct Tuning {
   int copy_unroll = 0;      // 16-byte vectors in flight per lane in copy_tiles, 0 = by size
-  int gather_unroll = 1;    // the same for pool -> dense buffer (dense writes measured best
-                            // with 4 KiB per workgroup: 6.27 vs 5.68 TB/s at 4 vectors)
+  int gather_unroll = 0;    // the same for pool -> dense buffer; by size, 1 for large launches (dense
+                            // writes measured best with 4 KiB per workgroup: 6.27 vs 5.68 TB/s at 4)
   int copy_nt = 1;          // non-temporal loads/stores in copy_tiles
   int copy_max_wgs = 0;     // 0 = one workgroup per chunk, else grid cap
   int copy_order = 0;       // copy_tiles: 1 = walk all blocks of a layer before the next layer
@@ -622,14 +622,15 @@ void launch_tiles_nt(const TileArgs& a, unsigned grid, hipStream_t s, bool nt) {
 }
 
 template <int VEC>
-int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt, int64_t n) {
+int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt, int64_t n, int large) {
   if (unroll <= 0) {
     // By size, from sweeps of copy_blocks (1 to 4096 pairs x 32 layers x 64 KiB):
     // a launch that fits a quarter of the resident workgroups runs best as few,
     // deep workgroups (the smallest depth that gets it there; up to a whole tile
     // per workgroup while that stays within half the resident set): 6-8 % faster
-    // than 4 vectors per lane from 32 to 128 MiB. Larger launches stream best
-    // with 2 vectors per lane.
+    // than 4 vectors per lane from 32 to 128 MiB (a gather: 12-15 % faster than
+    // with 1). Larger launches stream best with `large` vectors per lane: 2, or 1
+    // when the scattered side is the one being read (gather).
     const int64_t resident = resident_workgroups();
     const auto chunks = [&](int u) {
       const int64_t c = (int64_t)kThreads * VEC * u;
@@ -638,7 +639,7 @@ int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt
     unroll = 0;
     for (int u = 1; u <= 16 && !unroll; u *= 2)
       if (chunks(u) <= resident / 4) unroll = u;
-    if (!unroll) unroll = chunks(16) <= resident / 2 ? 16 : 2;
+    if (!unroll) unroll = chunks(16) <= resident / 2 ? 16 : large;
   }
   // do not carry more vectors per lane than the tile can fill
   while (unroll > 1 && (int64_t)kThreads * VEC * (unroll / 2) >= a.tile_bytes) unroll /= 2;
@@ -661,21 +662,22 @@ int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt
   return KVC_OK;
 }
 
-int launch_tiles(const TileArgs& a, int64_t n, int max_wgs, hipStream_t s, int unroll = 0) {
+// unroll > 0: fixed; 0: the copy_unroll knob (by size unless set); gather: the gather_unroll knob
+int launch_tiles(const TileArgs& a, int64_t n, int max_wgs, hipStream_t s, bool gather = false) {
   if (n == 0 || a.num_layers == 0 || a.tile_bytes == 0) return KVC_OK;
   const int vec = common_vec({(uint64_t)(uintptr_t)a.src_base, (uint64_t)(uintptr_t)a.dst_base,
                               (uint64_t)a.src_layer_stride, (uint64_t)a.src_block_stride,
                               (uint64_t)a.dst_layer_stride, (uint64_t)a.dst_block_stride,
                               (uint64_t)a.tile_bytes});
-  if (unroll <= 0) unroll = g_tune.copy_unroll;
+  int unroll = gather ? g_tune.gather_unroll : g_tune.copy_unroll;
   if (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8 && unroll != 16) unroll = 0;  // by size
   const bool nt = g_tune.copy_nt != 0;
   switch (vec) {
-    case 16: return launch_tiles_vec<16>(a, unroll, max_wgs, s, nt, n);
-    case 8: return launch_tiles_vec<8>(a, unroll, max_wgs, s, nt, n);
-    case 4: return launch_tiles_vec<4>(a, unroll, max_wgs, s, nt, n);
-    case 2: return launch_tiles_vec<2>(a, unroll, max_wgs, s, nt, n);
-    default: return launch_tiles_vec<1>(a, unroll, max_wgs, s, nt, n);
+    case 16: return launch_tiles_vec<16>(a, unroll, max_wgs, s, nt, n, gather ? 1 : 2);
+    case 8: return launch_tiles_vec<8>(a, unroll, max_wgs, s, nt, n, gather ? 1 : 2);
+    case 4: return launch_tiles_vec<4>(a, unroll, max_wgs, s, nt, n, gather ? 1 : 2);
+    case 2: return launch_tiles_vec<2>(a, unroll, max_wgs, s, nt, n, gather ? 1 : 2);
+    default: return launch_tiles_vec<1>(a, unroll, max_wgs, s, nt, n, gather ? 1 : 2);
   }
 }
 
@@ -893,7 +895,7 @@ int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_
       t.dst_base = slot; t.dst_ids = nullptr;
       t.dst_layer_stride = g.block_bytes; t.dst_block_stride = width;
       t.num_dst_blocks = count;
-      rc = launch_tiles(t, count, g_tune.copy_max_wgs, ks, g_tune.gather_unroll);
+      rc = launch_tiles(t, count, g_tune.copy_max_wgs, ks, true);
       if (rc != KVC_OK) return rc;
       if (two_streams) {
         KVC_HIP(hipEventRecord(c.filled[sl], ks));
@@ -1152,7 +1154,7 @@ static int run_gather_scatter(const char* fn, bool gather, char* pool, char* buf
     t.dst_layer_stride = layer_stride_bytes; t.dst_block_stride = block_bytes;
     t.num_dst_blocks = num_blocks;
   }
-  return launch_tiles(t, n, g_tune.copy_max_wgs, (hipStream_t)stream, gather ? g_tune.gather_unroll : 0);
+  return launch_tiles(t, n, g_tune.copy_max_wgs, (hipStream_t)stream, gather);
 }
 
 int kvc_gather_blocks(const void* pool, void* buffer, const int64_t* block_ids, int64_t n,
