@@ -113,3 +113,28 @@ def test_copy_blocks_skips_out_of_range_ids_on_the_device(gpu):
     kvc.copy_blocks(dpool, maps)
     torch.cuda.synchronize()
     assert np.array_equal(bits_of(dpool), want)
+
+
+@pytest.mark.parametrize("n", [1, 2, 4, 8, 16, 32, 100])
+def test_every_launch_shape_the_size_rule_picks_matches_the_oracle(gpu, n):
+    """Bytes per workgroup follow the launch size (1, 2, 4, 8 or 16 vectors per lane
+    for small launches, 2 or 1 for large ones): copy, gather and scatter at sizes
+    that reach each choice, Llama-3-8B block shape over 32 layers."""
+    s = wl.LLAMA_3_8B
+    L, nb = 32, 256
+    pool = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), seed=n)
+    flat, pairs = wl.copy_on_write_pairs(nb, n, seed=n)
+    want = pool.copy()
+    orc.c_copy_blocks(want, flat)
+    dpool = to_bf16(pool, gpu)
+    kvc.copy_blocks(dpool, pairs)
+    ids = torch.from_numpy(flat[1::2].copy()).to(gpu)               # the blocks just written
+    dense = kvc.gather_blocks(dpool, ids)
+    back = torch.from_numpy(flat[0::2].copy()).to(gpu)              # scatter them over their sources
+    kvc.scatter_blocks(dpool, back, dense)
+    torch.cuda.synchronize()
+    view = want.reshape(L, nb, -1)
+    want_dense = view[:, flat[1::2]].swapaxes(0, 1)
+    assert np.array_equal(bits_of(dense), want_dense)
+    view[:, flat[0::2]] = want_dense.swapaxes(0, 1)                 # a no-op by value: dst == src content
+    assert np.array_equal(bits_of(dpool), want)
