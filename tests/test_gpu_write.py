@@ -285,3 +285,33 @@ def test_dtype_mismatch_raises(gpu):
                                   torch.zeros(2, dtype=torch.int32, device=gpu),
                                   torch.zeros(2, dtype=torch.int32, device=gpu),
                                   torch.zeros(1, dtype=torch.int32, device=gpu))
+
+
+@pytest.mark.parametrize("T", [40, 64, 100, 128, 200, 256, 300])
+@pytest.mark.parametrize("paged", [False, True])
+def test_one_launch_write_through_every_shape_the_size_rule_picks(gpu, T, paged):
+    """32 layers of the Llama-3-8B row in one launch, at token counts on both sides
+    of each switch of the launch-shape rule (256 lanes x 1 vector; 128 lanes x 2;
+    128 lanes x 4; back to 256 x 1), slot-mapped and page-table addressed."""
+    s = wl.LLAMA_3_8B
+    L, nb, bs = 32, 96, s.block_size
+    w = wl.decode_step(s, num_blocks=nb, batch=T, max_context=4, seed=T) if T <= nb else \
+        wl.chunked_prefill(s, num_blocks=nb, num_seqs=4, chunk_tokens=T - T % 4, min_context=1,
+                           max_context=40, seed=T)
+    idx = w.index
+    n = w.num_tokens
+    key, value = bf16_bits((L, n, s.num_kv_heads, s.head_dim), T), bf16_bits((L, n, s.num_kv_heads, s.head_dim), T + 1)
+    pool = sentinel_pool((L, nb, 2, bs, s.num_kv_heads, s.head_dim), T + 2)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_reshape_and_cache(key[l], value[l], want[l], idx.slot_mapping)
+    dev = kvc.to_device(idx, bs, gpu)
+    dpool = to_bf16(pool, gpu)
+    if paged:
+        kvc.append_paged_kv_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dev.batch_indices,
+                                         dev.positions, dpool, dev.kv_block_indices,
+                                         dev.kv_block_indptrs, dev.kv_last_block_lens)
+    else:
+        kvc.reshape_and_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool, dev.slot_mapping)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), want)
