@@ -13,7 +13,7 @@
  *   - asynchronous on the given stream(s) unless the name ends in _sync;
  *   - never allocates or frees device memory; the caller owns every buffer
  *     (host-side helpers own small pinned bounce buffers, events and, in the
- *     disk tier, per-thread staging);
+ *     disk tier, per-thread staging; kvc_thread_release returns the swap's);
  *   - every offset is computed in 64 bits (one layer of a 65536-block Llama-3-8B
  *     pool already holds 2^31 elements);
  *   - block ids / slots outside [0, capacity) are skipped by the kernels
@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define KVC_ABI_VERSION 1
+#define KVC_ABI_VERSION 2
 
 typedef enum kvc_status {
   KVC_OK = 0,
@@ -71,10 +71,36 @@ const char* kvc_last_error_string(void);
  *   "write_threads"                   lanes per workgroup in the write kernel (0 = by size, 64, 128, 256)
  *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads
  *   "write_order"                     1 = a token's workgroups are neighbours in the grid
+ *   "write_narrow"                    rows under 1 KiB take the kernel whose lanes run over
+ *                                     consecutive tokens of one (layer, K|V) plane (0/1)
+ *   "write_narrow_vpt"                planes per lane in that kernel (0 = by size, 1, 2, 4, 8)
  *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
  *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier
- * Unknown key: KVC_ERR_INVALID_ARG. */
+ * Unknown key: KVC_ERR_INVALID_ARG. kvc_reset_tuning puts every knob back to its
+ * default; kvc_tuning_modified counts the knobs that are not at their default. */
 int kvc_set_tuning(const char* key, int value);
+int kvc_get_tuning(const char* key, int* value);
+int kvc_reset_tuning(void);
+int kvc_tuning_modified(void);
+
+/* Shape of the most recent kernel launch made by the calling thread (for tests
+ * and sweeps that must know which instantiation ran). No counterpart in the
+ * reference. Unknown `what`: KVC_ERR_INVALID_ARG. */
+enum {
+  KVC_KERNEL_NONE = 0,
+  KVC_KERNEL_WRITE_ROWS = 1,        /* token per workgroup                          */
+  KVC_KERNEL_COPY_TILES = 2,        /* block copy, gather, scatter, direct swap     */
+  KVC_KERNEL_WRITE_ROWS_NARROW = 3  /* rows under 1 KiB: lanes over tokens of a plane */
+};
+enum {
+  KVC_LAUNCH_KERNEL = 0,       /* one of KVC_KERNEL_*                               */
+  KVC_LAUNCH_VEC_BYTES = 1,    /* bytes per load/store instruction per lane         */
+  KVC_LAUNCH_PER_LANE = 2,     /* vectors (or planes) in flight per lane            */
+  KVC_LAUNCH_THREADS = 3,      /* lanes per workgroup                               */
+  KVC_LAUNCH_GRID = 4,         /* workgroups                                        */
+  KVC_LAUNCH_NON_TEMPORAL = 5  /* bit 0 stores, bit 1 loads (tile kernel: both = 1) */
+};
+int64_t kvc_last_launch_info(int what);
 
 /* ---------------------------------------------------------------------------
  * K/V write, slot-mapped.
@@ -159,6 +185,32 @@ int kvc_append_paged_kv_cache_layers(const void* append_key, const void* append_
                                      int64_t num_layers, int64_t key_layer_stride,
                                      int64_t value_layer_stride, int64_t cache_layer_stride,
                                      int elem_bytes, void* stream);
+
+/* The page-table write with its per-step arguments held by the library, so a
+ * layer-by-layer forward pass hands over three pointers per layer instead of
+ * twenty arguments. The reference builds the same five index tensors once per
+ * step (runtime/worker/llm_worker/model_worker.py:399-446) and passes them to
+ * every layer's append call (runtime/worker/llm_worker/models/llama.py:236-242,
+ * runtime/worker/llm_worker/models/layers/attention.py:76-85).
+ * kvc_write_plan_create copies the ARGUMENTS (pointers and sizes), not the
+ * arrays: the index arrays must stay valid on the device for as long as the
+ * plan is used. kvc_write_plan_append is kvc_append_paged_kv_cache with the
+ * plan's arguments and the layer's key, value (token strides in elements) and
+ * cache; same checks, same errors. Host-side object: create/destroy touch
+ * no device memory. */
+typedef struct kvc_write_plan kvc_write_plan;
+
+int kvc_write_plan_create(const int32_t* batch_indices, const int32_t* positions,
+                          const int32_t* kv_indices, const int32_t* kv_indptr,
+                          const int32_t* kv_last_page_len,
+                          int64_t nnz, int64_t batch_size, int64_t num_kv_indices,
+                          int64_t num_kv_heads, int64_t head_dim, int64_t page_size,
+                          int elem_bytes, kvc_write_plan** out);
+int kvc_write_plan_append(const kvc_write_plan* plan, const void* append_key,
+                          const void* append_value, int64_t key_token_stride,
+                          int64_t value_token_stride, void* paged_kv_cache,
+                          int64_t page_stride, int64_t num_pages, void* stream);
+int kvc_write_plan_destroy(kvc_write_plan* plan);
 
 /* ---------------------------------------------------------------------------
  * Index preparation for the paged write.
@@ -259,6 +311,44 @@ int kvc_swap_in(void* pool, const void* host_pool,
                 void* staging, int64_t staging_bytes, int mode,
                 void* kernel_stream, void* copy_stream);
 
+/* The id lists of a swap checked and uploaded ONCE, for callers that move the
+ * same blocks in several calls -- the reference's layer loops issue one call per
+ * layer with the same mappings (runtime/worker/llm_worker/kv_worker.py:249-295).
+ *   kvc_swap_prepare: range-checks gpu_ids against num_gpu_blocks and host_ids
+ *     against num_host_blocks (HOST int64 arrays of n entries) and uploads
+ *     [gpu_ids | host_ids] to the head of `staging` on `stream`.
+ *   kvc_swap_out_prepared / kvc_swap_in_prepared: kvc_swap_out / kvc_swap_in for a
+ *     layer range with the id lists read from the head of `staging` as
+ *     kvc_swap_prepare left them (gpu ids are the sources of a swap-out and the
+ *     destinations of a swap-in). Neither checks nor uploads anything; in
+ *     KVC_SWAP_DIRECT mode the call is one kernel launch and host_ids may be
+ *     NULL; KVC_SWAP_STAGED still needs the HOST array host_ids for its PCIe
+ *     extents. The caller orders these calls after the prepare call (same
+ *     stream, or an event) and keeps `staging` untouched in between.
+ * kvc_thread_release frees what the swap entry points keep per calling thread
+ * (events, pinned id bounce buffers); it waits for that thread's pending id
+ * uploads. Optional: a thread that never calls it keeps a few KiB of pinned
+ * memory until the process ends. */
+int kvc_swap_prepare(const int64_t* gpu_ids, const int64_t* host_ids, int64_t n,
+                     int64_t num_gpu_blocks, int64_t num_host_blocks,
+                     void* staging, int64_t staging_bytes, void* stream);
+
+int kvc_swap_out_prepared(const void* pool, void* host_pool, const int64_t* host_ids, int64_t n,
+                          int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                          int64_t num_gpu_blocks, int64_t num_host_blocks,
+                          int64_t layer_begin, int64_t layer_end,
+                          void* staging, int64_t staging_bytes, int mode,
+                          void* kernel_stream, void* copy_stream);
+
+int kvc_swap_in_prepared(void* pool, const void* host_pool, const int64_t* host_ids, int64_t n,
+                         int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                         int64_t num_gpu_blocks, int64_t num_host_blocks,
+                         int64_t layer_begin, int64_t layer_end,
+                         void* staging, int64_t staging_bytes, int mode,
+                         void* kernel_stream, void* copy_stream);
+
+int kvc_thread_release(void);
+
 /* ---------------------------------------------------------------------------
  * Rotary position embedding, alone or fused with the K/V write.
  * (Widening beyond the copy path: the rotation runs immediately before the
@@ -318,6 +408,30 @@ int kvc_rotary_pos_emb_and_append_paged(const void* query, const void* key, cons
                                         int64_t num_kv_indices, int64_t page_size,
                                         int64_t page_stride, int64_t num_pages, int dtype,
                                         void* stream);
+
+/* kvc_rotary_pos_emb_and_append_paged with its per-step arguments held by the
+ * library (see kvc_write_plan): per layer the caller hands over the layer's
+ * query/key/value with their token strides in elements (slices of a fused QKV
+ * projection are read in place), the output buffers (dense rows: query_out
+ * stride = num_heads*head_dim, key_out stride = num_kv_heads*head_dim; key_out
+ * may be NULL) and the layer's cache. The reference calls the rotation
+ * and the append once per layer with the same positions and index tensors
+ * (runtime/worker/llm_worker/models/llama.py:156-167, :236-242). */
+typedef struct kvc_rotary_plan kvc_rotary_plan;
+
+int kvc_rotary_plan_create(const int32_t* batch_indices, const int32_t* positions,
+                           const void* cos_sin_cache, int64_t max_position, int64_t nnz,
+                           int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                           int64_t rotary_dim, const int32_t* kv_indices,
+                           const int32_t* kv_indptr, int64_t batch_size,
+                           int64_t num_kv_indices, int64_t page_size, int dtype,
+                           kvc_rotary_plan** out);
+int kvc_rotary_plan_run(const kvc_rotary_plan* plan, const void* query, const void* key,
+                        const void* value, int64_t q_token_stride, int64_t k_token_stride,
+                        int64_t v_token_stride, void* query_out, void* key_out,
+                        void* paged_kv_cache, int64_t page_stride, int64_t num_pages,
+                        void* stream);
+int kvc_rotary_plan_destroy(kvc_rotary_plan* plan);
 
 /* The on-device half of a swap on its own: gather scattered pool blocks into a
  * dense device buffer laid out like the host pool, [n, layer_end-layer_begin,

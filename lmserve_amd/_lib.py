@@ -33,6 +33,19 @@ KVC_DISK_INFO_BOUNCED = 5
 KVC_SWAP_STAGED = 0
 KVC_SWAP_DIRECT = 1
 
+KVC_KERNEL_NONE = 0
+KVC_KERNEL_WRITE_ROWS = 1
+KVC_KERNEL_COPY_TILES = 2
+KVC_KERNEL_WRITE_ROWS_NARROW = 3
+KVC_LAUNCH_KERNEL = 0
+KVC_LAUNCH_VEC_BYTES = 1
+KVC_LAUNCH_PER_LANE = 2
+KVC_LAUNCH_THREADS = 3
+KVC_LAUNCH_GRID = 4
+KVC_LAUNCH_NON_TEMPORAL = 5
+
+KVC_ABI_VERSION = 2
+
 KVC_DTYPE_BF16 = 0
 KVC_DTYPE_F16 = 1
 KVC_DTYPE_F32 = 2
@@ -45,6 +58,24 @@ SIGNATURES = {
     "kvc_abi_version": (c_int, []),
     "kvc_last_error_string": (c_char_p, []),
     "kvc_set_tuning": (c_int, [c_char_p, c_int]),
+    "kvc_get_tuning": (c_int, [c_char_p, ctypes.POINTER(c_int)]),
+    "kvc_reset_tuning": (c_int, []),
+    "kvc_tuning_modified": (c_int, []),
+    "kvc_last_launch_info": (_I64, [c_int]),
+    "kvc_write_plan_create": (c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, c_int,
+                                      ctypes.POINTER(_P)]),
+    "kvc_write_plan_append": (c_int, [_P, _P, _P, _I64, _I64, _P, _I64, _I64, _P]),
+    "kvc_write_plan_destroy": (c_int, [_P]),
+    "kvc_rotary_plan_create": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _I64,
+                                       _I64, _I64, c_int, ctypes.POINTER(_P)]),
+    "kvc_rotary_plan_run": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P, _I64, _I64, _P]),
+    "kvc_rotary_plan_destroy": (c_int, [_P]),
+    "kvc_swap_prepare": (c_int, [_P, _P, _I64, _I64, _I64, _P, _I64, _P]),
+    "kvc_swap_out_prepared": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
+                                      _I64, c_int, _P, _P]),
+    "kvc_swap_in_prepared": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
+                                     _I64, c_int, _P, _P]),
+    "kvc_thread_release": (c_int, []),
     "kvc_reshape_and_cache": (c_int, [_P, _P, _P, _P, _P, c_int, _I64, _I64, _I64, _I64, _I64,
                                       _I64, _I64, _I64, c_int, _P]),
     "kvc_reshape_and_cache_layers": (c_int, [_P, _P, _P, _P, _P, c_int, _I64, _I64, _I64, _I64,
@@ -103,6 +134,11 @@ def lib() -> ctypes.CDLL:
             f"{LIB_PATH} is not built; run `python -m lmserve_amd.build` (needs hipcc). "
             "There is no CPU fallback for the KV-cache operators.")
     handle = ctypes.CDLL(LIB_PATH)
+    handle.kvc_abi_version.restype = c_int
+    if handle.kvc_abi_version() != KVC_ABI_VERSION:
+        raise KVCacheLibraryError(
+            f"{LIB_PATH} has ABI version {handle.kvc_abi_version()}, this package needs "
+            f"{KVC_ABI_VERSION}: rebuild it with `python -m lmserve_amd.build`")
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(handle, name)
         fn.restype = restype
@@ -133,3 +169,24 @@ def check(rc: int) -> None:
 
 def set_tuning(key: str, value: int) -> None:
     check(lib().kvc_set_tuning(key.encode(), int(value)))
+
+
+def get_tuning(key: str) -> int:
+    out = c_int(0)
+    check(lib().kvc_get_tuning(key.encode(), ctypes.byref(out)))
+    return out.value
+
+
+def reset_tuning() -> None:
+    check(lib().kvc_reset_tuning())
+
+
+def last_launch() -> dict:
+    """Shape of the calling thread's most recent kernel launch."""
+    L = lib()
+    return {"kernel": L.kvc_last_launch_info(KVC_LAUNCH_KERNEL),
+            "vec_bytes": L.kvc_last_launch_info(KVC_LAUNCH_VEC_BYTES),
+            "per_lane": L.kvc_last_launch_info(KVC_LAUNCH_PER_LANE),
+            "threads": L.kvc_last_launch_info(KVC_LAUNCH_THREADS),
+            "grid": L.kvc_last_launch_info(KVC_LAUNCH_GRID),
+            "non_temporal": L.kvc_last_launch_info(KVC_LAUNCH_NON_TEMPORAL)}

@@ -48,10 +48,30 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
-def ensure_built() -> None:
-    """For tests, the smoke check and the benchmark: use what is built, build
-    only what is missing. The operators themselves never build anything."""
+HEADERS = [os.path.join(PKG_DIR, "csrc", "common.h"), os.path.join(INCLUDE, "kvcache.h")]
+
+
+def is_stale() -> bool:
+    """True when the library is missing or older than one of its sources."""
     if not os.path.exists(LIB_PATH):
+        return True
+    built = os.path.getmtime(LIB_PATH)
+    return any(os.path.exists(f) and os.path.getmtime(f) > built for f in SOURCES + HEADERS)
+
+
+def ensure_built() -> None:
+    """For tests, the smoke check and the benchmark: use what is built; compile
+    when the library is missing, or older than its sources and a compiler is at
+    hand. The operators themselves never build anything."""
+    if not os.path.exists(LIB_PATH):
+        build(verbose=True)
+    elif is_stale():
+        try:
+            find_hipcc()
+        except RuntimeError:
+            print(f"warning: {LIB_PATH} is older than its sources and no hipcc was found",
+                  file=sys.stderr, flush=True)
+            return
         build(verbose=True)
 
 

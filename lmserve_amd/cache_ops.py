@@ -142,10 +142,12 @@ def _rows(t: torch.Tensor, name: str):
     if t.dim() != 3:
         raise ValueError(f"{name} must be [num_tokens, num_kv_heads, head_size]")
     T, H, D = t.shape
-    if T > 0 and H * D > 0 and (t.stride(2) != 1 or (H > 1 and t.stride(1) != D)):
+    if T > 0 and H * D > 0 and (t.stride(2) != 1 or (H > 1 and t.stride(1) != D)
+                                or (T > 1 and t.stride(0) < H * D)):
+        # rows that are not dense, or that overlap (an expanded or as_strided view)
         t = t.contiguous()
     stride = t.stride(0) if T > 1 else H * D
-    return t, H * D, max(stride, H * D)
+    return t, H * D, stride
 
 
 def fill_key_cache(

@@ -28,7 +28,9 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <new>
 
 #include "common.h"
 #include "kvcache.h"
@@ -65,10 +67,53 @@ struct Tuning {
   int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
   int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
+  int write_narrow = 1;     // rows under 1 KiB: lanes of a wavefront run over consecutive tokens of
+                            // one (layer, K|V) plane instead of over one token's planes
+  int write_narrow_vpt = 0; // planes per lane in that kernel (1, 2, 4, 8), 0 = by size
   int direct_max_wgs = 64;  // grid cap of the direct swap kernel: PCIe saturates with a few
                             // dozen workgroups, the rest of the GPU stays free for the model
 };
 Tuning g_tune;
+
+// name -> knob, for kvc_set_tuning / kvc_get_tuning / kvc_reset_tuning
+struct Knob {
+  const char* name;
+  int* value;
+  int initial;
+};
+Knob* knobs(int* count) {
+  static Knob table[] = {
+      {"copy_unroll", &g_tune.copy_unroll, 0},
+      {"gather_unroll", &g_tune.gather_unroll, 0},
+      {"copy_nt", &g_tune.copy_nt, 1},
+      {"copy_max_wgs", &g_tune.copy_max_wgs, 0},
+      {"copy_order", &g_tune.copy_order, 0},
+      {"write_vpt", &g_tune.write_vpt, 0},
+      {"write_nt", &g_tune.write_nt, 1},
+      {"write_order", &g_tune.write_order, 0},
+      {"write_threads", &g_tune.write_threads, 0},
+      {"write_narrow", &g_tune.write_narrow, 1},
+      {"write_narrow_vpt", &g_tune.write_narrow_vpt, 0},
+      {"direct_max_wgs", &g_tune.direct_max_wgs, 64},
+      {"rope_threads", &kvc::g_rope_tune.threads, 0},
+      {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
+  };
+  *count = (int)(sizeof(table) / sizeof(table[0]));
+  return table;
+}
+Knob* find_knob(const char* key) {
+  int n = 0;
+  Knob* t = knobs(&n);
+  for (int i = 0; i < n; ++i)
+    if (!strcmp(key, t[i].name)) return &t[i];
+  return nullptr;
+}
+
+// What the most recent kernel launch of this thread looked like (kvc_last_launch_info).
+struct LastLaunch {
+  int64_t kernel = KVC_KERNEL_NONE, vec = 0, per_lane = 0, threads = 0, grid = 0, nt = 0;
+};
+thread_local LastLaunch g_last;
 
 constexpr int kThreads = 256;
 
@@ -124,6 +169,10 @@ struct WriteArgs {
   int bs_shift;              // log2(block_size) or -1
   int64_t cache_block_stride, cache_slot_stride, cache_layer_stride;
   int64_t num_cache_blocks;
+  // narrow-row kernel only
+  uint32_t num_planes;        // 2 * num_layers; plane = (layer, K|V)
+  uint32_t tokens_per_wg;     // blockDim.x / vecs_per_row
+  uint32_t num_token_groups;  // ceil(num_tokens / tokens_per_wg)
 };
 
 // One workgroup = one token x a run of VPT*blockDim.x vectors out of the
@@ -215,6 +264,79 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   for (int j = 0; j < VPT; ++j) {
     if (dst_off[j] >= 0)
       st<NT>(reinterpret_cast<V*>((to_v[j] ? vc_row : kc_row) + dst_off[j]), data[j]);
+  }
+}
+
+// Rows shorter than the 1 KiB a wavefront moves per instruction (one KV head of a
+// tensor-parallel shard: 256-byte rows). With a token per workgroup a wavefront
+// would span several rows of several layers and neither side would be one run.
+// Here the lanes of a workgroup run over consecutive TOKENS of one (layer, K|V)
+// plane: the source side is one contiguous run of blockDim.x * 16 bytes, the
+// cache side one row per token. Each lane looks up its own token's slot (lanes
+// of one row read the same index words) and reuses it for its VPT planes, whose
+// loads are all issued before the lookup. 16-byte vectors and a power-of-two
+// number of them per row only; blockIdx.x = plane_group * num_token_groups +
+// token_group.
+template <int VPT, bool PAGED, bool NT>
+__global__ __launch_bounds__(kThreads) void write_rows_narrow_kernel(WriteArgs a) {
+  using V = u32x4;
+  const uint32_t pg = blockIdx.x / a.num_token_groups;
+  const uint32_t tg = blockIdx.x - pg * a.num_token_groups;
+  const uint32_t t = tg * a.tokens_per_wg + (threadIdx.x >> a.vpr_shift);
+  if (t >= a.num_tokens) return;
+  const int64_t vec_off = (int64_t)(threadIdx.x & (a.vecs_per_row - 1u)) * 16;
+  const char* key_row = a.key + (int64_t)t * a.key_token_stride + vec_off;
+  const char* value_row = a.value + (int64_t)t * a.value_token_stride + vec_off;
+  V data[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const uint32_t plane = pg * VPT + j;
+    if (plane < a.num_planes) {
+      const int64_t layer = plane >> 1;
+      const char* src = (plane & 1u) ? value_row + layer * a.value_layer_stride
+                                     : key_row + layer * a.key_layer_stride;
+      data[j] = *reinterpret_cast<const V*>(src);
+    }
+  }
+  int64_t blk, off;
+  if constexpr (PAGED) {
+    const int64_t b = a.batch_indices[t];
+    const int64_t p = a.positions[t];
+    if (b < 0 || b >= a.batch_size || p < 0) return;
+    int64_t pgi;
+    if (a.bs_shift >= 0) {
+      pgi = p >> a.bs_shift;
+      off = p & (a.block_size - 1);
+    } else {
+      pgi = p / a.block_size;
+      off = p - pgi * a.block_size;
+    }
+    const int64_t it = (int64_t)a.kv_indptr[b] + pgi;
+    if (it < 0 || it >= (int64_t)a.kv_indptr[b + 1] || it >= a.num_kv_indices) return;
+    blk = a.kv_indices[it];
+  } else {
+    const int64_t s = (a.slot_bytes == 8)
+                          ? reinterpret_cast<const int64_t*>(a.slot_mapping)[t]
+                          : (int64_t) reinterpret_cast<const int32_t*>(a.slot_mapping)[t];
+    if (s < 0) return;
+    if (a.bs_shift >= 0) {
+      blk = s >> a.bs_shift;
+      off = s & (a.block_size - 1);
+    } else {
+      blk = s / a.block_size;
+      off = s - blk * a.block_size;
+    }
+  }
+  if (blk < 0 || blk >= a.num_cache_blocks) return;
+  const int64_t slot_off = blk * a.cache_block_stride + off * a.cache_slot_stride + vec_off;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const uint32_t plane = pg * VPT + j;
+    if (plane < a.num_planes) {
+      char* dst = ((plane & 1u) ? a.value_cache : a.key_cache) + slot_off +
+                  (int64_t)(plane >> 1) * a.cache_layer_stride;
+      st<NT>(reinterpret_cast<V*>(dst), data[j]);
+    }
   }
 }
 
@@ -462,6 +584,23 @@ void launch_write(const WriteArgs& a, int vec, const WriteLaunch& l, hipStream_t
   }
 }
 
+template <int VPT, bool PAGED>
+void launch_narrow_nt(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
+  const dim3 grid(l.grid), block(l.threads);
+  if (l.nt) hipLaunchKernelGGL((write_rows_narrow_kernel<VPT, PAGED, true>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((write_rows_narrow_kernel<VPT, PAGED, false>), grid, block, 0, s, a);
+}
+
+template <bool PAGED>
+void launch_narrow(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
+  switch (l.vpt) {
+    case 1: launch_narrow_nt<1, PAGED>(a, l, s); break;
+    case 2: launch_narrow_nt<2, PAGED>(a, l, s); break;
+    case 4: launch_narrow_nt<4, PAGED>(a, l, s); break;
+    default: launch_narrow_nt<8, PAGED>(a, l, s); break;
+  }
+}
+
 struct WriteGeom {
   int64_t num_tokens, row_elems;
   int64_t key_token_stride, value_token_stride;       // elements
@@ -489,7 +628,7 @@ int check_write_geom(const char* fn, const void* key, const void* value, const v
   if (g.cache_slot_stride < g.row_elems || g.cache_block_stride < 0 || g.cache_layer_stride < 0 ||
       g.key_layer_stride < 0 || g.value_layer_stride < 0)
     return fail(KVC_ERR_INVALID_ARG, "%s: bad cache/layer stride", fn);
-  if (g.num_layers * 2 > 65535)
+  if (g.num_layers > 32767)
     return fail(KVC_ERR_UNSUPPORTED, "%s: num_layers=%lld exceeds 32767", fn, (long long)g.num_layers);
   if (g.row_elems * g.elem_bytes > (int64_t(1) << 30))
     return fail(KVC_ERR_UNSUPPORTED, "%s: row of %lld bytes is beyond 1 GiB", fn,
@@ -552,6 +691,51 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
   a.items_per_token = (uint32_t)items64;
 
+  // Rows under 1 KiB: lanes run over consecutive tokens of one plane.
+  if (g_tune.write_narrow && vec == 16 && a.vpr_shift >= 0 && a.vecs_per_row < 64) {
+    WriteLaunch l{};
+    const int64_t lanes_all = g.num_tokens * (int64_t)a.vecs_per_row;
+    l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes_all + 63) / 64 * 64);
+    a.tokens_per_wg = l.threads / a.vecs_per_row;
+    a.num_planes = (uint32_t)(2 * g.num_layers);
+    const int64_t token_groups_all = (g.num_tokens + a.tokens_per_wg - 1) / a.tokens_per_wg;
+    l.vpt = g_tune.write_narrow_vpt;
+    if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8) {
+      // the fewest planes per lane that keep the launch within one resident set
+      const int64_t resident = resident_workgroups();
+      l.vpt = 8;
+      for (int v = 1; v < 8; v *= 2)
+        if (token_groups_all * ((a.num_planes + v - 1) / v) <= resident) {
+          l.vpt = v;
+          break;
+        }
+    }
+    while (l.vpt > 1 && (uint32_t)(l.vpt / 2) >= a.num_planes) l.vpt /= 2;
+    l.nt = (g_tune.write_nt & 1) != 0;
+    const int64_t plane_groups = (a.num_planes + l.vpt - 1) / l.vpt;
+    const int64_t max_groups = std::max<int64_t>(1, 0x7fffffffll / plane_groups);
+    const int64_t max_tokens = max_groups * a.tokens_per_wg;
+    for (int64_t t0 = 0; t0 < g.num_tokens; t0 += max_tokens) {
+      const int64_t n_tok = std::min(max_tokens, g.num_tokens - t0);
+      a.num_tokens = (uint32_t)n_tok;
+      a.num_token_groups = (uint32_t)((n_tok + a.tokens_per_wg - 1) / a.tokens_per_wg);
+      l.grid = (unsigned)(a.num_token_groups * plane_groups);
+      a.key = (const char*)key + t0 * a.key_token_stride;
+      a.value = (const char*)value + t0 * a.value_token_stride;
+      if (paged) {
+        a.batch_indices = batch_indices + t0;
+        a.positions = positions + t0;
+        launch_narrow<true>(a, l, (hipStream_t)stream);
+      } else {
+        a.slot_mapping = (const char*)slot_mapping + t0 * slot_bytes;
+        launch_narrow<false>(a, l, (hipStream_t)stream);
+      }
+      KVC_HIP(hipGetLastError());
+    }
+    g_last = LastLaunch{KVC_KERNEL_WRITE_ROWS_NARROW, 16, l.vpt, l.threads, l.grid, l.nt};
+    return KVC_OK;
+  }
+
   // Launch shape, from sweeps on MI355X. 256-lane workgroups with one vector per
   // lane (the leanest lane, the most workgroups) are best whenever the launch is
   // either smaller than one resident set of workgroups (2048 lanes per CU) or
@@ -611,6 +795,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     }
     KVC_HIP(hipGetLastError());
   }
+  g_last = LastLaunch{KVC_KERNEL_WRITE_ROWS, vec, l.vpt, l.threads, l.grid, (l.nt ? 1 : 0) | (l.ntl ? 2 : 0)};
   return KVC_OK;
 }
 
@@ -658,6 +843,7 @@ int launch_tiles_vec(TileArgs a, int unroll, int max_wgs, hipStream_t s, bool nt
     case 8: launch_tiles_nt<VEC, 8>(a, (unsigned)grid, s, nt); break;
     default: launch_tiles_nt<VEC, 16>(a, (unsigned)grid, s, nt); break;
   }
+  g_last = LastLaunch{KVC_KERNEL_COPY_TILES, VEC, unroll, kThreads, (int64_t)grid, nt ? 1 : 0};
   KVC_HIP(hipGetLastError());
   return KVC_OK;
 }
@@ -687,52 +873,89 @@ inline int64_t round_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 inline int64_t ids_region_bytes(int64_t n) { return round_up(2 * n * (int64_t)sizeof(int64_t), kIdAlign); }
 
 // Per-thread resources of the swap entry points: events that order the two
-// streams, and a pinned bounce buffer from which the id lists are uploaded (the
-// caller's lists may be pageable and may be freed as soon as the call returns).
+// streams of a staged swap, and a small ring of pinned bounce buffers from
+// which id lists are uploaded (the caller's lists may be pageable and may be
+// freed as soon as the call returns). A bounce slot is reused only after its
+// upload has run, so a call waits on the host only when kBounceSlots uploads of
+// this thread are still queued. A slot that is too small is replaced by a
+// larger one (at least twice its size); the outgrown buffer is kept until
+// kvc_thread_release, because freeing pinned memory synchronises the device.
+constexpr int kBounceSlots = 4;
+
+struct Bounce {
+  int64_t* buf = nullptr;
+  int64_t cap = 0;  // int64 entries
+  hipEvent_t done = nullptr;
+  bool pending = false;
+};
+
 struct SwapCtx {
-  hipEvent_t start = nullptr, ids_done = nullptr, tail = nullptr;
+  hipEvent_t start = nullptr, tail = nullptr;
   hipEvent_t filled[2] = {nullptr, nullptr};   // staging slot holds fresh data
   hipEvent_t drained[2] = {nullptr, nullptr};  // staging slot may be overwritten
-  int64_t* ids_host = nullptr;
-  int64_t ids_cap = 0;
-  bool ids_pending = false;
+  Bounce bounce[kBounceSlots];
+  int next_bounce = 0;
+  int64_t** retired = nullptr;  // outgrown bounce buffers
+  int num_retired = 0, cap_retired = 0;
   int device = -1;
+
+  void all_events(hipEvent_t** out) {
+    int k = 0;
+    out[k++] = &start; out[k++] = &tail;
+    out[k++] = &filled[0]; out[k++] = &filled[1];
+    out[k++] = &drained[0]; out[k++] = &drained[1];
+    for (int i = 0; i < kBounceSlots; ++i) out[k++] = &bounce[i].done;
+  }
 };
+constexpr int kSwapEvents = 6 + kBounceSlots;
 thread_local SwapCtx g_swap;
 
-int swap_ctx_prepare(int64_t n) {
+void swap_ctx_drop_events(SwapCtx& c) {
+  for (int i = 0; i < kBounceSlots; ++i) {
+    if (c.bounce[i].pending) (void)hipEventSynchronize(c.bounce[i].done);
+    c.bounce[i].pending = false;
+  }
+  hipEvent_t* evs[kSwapEvents];
+  c.all_events(evs);
+  for (hipEvent_t* e : evs) {
+    if (*e) (void)hipEventDestroy(*e);
+    *e = nullptr;
+  }
+}
+
+// events of this thread on the current device (they belong to the device they
+// were created on: a thread that moves to another device starts over)
+int swap_ctx_prepare() {
   int dev = 0;
   KVC_HIP(hipGetDevice(&dev));
   SwapCtx& c = g_swap;
   if (c.device != dev) {
-    if (c.device >= 0) {
-      // events belong to the device they were created on: start over
-      if (c.ids_pending) (void)hipEventSynchronize(c.ids_done);
-      c.ids_pending = false;
-      hipEvent_t* evs[] = {&c.start, &c.ids_done, &c.tail, &c.filled[0], &c.filled[1],
-                           &c.drained[0], &c.drained[1]};
-      for (hipEvent_t* e : evs) {
-        if (*e) (void)hipEventDestroy(*e);
-        *e = nullptr;
-      }
-    }
-    hipEvent_t* evs[] = {&c.start, &c.ids_done, &c.tail, &c.filled[0], &c.filled[1],
-                         &c.drained[0], &c.drained[1]};
+    if (c.device >= 0) swap_ctx_drop_events(c);
+    c.device = -1;
+    hipEvent_t* evs[kSwapEvents];
+    c.all_events(evs);
     for (hipEvent_t* e : evs) KVC_HIP(hipEventCreateWithFlags(e, hipEventDisableTiming));
     c.device = dev;
   }
-  if (c.ids_pending) {
-    KVC_HIP(hipEventSynchronize(c.ids_done));
-    c.ids_pending = false;
+  return KVC_OK;
+}
+
+int swap_ctx_release() {
+  SwapCtx& c = g_swap;
+  if (c.device >= 0) swap_ctx_drop_events(c);
+  c.device = -1;
+  int rc = KVC_OK;
+  for (int i = 0; i < kBounceSlots; ++i) {
+    if (c.bounce[i].buf && hipHostFree(c.bounce[i].buf) != hipSuccess) rc = KVC_ERR_HIP;
+    c.bounce[i] = Bounce{};
   }
-  if (2 * n > c.ids_cap) {
-    if (c.ids_host) KVC_HIP(hipHostFree(c.ids_host));
-    c.ids_host = nullptr;
-    c.ids_cap = 0;
-    const int64_t cap = std::max<int64_t>(2 * n, 4096);
-    KVC_HIP(hipHostMalloc((void**)&c.ids_host, cap * sizeof(int64_t), hipHostMallocDefault));
-    c.ids_cap = cap;
-  }
+  for (int i = 0; i < c.num_retired; ++i)
+    if (hipHostFree(c.retired[i]) != hipSuccess) rc = KVC_ERR_HIP;
+  std::free(c.retired);
+  c.retired = nullptr;
+  c.num_retired = c.cap_retired = 0;
+  c.next_bounce = 0;
+  if (rc != KVC_OK) return fail(rc, "kvc_thread_release: hipHostFree failed");
   return KVC_OK;
 }
 
@@ -741,9 +964,25 @@ struct SwapGeom {
   int64_t num_gpu_blocks, num_host_blocks, layer_begin, layer_end;
 };
 
+int check_ids(const char* fn, const int64_t* gpu_ids, const int64_t* host_ids, int64_t n,
+              int64_t num_gpu_blocks, int64_t num_host_blocks) {
+  for (int64_t i = 0; i < n; ++i) {
+    if (gpu_ids[i] < 0 || gpu_ids[i] >= num_gpu_blocks)
+      return fail(KVC_ERR_OUT_OF_RANGE, "%s: gpu block id %lld (entry %lld) outside [0, %lld)", fn,
+                  (long long)gpu_ids[i], (long long)i, (long long)num_gpu_blocks);
+    if (host_ids[i] < 0 || host_ids[i] >= num_host_blocks)
+      return fail(KVC_ERR_OUT_OF_RANGE, "%s: host block id %lld (entry %lld) outside [0, %lld)", fn,
+                  (long long)host_ids[i], (long long)i, (long long)num_host_blocks);
+  }
+  return KVC_OK;
+}
+
+// prepared: the id lists already sit at the head of the staging buffer
+// (kvc_swap_prepare checked and uploaded them); gpu_ids is then unused and
+// host_ids is needed only by the staged mode's PCIe extents.
 int check_swap(const char* fn, const void* pool, const void* host, const int64_t* gpu_ids,
                const int64_t* host_ids, const SwapGeom& g, const void* staging,
-               int64_t staging_bytes, int mode, int64_t* chunk_blocks) {
+               int64_t staging_bytes, int mode, bool prepared, int64_t* chunk_blocks) {
   if (g.n < 0 || g.num_layers < 0 || g.block_bytes < 0 || g.layer_stride_bytes < 0)
     return fail(KVC_ERR_INVALID_ARG, "%s: negative size", fn);
   if (g.layer_begin < 0 || g.layer_end < g.layer_begin || g.layer_end > g.num_layers)
@@ -754,18 +993,15 @@ int check_swap(const char* fn, const void* pool, const void* host, const int64_t
   const int64_t nl = g.layer_end - g.layer_begin;
   *chunk_blocks = 0;
   if (g.n == 0 || nl == 0 || g.block_bytes == 0) return KVC_OK;
-  if (!pool || !host || !gpu_ids || !host_ids)
-    return fail(KVC_ERR_INVALID_ARG, "%s: null pool/host/id pointer", fn);
+  if (!pool || !host) return fail(KVC_ERR_INVALID_ARG, "%s: null pool/host pointer", fn);
+  if (prepared ? (mode == KVC_SWAP_STAGED && !host_ids) : (!gpu_ids || !host_ids))
+    return fail(KVC_ERR_INVALID_ARG, "%s: null id list", fn);
   if (g.layer_stride_bytes < g.block_bytes)
     return fail(KVC_ERR_INVALID_ARG, "%s: layer stride smaller than a block", fn);
   if (nl > 0xffffffffll) return fail(KVC_ERR_UNSUPPORTED, "%s: too many layers", fn);
-  for (int64_t i = 0; i < g.n; ++i) {
-    if (gpu_ids[i] < 0 || gpu_ids[i] >= g.num_gpu_blocks)
-      return fail(KVC_ERR_OUT_OF_RANGE, "%s: gpu block id %lld (entry %lld) outside [0, %lld)", fn,
-                  (long long)gpu_ids[i], (long long)i, (long long)g.num_gpu_blocks);
-    if (host_ids[i] < 0 || host_ids[i] >= g.num_host_blocks)
-      return fail(KVC_ERR_OUT_OF_RANGE, "%s: host block id %lld (entry %lld) outside [0, %lld)", fn,
-                  (long long)host_ids[i], (long long)i, (long long)g.num_host_blocks);
+  if (!prepared) {
+    const int rc = check_ids(fn, gpu_ids, host_ids, g.n, g.num_gpu_blocks, g.num_host_blocks);
+    if (rc != KVC_OK) return rc;
   }
   if (!staging) return fail(KVC_ERR_STAGING, "%s: null staging buffer", fn);
   if ((uintptr_t)staging % kIdAlign)
@@ -789,11 +1025,34 @@ int check_swap(const char* fn, const void* pool, const void* host, const int64_t
 int upload_ids(const int64_t* gpu_ids, const int64_t* host_ids, int64_t n, void* staging,
                hipStream_t s) {
   SwapCtx& c = g_swap;
-  std::memcpy(c.ids_host, gpu_ids, n * sizeof(int64_t));
-  std::memcpy(c.ids_host + n, host_ids, n * sizeof(int64_t));
-  KVC_HIP(hipMemcpyAsync(staging, c.ids_host, 2 * n * sizeof(int64_t), hipMemcpyHostToDevice, s));
-  KVC_HIP(hipEventRecord(c.ids_done, s));
-  c.ids_pending = true;
+  Bounce& b = c.bounce[c.next_bounce];
+  c.next_bounce = (c.next_bounce + 1) % kBounceSlots;
+  if (b.pending) {
+    KVC_HIP(hipEventSynchronize(b.done));
+    b.pending = false;
+  }
+  if (2 * n > b.cap) {
+    if (b.buf) {
+      if (c.num_retired == c.cap_retired) {
+        const int cap = c.cap_retired ? 2 * c.cap_retired : 8;
+        int64_t** grown = (int64_t**)std::realloc(c.retired, cap * sizeof(int64_t*));
+        if (!grown) return fail(KVC_ERR_HIP, "out of host memory");
+        c.retired = grown;
+        c.cap_retired = cap;
+      }
+      c.retired[c.num_retired++] = b.buf;
+      b.buf = nullptr;
+    }
+    const int64_t cap = std::max<int64_t>(std::max<int64_t>(2 * n, 2 * b.cap), 4096);
+    b.cap = 0;
+    KVC_HIP(hipHostMalloc((void**)&b.buf, cap * sizeof(int64_t), hipHostMallocDefault));
+    b.cap = cap;
+  }
+  std::memcpy(b.buf, gpu_ids, n * sizeof(int64_t));
+  std::memcpy(b.buf + n, host_ids, n * sizeof(int64_t));
+  KVC_HIP(hipMemcpyAsync(staging, b.buf, 2 * n * sizeof(int64_t), hipMemcpyHostToDevice, s));
+  KVC_HIP(hipEventRecord(b.done, s));
+  b.pending = true;
   return KVC_OK;
 }
 
@@ -824,54 +1083,75 @@ int copy_chunk_rows(char* slot, char* host_pool, const int64_t* host_ids, int64_
   return KVC_OK;
 }
 
+// the tile-kernel arguments of a direct swap: pool <-> mapped host pool
+TileArgs direct_swap_tiles(bool out, char* pool, char* host_pool, const int64_t* d_gpu_ids,
+                           const int64_t* d_host_ids, const SwapGeom& g) {
+  const int64_t host_block_bytes = g.num_layers * g.block_bytes;
+  char* pool_l0 = pool + g.layer_begin * g.layer_stride_bytes;
+  char* host_l0 = host_pool + g.layer_begin * g.block_bytes;
+  TileArgs t{};
+  t.id_stride = 1;
+  t.tile_bytes = g.block_bytes;
+  t.num_layers = (uint32_t)(g.layer_end - g.layer_begin);
+  if (out) {
+    t.src_base = pool_l0; t.src_ids = d_gpu_ids;
+    t.src_layer_stride = g.layer_stride_bytes; t.src_block_stride = g.block_bytes;
+    t.num_src_blocks = g.num_gpu_blocks;
+    t.dst_base = host_l0; t.dst_ids = d_host_ids;
+    t.dst_layer_stride = g.block_bytes; t.dst_block_stride = host_block_bytes;
+    t.num_dst_blocks = g.num_host_blocks;
+  } else {
+    t.src_base = host_l0; t.src_ids = d_host_ids;
+    t.src_layer_stride = g.block_bytes; t.src_block_stride = host_block_bytes;
+    t.num_src_blocks = g.num_host_blocks;
+    t.dst_base = pool_l0; t.dst_ids = d_gpu_ids;
+    t.dst_layer_stride = g.layer_stride_bytes; t.dst_block_stride = g.block_bytes;
+    t.num_dst_blocks = g.num_gpu_blocks;
+  }
+  return t;
+}
+
 int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_t* gpu_ids,
              const int64_t* host_ids, const SwapGeom& g, void* staging, int64_t staging_bytes,
-             int mode, void* kernel_stream, void* copy_stream) {
+             int mode, bool prepared, void* kernel_stream, void* copy_stream) {
   int64_t chunk_blocks = 0;
   int rc = check_swap(fn, pool, host_pool, gpu_ids, host_ids, g, staging, staging_bytes, mode,
-                      &chunk_blocks);
+                      prepared, &chunk_blocks);
   if (rc != KVC_OK) return rc;
   const int64_t nl = g.layer_end - g.layer_begin;
   if (g.n == 0 || nl == 0 || g.block_bytes == 0) return KVC_OK;
-  rc = swap_ctx_prepare(g.n);
-  if (rc != KVC_OK) return rc;
-  SwapCtx& c = g_swap;
   hipStream_t ks = (hipStream_t)kernel_stream;
   hipStream_t cs = (hipStream_t)copy_stream;
   const bool two_streams = ks != cs;
-
-  rc = upload_ids(gpu_ids, host_ids, g.n, staging, ks);
-  if (rc != KVC_OK) return rc;
   const int64_t* d_gpu_ids = (const int64_t*)staging;
   const int64_t* d_host_ids = d_gpu_ids + g.n;
+
+  if (mode == KVC_SWAP_DIRECT && prepared) {
+    // nothing but the launch: no events, no upload
+    const TileArgs t = direct_swap_tiles(out, pool, host_pool, d_gpu_ids, d_host_ids, g);
+    return launch_tiles(t, g.n, g_tune.direct_max_wgs, ks);
+  }
+  rc = swap_ctx_prepare();
+  if (rc != KVC_OK) return rc;
+  SwapCtx& c = g_swap;
+  if (!prepared) {
+    rc = upload_ids(gpu_ids, host_ids, g.n, staging, ks);
+    if (rc != KVC_OK) return rc;
+  }
   const int64_t host_block_bytes = g.num_layers * g.block_bytes;
   char* pool_l0 = pool + g.layer_begin * g.layer_stride_bytes;
   const int64_t host_row_offset = g.layer_begin * g.block_bytes;
+
+  if (mode == KVC_SWAP_DIRECT) {
+    // pool <-> mapped host pool in a single kernel
+    const TileArgs t = direct_swap_tiles(out, pool, host_pool, d_gpu_ids, d_host_ids, g);
+    return launch_tiles(t, g.n, g_tune.direct_max_wgs, ks);
+  }
 
   TileArgs t{};
   t.id_stride = 1;
   t.tile_bytes = g.block_bytes;
   t.num_layers = (uint32_t)nl;
-
-  if (mode == KVC_SWAP_DIRECT) {
-    // pool <-> mapped host pool in a single kernel
-    if (out) {
-      t.src_base = pool_l0; t.src_ids = d_gpu_ids;
-      t.src_layer_stride = g.layer_stride_bytes; t.src_block_stride = g.block_bytes;
-      t.num_src_blocks = g.num_gpu_blocks;
-      t.dst_base = host_pool + host_row_offset; t.dst_ids = d_host_ids;
-      t.dst_layer_stride = g.block_bytes; t.dst_block_stride = host_block_bytes;
-      t.num_dst_blocks = g.num_host_blocks;
-    } else {
-      t.src_base = host_pool + host_row_offset; t.src_ids = d_host_ids;
-      t.src_layer_stride = g.block_bytes; t.src_block_stride = host_block_bytes;
-      t.num_src_blocks = g.num_host_blocks;
-      t.dst_base = pool_l0; t.dst_ids = d_gpu_ids;
-      t.dst_layer_stride = g.layer_stride_bytes; t.dst_block_stride = g.block_bytes;
-      t.num_dst_blocks = g.num_gpu_blocks;
-    }
-    return launch_tiles(t, g.n, g_tune.direct_max_wgs, ks);
-  }
 
   // staged: two ring slots, kernel on ks, PCIe extents on cs
   const int64_t width = nl * g.block_bytes;  // bytes of one block's layer range
@@ -949,20 +1229,44 @@ const char* kvc_last_error_string(void) { return kvc::g_err; }
 // KVC_ERR_INVALID_ARG for an unknown key.
 int kvc_set_tuning(const char* key, int value) {
   if (!key) return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: null key");
-  if (!strcmp(key, "copy_unroll")) g_tune.copy_unroll = value;
-  else if (!strcmp(key, "gather_unroll")) g_tune.gather_unroll = value;
-  else if (!strcmp(key, "copy_nt")) g_tune.copy_nt = value;
-  else if (!strcmp(key, "copy_max_wgs")) g_tune.copy_max_wgs = value;
-  else if (!strcmp(key, "copy_order")) g_tune.copy_order = value;
-  else if (!strcmp(key, "write_vpt")) g_tune.write_vpt = value;
-  else if (!strcmp(key, "write_nt")) g_tune.write_nt = value;
-  else if (!strcmp(key, "write_order")) g_tune.write_order = value;
-  else if (!strcmp(key, "write_threads")) g_tune.write_threads = value;
-  else if (!strcmp(key, "direct_max_wgs")) g_tune.direct_max_wgs = value;
-  else if (!strcmp(key, "rope_threads")) kvc::g_rope_tune.threads = value;
-  else if (!strcmp(key, "disk_bounce_mib")) kvc::g_disk_bounce_mib = value;
-  else return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: unknown key '%s'", key);
+  Knob* k = find_knob(key);
+  if (!k) return fail(KVC_ERR_INVALID_ARG, "kvc_set_tuning: unknown key '%s'", key);
+  *k->value = value;
   return KVC_OK;
+}
+
+int kvc_get_tuning(const char* key, int* value) {
+  if (!key || !value) return fail(KVC_ERR_INVALID_ARG, "kvc_get_tuning: null argument");
+  Knob* k = find_knob(key);
+  if (!k) return fail(KVC_ERR_INVALID_ARG, "kvc_get_tuning: unknown key '%s'", key);
+  *value = *k->value;
+  return KVC_OK;
+}
+
+int kvc_reset_tuning(void) {
+  int n = 0;
+  Knob* t = knobs(&n);
+  for (int i = 0; i < n; ++i) *t[i].value = t[i].initial;
+  return KVC_OK;
+}
+
+int kvc_tuning_modified(void) {
+  int n = 0, changed = 0;
+  Knob* t = knobs(&n);
+  for (int i = 0; i < n; ++i) changed += *t[i].value != t[i].initial;
+  return changed;
+}
+
+int64_t kvc_last_launch_info(int what) {
+  switch (what) {
+    case KVC_LAUNCH_KERNEL: return g_last.kernel;
+    case KVC_LAUNCH_VEC_BYTES: return g_last.vec;
+    case KVC_LAUNCH_PER_LANE: return g_last.per_lane;
+    case KVC_LAUNCH_THREADS: return g_last.threads;
+    case KVC_LAUNCH_GRID: return g_last.grid;
+    case KVC_LAUNCH_NON_TEMPORAL: return g_last.nt;
+    default: return KVC_ERR_INVALID_ARG;
+  }
 }
 
 int kvc_reshape_and_cache_layers(const void* key, const void* value, void* key_cache,
@@ -1033,6 +1337,58 @@ int kvc_append_paged_kv_cache(const void* append_key, const void* append_value,
                                           nnz, batch_size, num_kv_indices, num_kv_heads, head_dim,
                                           page_size, key_token_stride, value_token_stride,
                                           page_stride, num_pages, 1, 0, 0, 0, elem_bytes, stream);
+}
+
+// ---- per-step plan of the page-table write ----------------------------------
+struct kvc_write_plan {
+  const int32_t* batch_indices;
+  const int32_t* positions;
+  const int32_t* kv_indices;
+  const int32_t* kv_indptr;
+  const int32_t* kv_last_page_len;
+  int64_t nnz, batch_size, num_kv_indices, num_kv_heads, head_dim, page_size;
+  int elem_bytes;
+};
+
+int kvc_write_plan_create(const int32_t* batch_indices, const int32_t* positions,
+                          const int32_t* kv_indices, const int32_t* kv_indptr,
+                          const int32_t* kv_last_page_len, int64_t nnz, int64_t batch_size,
+                          int64_t num_kv_indices, int64_t num_kv_heads, int64_t head_dim,
+                          int64_t page_size, int elem_bytes, kvc_write_plan** out) {
+  if (!out) return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_create: null out");
+  *out = nullptr;
+  if (num_kv_heads < 0 || head_dim < 0 || page_size <= 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_create: bad H/D/page_size");
+  if (nnz < 0 || batch_size < 0 || num_kv_indices < 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_create: negative size");
+  if (nnz > 0 && (!batch_indices || !positions || !kv_indices || !kv_indptr))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_create: null index array");
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return fail(KVC_ERR_UNSUPPORTED, "kvc_write_plan_create: elem_bytes=%d (need 1, 2, 4 or 8)", elem_bytes);
+  kvc_write_plan* p = new (std::nothrow) kvc_write_plan{
+      batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len, nnz, batch_size,
+      num_kv_indices, num_kv_heads, head_dim, page_size, elem_bytes};
+  if (!p) return fail(KVC_ERR_HIP, "kvc_write_plan_create: out of host memory");
+  *out = p;
+  return KVC_OK;
+}
+
+int kvc_write_plan_append(const kvc_write_plan* plan, const void* append_key,
+                          const void* append_value, int64_t key_token_stride,
+                          int64_t value_token_stride, void* paged_kv_cache, int64_t page_stride,
+                          int64_t num_pages, void* stream) {
+  if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_append: null plan");
+  return kvc_append_paged_kv_cache(append_key, append_value, plan->batch_indices, plan->positions,
+                                   paged_kv_cache, plan->kv_indices, plan->kv_indptr,
+                                   plan->kv_last_page_len, plan->nnz, plan->batch_size,
+                                   plan->num_kv_indices, plan->num_kv_heads, plan->head_dim,
+                                   plan->page_size, key_token_stride, value_token_stride,
+                                   page_stride, num_pages, plan->elem_bytes, stream);
+}
+
+int kvc_write_plan_destroy(kvc_write_plan* plan) {
+  delete plan;
+  return KVC_OK;
 }
 
 int kvc_get_seq_lens(const int32_t* kv_indptr, const int32_t* kv_last_page_len, int64_t batch_size,
@@ -1197,7 +1553,7 @@ int kvc_swap_out(const void* pool, void* host_pool, const int64_t* src_ids, cons
   SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
              layer_begin, layer_end};
   return run_swap("kvc_swap_out", true, (char*)pool, (char*)host_pool, src_ids, dst_ids, g,
-                  staging, staging_bytes, mode, kernel_stream, copy_stream);
+                  staging, staging_bytes, mode, false, kernel_stream, copy_stream);
 }
 
 int kvc_swap_in(void* pool, const void* host_pool, const int64_t* src_ids, const int64_t* dst_ids,
@@ -1208,8 +1564,53 @@ int kvc_swap_in(void* pool, const void* host_pool, const int64_t* src_ids, const
   SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
              layer_begin, layer_end};
   return run_swap("kvc_swap_in", false, (char*)pool, (char*)host_pool, dst_ids, src_ids, g, staging,
-                  staging_bytes, mode, kernel_stream, copy_stream);
+                  staging_bytes, mode, false, kernel_stream, copy_stream);
 }
+
+int kvc_swap_prepare(const int64_t* gpu_ids, const int64_t* host_ids, int64_t n,
+                     int64_t num_gpu_blocks, int64_t num_host_blocks, void* staging,
+                     int64_t staging_bytes, void* stream) {
+  if (n < 0 || num_gpu_blocks < 0 || num_host_blocks < 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_swap_prepare: negative size");
+  if (n == 0) return KVC_OK;
+  if (!gpu_ids || !host_ids) return fail(KVC_ERR_INVALID_ARG, "kvc_swap_prepare: null id list");
+  int rc = check_ids("kvc_swap_prepare", gpu_ids, host_ids, n, num_gpu_blocks, num_host_blocks);
+  if (rc != KVC_OK) return rc;
+  if (!staging) return fail(KVC_ERR_STAGING, "kvc_swap_prepare: null staging buffer");
+  if ((uintptr_t)staging % kIdAlign)
+    return fail(KVC_ERR_STAGING, "kvc_swap_prepare: staging buffer must be %lld-byte aligned",
+                (long long)kIdAlign);
+  if (staging_bytes < ids_region_bytes(n))
+    return fail(KVC_ERR_STAGING, "kvc_swap_prepare: staging of %lld bytes cannot hold the id lists (%lld)",
+                (long long)staging_bytes, (long long)ids_region_bytes(n));
+  rc = swap_ctx_prepare();
+  if (rc != KVC_OK) return rc;
+  return upload_ids(gpu_ids, host_ids, n, staging, (hipStream_t)stream);
+}
+
+int kvc_swap_out_prepared(const void* pool, void* host_pool, const int64_t* host_ids, int64_t n,
+                          int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                          int64_t num_gpu_blocks, int64_t num_host_blocks, int64_t layer_begin,
+                          int64_t layer_end, void* staging, int64_t staging_bytes, int mode,
+                          void* kernel_stream, void* copy_stream) {
+  SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
+             layer_begin, layer_end};
+  return run_swap("kvc_swap_out_prepared", true, (char*)pool, (char*)host_pool, nullptr, host_ids, g,
+                  staging, staging_bytes, mode, true, kernel_stream, copy_stream);
+}
+
+int kvc_swap_in_prepared(void* pool, const void* host_pool, const int64_t* host_ids, int64_t n,
+                         int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                         int64_t num_gpu_blocks, int64_t num_host_blocks, int64_t layer_begin,
+                         int64_t layer_end, void* staging, int64_t staging_bytes, int mode,
+                         void* kernel_stream, void* copy_stream) {
+  SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
+             layer_begin, layer_end};
+  return run_swap("kvc_swap_in_prepared", false, (char*)pool, (char*)host_pool, nullptr, host_ids, g,
+                  staging, staging_bytes, mode, true, kernel_stream, copy_stream);
+}
+
+int kvc_thread_release(void) { return swap_ctx_release(); }
 
 void* kvc_host_alloc_pinned(size_t bytes) {
   void* p = nullptr;

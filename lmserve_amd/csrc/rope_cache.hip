@@ -17,6 +17,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <new>
 
 #include "common.h"
 #include "kvcache.h"
@@ -545,6 +546,68 @@ int kvc_rotary_pos_emb_and_append_paged(const void* query, const void* key, cons
               num_kv_indices, page_size, page_stride, row, num_pages};
   return run_rope("kvc_rotary_pos_emb_and_append_paged", query, key, value, query_out, key_out,
                   positions, 4, cos_sin_cache, g, &c, stream);
+}
+
+// ---- per-step plan of the fused rotation + page-table write ------------------
+struct kvc_rotary_plan {
+  const int32_t* batch_indices;
+  const int32_t* positions;
+  const void* cos_sin_cache;
+  const int32_t* kv_indices;
+  const int32_t* kv_indptr;
+  int64_t max_position, nnz, num_heads, num_kv_heads, head_dim, rotary_dim;
+  int64_t batch_size, num_kv_indices, page_size;
+  int dtype;
+};
+
+int kvc_rotary_plan_create(const int32_t* batch_indices, const int32_t* positions,
+                           const void* cos_sin_cache, int64_t max_position, int64_t nnz,
+                           int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                           int64_t rotary_dim, const int32_t* kv_indices,
+                           const int32_t* kv_indptr, int64_t batch_size, int64_t num_kv_indices,
+                           int64_t page_size, int dtype, kvc_rotary_plan** out) {
+  if (!out) return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_create: null out");
+  *out = nullptr;
+  if (dtype != KVC_DTYPE_BF16 && dtype != KVC_DTYPE_F16 && dtype != KVC_DTYPE_F32)
+    return fail(KVC_ERR_UNSUPPORTED, "kvc_rotary_plan_create: dtype %d (need bf16, f16 or f32)", dtype);
+  if (nnz < 0 || num_heads < 0 || num_kv_heads < 0 || head_dim <= 0 || rotary_dim < 0 ||
+      max_position < 0 || batch_size < 0 || num_kv_indices < 0 || page_size <= 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_create: bad size");
+  if (rotary_dim > head_dim || (rotary_dim & 1))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_create: rotary_dim %lld must be even and <= head_dim %lld",
+                (long long)rotary_dim, (long long)head_dim);
+  if (rotary_dim > kMaxRotaryDim)
+    return fail(KVC_ERR_UNSUPPORTED, "kvc_rotary_plan_create: rotary_dim %lld exceeds %d",
+                (long long)rotary_dim, kMaxRotaryDim);
+  if (nnz > 0 && (!batch_indices || !positions || !cos_sin_cache || !kv_indices || !kv_indptr))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_create: null pointer");
+  kvc_rotary_plan* p = new (std::nothrow) kvc_rotary_plan{
+      batch_indices, positions, cos_sin_cache, kv_indices, kv_indptr, max_position, nnz, num_heads,
+      num_kv_heads, head_dim, rotary_dim, batch_size, num_kv_indices, page_size, dtype};
+  if (!p) return fail(KVC_ERR_HIP, "kvc_rotary_plan_create: out of host memory");
+  *out = p;
+  return KVC_OK;
+}
+
+int kvc_rotary_plan_run(const kvc_rotary_plan* plan, const void* query, const void* key,
+                        const void* value, int64_t q_token_stride, int64_t k_token_stride,
+                        int64_t v_token_stride, void* query_out, void* key_out,
+                        void* paged_kv_cache, int64_t page_stride, int64_t num_pages,
+                        void* stream) {
+  if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_run: null plan");
+  const int64_t q_row = plan->num_heads * plan->head_dim;
+  const int64_t k_row = plan->num_kv_heads * plan->head_dim;
+  return kvc_rotary_pos_emb_and_append_paged(
+      query, key, value, plan->batch_indices, plan->positions, plan->cos_sin_cache,
+      plan->max_position, plan->nnz, plan->num_heads, plan->num_kv_heads, plan->head_dim,
+      plan->rotary_dim, q_token_stride, k_token_stride, v_token_stride, query_out, key_out, q_row,
+      k_row, paged_kv_cache, plan->kv_indices, plan->kv_indptr, plan->batch_size,
+      plan->num_kv_indices, plan->page_size, page_stride, num_pages, plan->dtype, stream);
+}
+
+int kvc_rotary_plan_destroy(kvc_rotary_plan* plan) {
+  delete plan;
+  return KVC_OK;
 }
 
 }  // extern "C"

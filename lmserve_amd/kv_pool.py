@@ -1,4 +1,4 @@
-"""Pool sizing, block-id allocation order and the layer-sync handle.
+"""Pool sizing and the layer-sync handle.
 
 Host-side mirrors of the pieces that decide what the data-movement kernels are
 handed:
@@ -6,9 +6,6 @@ handed:
 * `plan_cache` / `allocate_kv_caches` -- the pool arithmetic and layout of
   `ModelWorker.init_cache` (runtime/worker/llm_worker/model_worker.py:200-228,
   :278-281).
-* `BlockAllocator` -- the id order of the Rust allocator
-  (runtime/src/llm_engine/block_manager.rs:62-165): a FIFO free list that
-  starts as 0..nb, so block tables turn into an arbitrary scatter under churn.
 * `KVWorkerHandle` / `LayerSyncHooks` -- the per-layer event + queue protocol
   between the model's forward pass and the swap engine
   (model_worker.py:232-276, kv_worker.py:25-30), with `torch.cuda.Event`
@@ -17,7 +14,6 @@ handed:
 from __future__ import annotations
 
 import queue
-from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Any, Iterable, List, Optional
 
@@ -48,57 +44,6 @@ def allocate_kv_caches(num_layers: int, num_gpu_blocks: int, block_size: int, nu
     (model_worker.py:221-228)."""
     return torch.empty(num_layers, num_gpu_blocks, 2, block_size, num_kv_heads, head_dim,
                        dtype=dtype, device=device)
-
-
-class BlockAllocator:
-    """Block ids in the order the reference's allocator hands them out.
-
-    The free list is an insertion-ordered set initialised with 0..num_blocks-1;
-    `alloc_block` pops its front, `free_block` appends at its back once the
-    reference count reaches zero, `alloc_block_by_id` takes a named block
-    (prefix sharing bumps the count of a block already in use).
-    """
-
-    def __init__(self, num_blocks: int):
-        self.num_total_blocks = int(num_blocks)
-        self.ref_cnt = [0] * self.num_total_blocks
-        self.free_block_ids: "OrderedDict[int, None]" = OrderedDict(
-            (i, None) for i in range(self.num_total_blocks))
-
-    def can_alloc_blocks(self, num_required_blocks: int, watermark: float = 1.0) -> bool:
-        assert 0.0 < watermark <= 1.0, "watermark must be in (0, 1]"
-        used = self.num_total_blocks - len(self.free_block_ids)
-        return used + num_required_blocks <= int(watermark * self.num_total_blocks)
-
-    def alloc_block(self) -> int:
-        if not self.free_block_ids:
-            raise RuntimeError("Cannot allocate block: all blocks are already in use.")
-        block_id, _ = self.free_block_ids.popitem(last=False)
-        assert self.ref_cnt[block_id] == 0
-        self.ref_cnt[block_id] = 1
-        return block_id
-
-    def alloc_blocks(self, n: int) -> List[int]:
-        return [self.alloc_block() for _ in range(n)]
-
-    def alloc_block_by_id(self, block_id: int) -> int:
-        if self.ref_cnt[block_id] == 0:
-            del self.free_block_ids[block_id]
-        self.ref_cnt[block_id] += 1
-        return block_id
-
-    def free_block(self, block_id: int) -> None:
-        assert self.ref_cnt[block_id] > 0, f"Double free detected for block {block_id}."
-        self.ref_cnt[block_id] -= 1
-        if self.ref_cnt[block_id] == 0:
-            self.free_block_ids[block_id] = None
-
-    def free_blocks(self, block_ids: Iterable[int]) -> None:
-        for b in block_ids:
-            self.free_block(b)
-
-    def get_block_usage(self) -> float:
-        return (self.num_total_blocks - len(self.free_block_ids)) / self.num_total_blocks
 
 
 @dataclass

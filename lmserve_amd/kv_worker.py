@@ -11,8 +11,14 @@ hands the whole mapping list to libkvcache (`kvc_swap_out` / `kvc_swap_in`):
 a gather/scatter kernel plus large PCIe extents on a second stream, or one
 kernel that addresses the mapped host pool directly.
 
-The Host<->Disk legs (kv_worker.py:229-247) are plain NumPy row copies on a
-`.npy` memory map, as in the reference; they involve no GPU work.
+A copy that runs layer by layer (the reference's protocol with the model's
+forward pass) flattens, checks and uploads its id lists once
+(`kvc_swap_prepare`); each layer is then a single launch
+(`kvc_swap_out_prepared` / `kvc_swap_in_prepared`).
+
+The Host<->Disk legs (kv_worker.py:229-247) go through the native disk tier of
+the same library (`disk_tier.DiskTier`: whole-block positional I/O on the
+reference's `.npy` file); they involve no GPU work.
 """
 from __future__ import annotations
 
@@ -115,6 +121,18 @@ def memmap_disk_kv_cache(kv_cache_file: str, shape: Tuple[int, ...], dtype, mode
     return np.lib.format.open_memmap(kv_cache_file, mode="w+", dtype=dtype, shape=tuple(shape))
 
 
+@dataclass
+class PreparedSwap:
+    """Id lists of one copy, already checked and resident on the device
+    (`KVWorker.prepare_swap`)."""
+    direction: str                 # "out" (GPU->Host) or "in" (Host->GPU)
+    n: int
+    host_ids: np.ndarray           # kept alive: the staged mode reads it per call
+    staging: torch.Tensor          # head: [gpu_ids | host_ids] on the device
+    stream: torch.cuda.Stream
+    copy_stream: torch.cuda.Stream
+
+
 class KVWorker:
     """Owns the host pool and moves blocks between the tiers.
 
@@ -207,12 +225,17 @@ class KVWorker:
         }
 
     # ------------------------------------------------------------------ GPU legs
-    def _staging_for(self, direction: str, n: int, num_layers_in_range: int) -> torch.Tensor:
+    def _staging_for(self, direction: str, n: int, *layers_per_call: int) -> torch.Tensor:
+        """Device workspace of one direction, large enough for calls that cover
+        any of the given numbers of layers."""
         mode = SWAP_MODES[self.swap_mode]
-        need = _lib.lib().kvc_swap_staging_bytes(n, num_layers_in_range, self.block_stride, mode,
-                                                 self.staging_chunk_blocks)
-        if need < 0:
-            raise ValueError("bad swap geometry")
+        need = 0
+        for nl in layers_per_call:
+            b = _lib.lib().kvc_swap_staging_bytes(n, nl, self.block_stride, mode,
+                                                  self.staging_chunk_blocks)
+            if b < 0:
+                raise ValueError("bad swap geometry")
+            need = max(need, b)
         buf = self._staging[direction]
         if buf is None or buf.numel() < need:
             buf = torch.empty(int(need), dtype=torch.uint8, device=self.device)
@@ -260,21 +283,69 @@ class KVWorker:
         self._swap("in", src, dst, layer_begin, self.num_layers if layer_end is None else layer_end,
                    stream or self.htod_stream, self._htod_copy_stream)
 
+    # ------------------------------------------------- layer by layer, ids uploaded once
+    def prepare_swap(self, direction: str, block_mappings: Sequence[BlockMapping],
+                     stream: Optional[torch.cuda.Stream] = None) -> Optional["PreparedSwap"]:
+        """Flatten the mappings, range-check them and upload the id lists once, on
+        `stream`; the result feeds `swap_prepared_layers` any number of times.
+        direction: "out" (GPU->Host) or "in" (Host->GPU). None when there is
+        nothing to move."""
+        if direction not in ("out", "in"):
+            raise ValueError("direction must be 'out' or 'in'")
+        if len(block_mappings) == 0:
+            return None
+        src, dst = flatten_block_mappings(block_mappings)
+        n = int(src.shape[0])
+        if n == 0:
+            return None
+        gpu_ids, host_ids = (src, dst) if direction == "out" else (dst, src)
+        if stream is None:
+            stream = self.dtoh_stream if direction == "out" else self.htod_stream
+        copy_stream = self._dtoh_copy_stream if direction == "out" else self._htod_copy_stream
+        with torch.cuda.device(self.device):
+            stream.wait_stream(torch.cuda.current_stream(self.device))
+            # room for one layer per call and for the whole range in one call
+            staging = self._staging_for(direction, n, 1, self.num_layers)
+            staging.record_stream(stream)
+            staging.record_stream(copy_stream)
+            _lib.check(_lib.lib().kvc_swap_prepare(
+                gpu_ids.ctypes.data, host_ids.ctypes.data, n, self.num_gpu_blocks,
+                self.num_host_blocks, staging.data_ptr(), staging.numel(), stream.cuda_stream))
+        return PreparedSwap(direction, n, host_ids, staging, stream, copy_stream)
+
+    def swap_prepared_layers(self, prepared: Optional["PreparedSwap"], layer_begin: int,
+                             layer_end: int) -> None:
+        """Enqueue layers [layer_begin, layer_end) of a prepared swap on its stream:
+        one launch in direct mode, no id traffic, nothing to wait for on the host."""
+        if prepared is None or layer_end <= layer_begin:
+            return
+        lib = _lib.lib()
+        fn = lib.kvc_swap_out_prepared if prepared.direction == "out" else lib.kvc_swap_in_prepared
+        with torch.cuda.device(self.device):
+            _lib.check(fn(self.gpu_kv_caches.data_ptr(), self._host_pool.ptr,
+                          prepared.host_ids.ctypes.data, prepared.n, self.num_layers,
+                          self.layer_stride, self.block_stride, self.num_gpu_blocks,
+                          self.num_host_blocks, layer_begin, layer_end, prepared.staging.data_ptr(),
+                          prepared.staging.numel(), SWAP_MODES[self.swap_mode],
+                          prepared.stream.cuda_stream, prepared.copy_stream.cuda_stream))
+
     async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
                                      stream: torch.cuda.Stream) -> None:
         """GPU->Host (kv_worker.py:272-295). With a handle: per layer, wait for the
         model's doorbell, make `stream` wait for `post_events[layer]`, then save
-        that layer of every mapped block."""
+        that layer of every mapped block. The mappings are flattened, checked and
+        uploaded once, before the first layer."""
         handle = self.kv_worker_handle
         if handle is None:
             self.save_kv_blocks_to_host_nowait(block_mappings, stream)
         elif len(block_mappings) > 0:
+            prepared = self.prepare_swap("out", block_mappings, stream)
             for layer_idx in range(self.num_layers):
                 while handle.kv_queue.empty():
                     await asyncio.sleep(1e-5)
                 handle.kv_queue.get()
                 stream.wait_event(handle.post_events[layer_idx])
-                self.save_kv_blocks_to_host_nowait(block_mappings, stream, layer_idx, layer_idx + 1)
+                self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
                 await asyncio.sleep(0)  # let other tasks of the loop run
         await asyncio.to_thread(stream.synchronize)
 
@@ -287,8 +358,9 @@ class KVWorker:
         if handle is None:
             self.load_kv_blocks_from_host_nowait(block_mappings, stream)
         elif len(block_mappings) > 0:
+            prepared = self.prepare_swap("in", block_mappings, stream)
             for layer_idx in range(self.num_layers):
-                self.load_kv_blocks_from_host_nowait(block_mappings, stream, layer_idx, layer_idx + 1)
+                self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
                 await asyncio.sleep(0)
                 handle.pre_events[layer_idx].record(stream)
                 handle.model_queue.put(b"")
@@ -361,3 +433,5 @@ class KVWorker:
             self.disk_tier = None
         self._host_pool.close()
         self._staging = {"out": None, "in": None}
+        # events and id bounce buffers the library kept for this thread
+        _lib.check(_lib.lib().kvc_thread_release())

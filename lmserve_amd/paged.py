@@ -12,6 +12,7 @@ tensor layouts are those calls'; the "NHD" single-tensor cache
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Tuple
 
 import torch
@@ -182,14 +183,15 @@ def append_paged_kv_cache_layers(
 
 
 class PagedKVWritePlan:
-    """The page-table write with its per-step arguments checked ONCE.
+    """The page-table write with its per-step arguments handed over ONCE.
 
     A forward pass calls `append_paged_kv_cache` once per layer with the same
     five index tensors (runtime/worker/llm_worker/models/layers/attention.py:76-85
-    inside the layer loop of models/llama.py:236-242). Building a plan per step
-    (where the reference builds `InputParams`, model_worker.py:435-446) and
-    calling `plan.append(key, value, kv_caches[i])` per layer leaves only three
-    pointer reads and the library call on the host's critical path.
+    inside the layer loop of models/llama.py:236-242). A plan is built per step
+    (where the reference builds `InputParams`, model_worker.py:435-446): the
+    library keeps the index arguments (`kvc_write_plan_create`), and
+    `plan.append(key, value, kv_caches[i])` per layer marshals only the layer's
+    three pointers, their strides and the stream (`kvc_write_plan_append`).
 
     The plan keeps references to the index tensors, so their memory stays valid
     for as long as the plan lives.
@@ -207,47 +209,69 @@ class PagedKVWritePlan:
         self.row = self.H * self.D
         self.nnz = self.batch_indices.numel()
         self.elem = torch.empty(0, dtype=dtype).element_size()
-        self._fn = _lib.lib().kvc_append_paged_kv_cache
-        # [key, value, bi, pos, cache, indices, indptr, last, nnz, B, n_idx, H, D, ps,
-        #  k_stride, v_stride, page_stride, num_pages, elem, stream]
-        self._args = [0, 0, self.batch_indices.data_ptr(), self.positions.data_ptr(), 0,
-                      self.kv_indices.data_ptr(), self.kv_indptr.data_ptr(),
-                      self.kv_last_page_len.data_ptr(), self.nnz, self.kv_indptr.numel() - 1,
-                      self.kv_indices.numel(), self.H, self.D, self.page_size,
-                      self.row, self.row, 2 * self.page_size * self.row, 0, self.elem, 0]
+        lib = _lib.lib()
+        handle = ctypes.c_void_p()
+        _lib.check(lib.kvc_write_plan_create(
+            self.batch_indices.data_ptr(), self.positions.data_ptr(), self.kv_indices.data_ptr(),
+            self.kv_indptr.data_ptr(), self.kv_last_page_len.data_ptr(), self.nnz,
+            self.kv_indptr.numel() - 1, self.kv_indices.numel(), self.H, self.D, self.page_size,
+            self.elem, ctypes.byref(handle)))
+        self._plan = handle.value
+        self._append = lib.kvc_write_plan_append
+        self._destroy = lib.kvc_write_plan_destroy
         self._cache_shape_tail = (2, self.page_size, self.H, self.D)
+        self._dense_page = 2 * self.page_size * self.row
+        self._dev_index = self.device.index
+        self._get_stream = torch._C._cuda_getCurrentRawStream
+
+    def __del__(self):
+        plan, self._plan = getattr(self, "_plan", None), None
+        if plan:
+            self._destroy(plan)
+
+    def _row_stride(self, t: torch.Tensor, name: str) -> int:
+        """Token stride of `[nnz, H, D]` / `[nnz, H*D]` rows that are dense inside a token."""
+        if t.dtype != self.dtype or t.device != self.device:
+            raise TypeError(f"{name} must have the plan's dtype and device")
+        st = t.stride()
+        if t.dim() == 3:
+            ok = st[2] == 1 and (st[1] == self.D or self.H == 1) and t.shape[1] * t.shape[2] == self.row
+        else:
+            ok = t.dim() == 2 and st[1] == 1 and t.shape[1] == self.row
+        if not ok or t.shape[0] < self.nnz:
+            raise ValueError(f"{name} must be [nnz, H, D] (or [nnz, H*D]) with dense rows")
+        if self.nnz > 1 and st[0] < self.row:
+            raise ValueError(f"{name} rows overlap (token stride {st[0]} < {self.row})")
+        return st[0] if self.nnz > 1 else self.row
 
     def append(self, append_key: torch.Tensor, append_value: torch.Tensor,
                paged_kv_cache: torch.Tensor) -> None:
         """`append_paged_kv_cache` for one layer. Requirements (checked): key/value
-        dense `[nnz, H, D]` (or `[nnz, H*D]`) of the plan's dtype on its device,
-        `paged_kv_cache` `[num_pages, 2, page_size, H, D]` with contiguous pages."""
+        `[nnz, H, D]` (or `[nnz, H*D]`) of the plan's dtype on its device with dense
+        rows (any token stride: slices of a fused QKV projection are read in
+        place), `paged_kv_cache` `[num_pages, 2, page_size, H, D]` with contiguous
+        pages. Launches on the current stream of the plan's device, which must be
+        the current device."""
         if self.nnz == 0:
             return
-        if append_key.dtype != self.dtype or append_value.dtype != self.dtype \
-                or paged_kv_cache.dtype != self.dtype:
-            raise TypeError("append_key/append_value/paged_kv_cache must have the plan's dtype")
-        if append_key.device != self.device or append_value.device != self.device \
-                or paged_kv_cache.device != self.device:
-            raise ValueError("tensors must live on the plan's device")
-        if tuple(paged_kv_cache.shape[1:]) != self._cache_shape_tail or \
-                not _inner_contiguous(paged_kv_cache):
-            raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
-        if not append_key.is_contiguous() or not append_value.is_contiguous() \
-                or append_key.numel() < self.nnz * self.row or append_value.numel() < self.nnz * self.row:
-            raise ValueError("append_key/append_value must be dense [nnz, H, D]")
-        num_pages = paged_kv_cache.shape[0]
+        k_stride = self._row_stride(append_key, "append_key")
+        v_stride = self._row_stride(append_value, "append_value")
+        shape = paged_kv_cache.shape
+        if paged_kv_cache.dtype != self.dtype or paged_kv_cache.device != self.device:
+            raise TypeError("paged_kv_cache must have the plan's dtype and device")
+        num_pages = shape[0]
         if num_pages == 0:
             return
-        a = self._args
-        a[0] = append_key.data_ptr()
-        a[1] = append_value.data_ptr()
-        a[4] = paged_kv_cache.data_ptr()
-        a[16] = paged_kv_cache.stride(0) if num_pages > 1 else 2 * self.page_size * self.row
-        a[17] = num_pages
-        a[19] = _stream_of(paged_kv_cache)
-        with _on_device_of(paged_kv_cache):
-            _lib.check(self._fn(*a))
+        st = paged_kv_cache.stride()
+        if tuple(shape[1:]) != self._cache_shape_tail or st[4] != 1 or st[3] != self.D \
+                or st[2] != self.row or st[1] != self.page_size * self.row:
+            raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
+        rc = self._append(self._plan, append_key.data_ptr(), append_value.data_ptr(), k_stride,
+                          v_stride, paged_kv_cache.data_ptr(),
+                          st[0] if num_pages > 1 else self._dense_page, num_pages,
+                          self._get_stream(self._dev_index))
+        if rc:
+            _lib.check(rc)
 
 
 def build_write_index(input_lens: torch.Tensor, context_lens: torch.Tensor,

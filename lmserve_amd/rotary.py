@@ -13,6 +13,7 @@ Arithmetic: fp32 with one rounding to the tensors' dtype.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Optional, Tuple
 
@@ -233,26 +234,39 @@ class PagedRotaryWritePlan:
         self.Hq, self.H, self.D, self.page_size = int(num_heads), int(num_kv_heads), int(head_dim), int(page_size)
         self.nnz = positions.numel()
         self.q_row, self.kv_row = self.Hq * self.D, self.H * self.D
-        self._fn = _lib.lib().kvc_rotary_pos_emb_and_append_paged
-        # [q, k, v, bi, pos, cs, max_pos, nnz, Hq, H, D, rd, q_stride, k_stride, v_stride, q_out, k_out,
-        #  qo_stride, ko_stride, cache, indices, indptr, B, n_idx, page_size, page_stride, num_pages,
-        #  dtype, stream]
-        self._args = [0, 0, 0, batch_indices.data_ptr(), positions.data_ptr(), cos_sin_cache.data_ptr(),
-                      cos_sin_cache.shape[0], self.nnz, self.Hq, self.H, self.D,
-                      cos_sin_cache.shape[1] // 2, 0, 0, 0, 0, None, self.q_row, self.kv_row, 0,
-                      kv_indices.data_ptr(), kv_indptr.data_ptr(), kv_indptr.numel() - 1,
-                      kv_indices.numel(), self.page_size, 0, 0, self.kd, 0]
+        lib = _lib.lib()
+        handle = ctypes.c_void_p()
+        _lib.check(lib.kvc_rotary_plan_create(
+            batch_indices.data_ptr(), positions.data_ptr(), cos_sin_cache.data_ptr(),
+            cos_sin_cache.shape[0], self.nnz, self.Hq, self.H, self.D, cos_sin_cache.shape[1] // 2,
+            kv_indices.data_ptr(), kv_indptr.data_ptr(), kv_indptr.numel() - 1, kv_indices.numel(),
+            self.page_size, self.kd, ctypes.byref(handle)))
+        self._plan = handle.value
+        self._run = lib.kvc_rotary_plan_run
+        self._destroy = lib.kvc_rotary_plan_destroy
         self._cache_shape_tail = (2, self.page_size, self.H, self.D)
+        self._dense_page = 2 * self.page_size * self.kv_row
+        self._dev_index = self.device.index
+        self._get_stream = torch._C._cuda_getCurrentRawStream
 
-    def _rows(self, t: torch.Tensor, width: int, name: str) -> int:
+    def __del__(self):
+        plan, self._plan = getattr(self, "_plan", None), None
+        if plan:
+            self._destroy(plan)
+
+    def _rows(self, t: torch.Tensor, width: int, name: str, dense: bool = False) -> int:
         """Token stride (elements) of a `[nnz, width]` / `[nnz, heads, D]` tensor with dense rows."""
         if t.dtype != self.dtype or t.device != self.device:
             raise TypeError(f"{name} must have the plan's dtype and device")
+        st = t.stride()
         if t.shape[0] != self.nnz or t.numel() != self.nnz * width:
             raise ValueError(f"{name} must hold [nnz, {width}] elements")
-        if t.stride(-1) != 1 or (t.dim() == 3 and t.stride(1) != t.shape[2]):
+        if st[-1] != 1 or (t.dim() == 3 and st[1] != t.shape[2]):
             raise ValueError(f"{name} rows must be dense")
-        return t.stride(0) if self.nnz > 1 else width
+        stride = st[0] if self.nnz > 1 else width
+        if stride < width or (dense and stride != width):
+            raise ValueError(f"{name} must have {'contiguous' if dense else 'non-overlapping'} rows")
+        return stride
 
     def run(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
             paged_kv_cache: torch.Tensor, query_out: torch.Tensor = None,
@@ -260,7 +274,9 @@ class PagedRotaryWritePlan:
         """One layer: rotates `query` and `key`, writes the rotated key and `value`
         into the pages. Returns `(query_out, key_out)`; `key_out` is None unless a
         buffer is given or `return_key` is set. Token-strided inputs (slices of a
-        fused QKV projection) are read in place."""
+        fused QKV projection) are read in place; the output buffers are contiguous.
+        Launches on the current stream of the plan's device, which must be the
+        current device."""
         if query_out is None:
             query_out = torch.empty((self.nnz, self.q_row), dtype=self.dtype, device=self.device)
         if key_out is None and return_key:
@@ -269,30 +285,27 @@ class PagedRotaryWritePlan:
             return query_out, key_out
         if paged_kv_cache.dtype != self.dtype or paged_kv_cache.device != self.device:
             raise TypeError("paged_kv_cache must have the plan's dtype and device")
-        if tuple(paged_kv_cache.shape[1:]) != self._cache_shape_tail or \
-                not _inner_contiguous(paged_kv_cache):
+        shape, st = paged_kv_cache.shape, paged_kv_cache.stride()
+        if tuple(shape[1:]) != self._cache_shape_tail or st[4] != 1 or st[3] != self.D \
+                or st[2] != self.kv_row or st[1] != self.page_size * self.kv_row:
             raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
-        num_pages = paged_kv_cache.shape[0]
-        a = self._args
-        a[12] = self._rows(query, self.q_row, "query")
-        a[13] = self._rows(key, self.kv_row, "key")
-        a[14] = self._rows(value, self.kv_row, "value")
-        a[17] = self._rows(query_out, self.q_row, "query_out")
-        a[0], a[1], a[2] = query.data_ptr(), key.data_ptr(), value.data_ptr()
-        a[15] = query_out.data_ptr()
-        if key_out is not None:
-            a[18] = self._rows(key_out, self.kv_row, "key_out")
-            a[16] = key_out.data_ptr()
-        else:
-            a[16] = None
+        num_pages = shape[0]
         if num_pages == 0:
             raise ValueError("paged_kv_cache has no pages")
-        a[19] = paged_kv_cache.data_ptr()
-        a[25] = paged_kv_cache.stride(0) if num_pages > 1 else 2 * self.page_size * self.kv_row
-        a[26] = num_pages
-        a[28] = _stream_of(paged_kv_cache)
-        with _on_device_of(paged_kv_cache):
-            _lib.check(self._fn(*a))
+        q_stride = self._rows(query, self.q_row, "query")
+        k_stride = self._rows(key, self.kv_row, "key")
+        v_stride = self._rows(value, self.kv_row, "value")
+        self._rows(query_out, self.q_row, "query_out", dense=True)
+        ko_ptr = None
+        if key_out is not None:
+            self._rows(key_out, self.kv_row, "key_out", dense=True)
+            ko_ptr = key_out.data_ptr()
+        rc = self._run(self._plan, query.data_ptr(), key.data_ptr(), value.data_ptr(), q_stride,
+                       k_stride, v_stride, query_out.data_ptr(), ko_ptr, paged_kv_cache.data_ptr(),
+                       st[0] if num_pages > 1 else self._dense_page, num_pages,
+                       self._get_stream(self._dev_index))
+        if rc:
+            _lib.check(rc)
         return query_out, key_out
 
 

@@ -25,3 +25,15 @@ def gpu():
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     _lib.lib()  # raises if libkvcache.so is not built
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def default_tuning():
+    """Every test starts and ends with the library's launch-shape knobs at their
+    defaults, whatever an earlier test set."""
+    from lmserve_amd import _lib
+
+    L = _lib.lib()
+    assert L.kvc_tuning_modified() == 0, "a tuning knob was left modified by an earlier test"
+    yield
+    _lib.reset_tuning()

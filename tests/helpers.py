@@ -40,3 +40,38 @@ def to_bf16(a: np.ndarray, device=None) -> torch.Tensor:
 def bits_of(t: torch.Tensor) -> np.ndarray:
     """torch tensor of a 16-bit dtype -> uint16 bit patterns on the host."""
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+class FifoBlockIds:
+    """Block ids in the order the reference's allocator produces them under churn
+    (runtime/src/llm_engine/block_manager.rs:62-140): ids are taken from the front
+    of a queue that starts as 0..n-1 and go to its back when their last user
+    lets go, so live block tables end up scattered over the pool. Test input
+    generator only."""
+
+    def __init__(self, n: int):
+        from collections import deque
+        self.queue = deque(range(n))
+        self.users = [0] * n
+
+    def take(self, count: int = 1):
+        if count > len(self.queue):
+            raise RuntimeError("no free block ids left")
+        ids = [self.queue.popleft() for _ in range(count)]
+        for i in ids:
+            self.users[i] = 1
+        return ids
+
+    def share(self, block_id: int) -> int:
+        """One more user of a block (prefix sharing); a free id is claimed."""
+        if self.users[block_id] == 0:
+            self.queue.remove(block_id)
+        self.users[block_id] += 1
+        return block_id
+
+    def give_back(self, ids) -> None:
+        for i in ids:
+            assert self.users[i] > 0, f"block {i} given back twice"
+            self.users[i] -= 1
+            if self.users[i] == 0:
+                self.queue.append(i)

@@ -4,6 +4,7 @@
 // (oracle/kvc_oracle.c, linked in) or with arrays written out by hand.
 // Exit status 0 and a final "ABI CHECK PASSED" line on success.
 #include <hip/hip_runtime.h>
+#include <time.h>
 #include <unistd.h>
 
 #include <cstdint>
@@ -144,6 +145,73 @@ int main() {
   expect_equal("kvc_append_paged_kv_cache == oracle", got.data(), want_paged.data(), pool_bytes);
   expect_equal("page-table write == slot-mapped write", want_paged.data(), want.data(), pool_bytes);
 
+  // 3b. the same page-table write through a per-step plan: three pointers per layer
+  {
+    HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+    kvc_write_plan* plan = nullptr;
+    KVC_OK_OR_DIE(kvc_write_plan_create((const int32_t*)d_bi, (const int32_t*)d_pos, (const int32_t*)d_ind,
+                                        (const int32_t*)d_ptr, (const int32_t*)d_last, T, 2,
+                                        (int64_t)kv_indices.size(), H, D, bs, (int)E, &plan));
+    for (int64_t l = 0; l < L; ++l)
+      KVC_OK_OR_DIE(kvc_write_plan_append(plan, (char*)d_key + l * T * row * E,
+                                          (char*)d_value + l * T * row * E, row, row,
+                                          (char*)d_pool + l * layer_elems * E, blk_elems, nb, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+    expect_equal("kvc_write_plan_append == oracle", got.data(), want_paged.data(), pool_bytes);
+    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS_NARROW ||
+        kvc_last_launch_info(KVC_LAUNCH_VEC_BYTES) != 16) {
+      std::fprintf(stderr, "256-byte rows did not take the narrow-row kernel\n");
+      ++fails;
+    }
+    // host cost of one planned launch (informational)
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    const int reps = 2000;
+    timespec t0, t1;
+    HIP_OK(hipEventRecord(e0, stream));
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (int i = 0; i < reps; ++i)
+      KVC_OK_OR_DIE(kvc_write_plan_append(plan, d_key, d_value, row, row, d_pool, blk_elems, nb, stream));
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    HIP_OK(hipEventRecord(e1, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    float ms = 0;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    std::printf("kvc_write_plan_append: %.2f us of host time per call, %.2f us per call on the stream\n",
+                ((t1.tv_sec - t0.tv_sec) * 1e9 + (t1.tv_nsec - t0.tv_nsec)) / 1e3 / reps, ms * 1e3 / reps);
+    HIP_OK(hipEventDestroy(e0));
+    HIP_OK(hipEventDestroy(e1));
+    KVC_OK_OR_DIE(kvc_write_plan_destroy(plan));
+    if (kvc_write_plan_append(nullptr, d_key, d_value, row, row, d_pool, blk_elems, nb, stream) !=
+        KVC_ERR_INVALID_ARG) {
+      std::fprintf(stderr, "expected KVC_ERR_INVALID_ARG for a null plan\n");
+      ++fails;
+    }
+    // tuning knobs: set, read back, reset
+    int v = -1;
+    KVC_OK_OR_DIE(kvc_set_tuning("write_narrow", 0));
+    KVC_OK_OR_DIE(kvc_get_tuning("write_narrow", &v));
+    if (v != 0 || kvc_tuning_modified() != 1) { std::fprintf(stderr, "tuning read-back failed\n"); ++fails; }
+    HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+    for (int64_t l = 0; l < L; ++l)
+      KVC_OK_OR_DIE(kvc_reshape_and_cache((char*)d_key + l * T * row * E, (char*)d_value + l * T * row * E,
+                                          (char*)d_pool + l * layer_elems * E,
+                                          (char*)d_pool + l * layer_elems * E + bs * row * E, d_slots, 8, T,
+                                          row, row, row, bs, blk_elems, row, nb, (int)E, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+    expect_equal("token-per-workgroup kernel on 256-byte rows == oracle", got.data(), want.data(), pool_bytes);
+    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS) {
+      std::fprintf(stderr, "write_narrow = 0 did not select the token-per-workgroup kernel\n");
+      ++fails;
+    }
+    KVC_OK_OR_DIE(kvc_reset_tuning());
+    KVC_OK_OR_DIE(kvc_get_tuning("write_narrow", &v));
+    if (v != 1 || kvc_tuning_modified() != 0) { std::fprintf(stderr, "tuning reset failed\n"); ++fails; }
+  }
+
   // 4. copy_blocks
   std::vector<int64_t> maps = {7, 0, 7, 1, 19, 30, 5, 5, 40, 47};
   HIP_OK(hipMalloc(&d_maps, maps.size() * 8));
@@ -185,6 +253,40 @@ int main() {
     HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
     expect_equal(mode ? "kvc_swap_in (direct) == oracle" : "kvc_swap_in (staged) == oracle", got.data(),
                  want.data(), pool_bytes);
+    // the same ids checked and uploaded once, then one call per layer
+    {
+      std::vector<int64_t> p_gpu = {1, 46, 22, 9}, p_host = {1, 5, 7, 8};
+      KVC_OK_OR_DIE(kvc_swap_prepare(p_gpu.data(), p_host.data(), 4, nb, nhb, staging, staging_bytes, stream));
+      for (int64_t l = 0; l < L; ++l)
+        KVC_OK_OR_DIE(kvc_swap_out_prepared(d_pool, host, p_host.data(), 4, L, layer_elems * E, blk_bytes,
+                                            nb, nhb, l, l + 1, staging, staging_bytes, mode, stream,
+                                            copy_stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      oracle_save_blocks_to_host(want.data(), want_host.data(), p_gpu.data(), p_host.data(), 4, L, nb,
+                                 blk_bytes, 0, L);
+      expect_equal(mode ? "kvc_swap_out_prepared per layer (direct) == oracle"
+                        : "kvc_swap_out_prepared per layer (staged) == oracle",
+                   host, want_host.data(), host_bytes);
+      std::vector<int64_t> q_gpu = {33, 34, 35, 2};
+      KVC_OK_OR_DIE(kvc_swap_prepare(q_gpu.data(), p_host.data(), 4, nb, nhb, staging, staging_bytes, stream));
+      for (int64_t l = L; l-- > 0;)
+        KVC_OK_OR_DIE(kvc_swap_in_prepared(d_pool, host, p_host.data(), 4, L, layer_elems * E, blk_bytes,
+                                           nb, nhb, l, l + 1, staging, staging_bytes, mode, stream,
+                                           copy_stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      oracle_load_blocks_from_host(want.data(), want_host.data(), p_host.data(), q_gpu.data(), 4, L, nb,
+                                   blk_bytes, 0, L);
+      HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+      expect_equal(mode ? "kvc_swap_in_prepared per layer (direct) == oracle"
+                        : "kvc_swap_in_prepared per layer (staged) == oracle",
+                   got.data(), want.data(), pool_bytes);
+      std::vector<int64_t> bad_gpu = {nb};
+      if (kvc_swap_prepare(bad_gpu.data(), p_host.data(), 1, nb, nhb, staging, staging_bytes, stream) !=
+          KVC_ERR_OUT_OF_RANGE) {
+        std::fprintf(stderr, "expected KVC_ERR_OUT_OF_RANGE from kvc_swap_prepare\n");
+        ++fails;
+      }
+    }
     // an id outside the host pool is rejected before anything runs
     std::vector<int64_t> bad = {nhb};
     const int rc = kvc_swap_out(d_pool, host, out_src.data(), bad.data(), 1, L, layer_elems * E,
@@ -295,6 +397,7 @@ int main() {
     KVC_OK_OR_DIE(kvc_host_free_pinned(host));
   }
 
+  KVC_OK_OR_DIE(kvc_thread_release());
   HIP_OK(hipDeviceSynchronize());
   if (fails) {
     std::printf("ABI CHECK FAILED (%d mismatches)\n", fails);

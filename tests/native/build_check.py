@@ -38,8 +38,16 @@ def build_native_check(verbose: bool = False) -> str:
 
 
 def ensure_native_check() -> str:
-    """Use the built binary; build only if there is none."""
-    if not os.path.exists(NATIVE_CHECK_BIN):
+    """Use the built binary; build it if there is none, or if it is older than
+    its source and a compiler is at hand."""
+    stale = os.path.exists(NATIVE_CHECK_BIN) and \
+        os.path.getmtime(NATIVE_CHECK_BIN) < os.path.getmtime(NATIVE_CHECK_SRC)
+    if stale:
+        try:
+            find_hipcc()
+        except RuntimeError:
+            stale = False
+    if stale or not os.path.exists(NATIVE_CHECK_BIN):
         build_native_check(verbose=True)
     return NATIVE_CHECK_BIN
 

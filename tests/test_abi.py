@@ -56,7 +56,7 @@ def test_binding_arity_matches_the_header():
 
 
 def test_abi_version():
-    assert _lib.lib().kvc_abi_version() == 1
+    assert _lib.lib().kvc_abi_version() == _lib.KVC_ABI_VERSION
 
 
 def test_argument_validation_returns_codes_not_crashes():
@@ -145,6 +145,84 @@ def test_rope_and_index_build_validate_their_arguments():
     assert g(None, None, None, None, 2, 0, 16, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
     assert g(1, 1, 1, 1, 2, 4, 0, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG   # page_size 0
     assert L.kvc_set_tuning(b"no_such_knob", 1) == _lib.KVC_ERR_INVALID_ARG
+
+
+def test_tuning_knobs_read_back_and_reset():
+    L = _lib.lib()
+    assert L.kvc_tuning_modified() == 0
+    defaults = {"copy_unroll": 0, "gather_unroll": 0, "copy_nt": 1, "copy_max_wgs": 0, "copy_order": 0,
+                "write_vpt": 0, "write_nt": 1, "write_order": 0, "write_threads": 0, "write_narrow": 1,
+                "write_narrow_vpt": 0, "direct_max_wgs": 64, "rope_threads": 0, "disk_bounce_mib": 4}
+    for key, value in defaults.items():
+        assert _lib.get_tuning(key) == value, key
+    for i, key in enumerate(defaults):
+        _lib.set_tuning(key, 100 + i)
+        assert _lib.get_tuning(key) == 100 + i
+        assert L.kvc_tuning_modified() == i + 1
+    _lib.reset_tuning()
+    assert L.kvc_tuning_modified() == 0
+    for key, value in defaults.items():
+        assert _lib.get_tuning(key) == value, key
+    out = ctypes.c_int(0)
+    assert L.kvc_get_tuning(b"no_such_knob", ctypes.byref(out)) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_get_tuning(b"copy_nt", None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_last_launch_info(99) == _lib.KVC_ERR_INVALID_ARG
+    assert _lib.last_launch()["kernel"] == _lib.KVC_KERNEL_NONE     # nothing launched in this process
+
+
+def test_plans_and_prepared_swap_validate_before_touching_the_gpu():
+    L = _lib.lib()
+    h = ctypes.c_void_p()
+    create = L.kvc_write_plan_create
+    assert create(1, 1, 1, 1, 1, 4, 2, 8, 8, 128, 16, 2, ctypes.byref(h)) == _lib.KVC_OK and h.value
+    # a null key pointer is caught by the write's own checks, before any launch
+    assert L.kvc_write_plan_append(h, None, 1, 1024, 1024, 1, 32768, 4, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_write_plan_append(h, 1, 1, 512, 1024, 1, 32768, 4, None) == _lib.KVC_ERR_INVALID_ARG
+    assert "stride" in _lib.last_error()
+    assert L.kvc_write_plan_destroy(h) == _lib.KVC_OK
+    assert L.kvc_write_plan_destroy(None) == _lib.KVC_OK
+    assert create(1, 1, 1, 1, 1, 4, 2, 8, 8, 128, 0, 2, ctypes.byref(h)) == _lib.KVC_ERR_INVALID_ARG
+    assert h.value is None
+    assert create(1, 1, 1, 1, 1, 4, 2, 8, 8, 128, 16, 3, ctypes.byref(h)) == _lib.KVC_ERR_UNSUPPORTED
+    assert create(None, 1, 1, 1, 1, 4, 2, 8, 8, 128, 16, 2, ctypes.byref(h)) == _lib.KVC_ERR_INVALID_ARG
+    assert create(1, 1, 1, 1, 1, 4, 2, 8, 8, 128, 16, 2, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_write_plan_append(None, 1, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
+
+    rcreate = L.kvc_rotary_plan_create
+    #        bi pos cs max nnz Hq Hkv D rd idx ptr B nidx ps dtype out
+    assert rcreate(1, 1, 1, 100, 4, 8, 2, 64, 64, 1, 1, 2, 8, 16, 0, ctypes.byref(h)) == _lib.KVC_OK
+    assert L.kvc_rotary_plan_run(h, None, 1, 1, 512, 128, 128, 1, None, 1, 4096, 4, None) == \
+        _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_rotary_plan_destroy(h) == _lib.KVC_OK
+    assert rcreate(1, 1, 1, 100, 4, 8, 2, 64, 63, 1, 1, 2, 8, 16, 0, ctypes.byref(h)) == _lib.KVC_ERR_INVALID_ARG
+    assert rcreate(1, 1, 1, 100, 4, 8, 2, 64, 64, 1, 1, 2, 8, 16, 9, ctypes.byref(h)) == _lib.KVC_ERR_UNSUPPORTED
+    assert rcreate(1, 1, None, 100, 4, 8, 2, 64, 64, 1, 1, 2, 8, 16, 0, ctypes.byref(h)) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_rotary_plan_run(None, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
+
+    ids = np.asarray([0, 5, 63], dtype=np.int64)
+    bad = np.asarray([0, 64, 1], dtype=np.int64)
+    prep = L.kvc_swap_prepare
+    assert prep(None, None, 0, 64, 8, None, 0, None) == _lib.KVC_OK            # nothing to prepare
+    assert prep(bad.ctypes.data, ids.ctypes.data, 3, 64, 64, 4096, 4096, None) == _lib.KVC_ERR_OUT_OF_RANGE
+    assert "gpu block id 64" in _lib.last_error()
+    assert prep(ids.ctypes.data, bad.ctypes.data, 3, 64, 64, 4096, 4096, None) == _lib.KVC_ERR_OUT_OF_RANGE
+    assert prep(ids.ctypes.data, None, 3, 64, 64, 4096, 4096, None) == _lib.KVC_ERR_INVALID_ARG
+    assert prep(ids.ctypes.data, ids.ctypes.data, 3, 64, 64, None, 4096, None) == _lib.KVC_ERR_STAGING
+    assert prep(ids.ctypes.data, ids.ctypes.data, 3, 64, 64, 4096 + 8, 4096, None) == _lib.KVC_ERR_STAGING
+    assert prep(ids.ctypes.data, ids.ctypes.data, 3, 64, 64, 4096, 16, None) == _lib.KVC_ERR_STAGING
+    out = L.kvc_swap_out_prepared
+    #  pool host host_ids n L layer_stride block nb nhb lb le staging bytes mode ks cs
+    assert out(4096, 4096, None, 3, 2, 65536, 1024, 64, 64, 0, 2, 4096, 4096, _lib.KVC_SWAP_STAGED,
+               None, None) == _lib.KVC_ERR_INVALID_ARG                          # staged needs the host ids
+    assert out(4096, 4096, None, 3, 2, 65536, 1024, 64, 64, 1, 3, 4096, 4096, _lib.KVC_SWAP_DIRECT,
+               None, None) == _lib.KVC_ERR_INVALID_ARG                          # layer range
+    assert out(4096, 4096, None, 3, 2, 65536, 1024, 64, 64, 0, 2, 4096, 16, _lib.KVC_SWAP_DIRECT,
+               None, None) == _lib.KVC_ERR_STAGING
+    assert out(4096, 4096, None, 0, 2, 65536, 1024, 64, 64, 0, 2, None, 0, _lib.KVC_SWAP_DIRECT,
+               None, None) == _lib.KVC_OK
+    assert L.kvc_swap_in_prepared(None, 4096, None, 3, 2, 65536, 1024, 64, 64, 0, 2, 4096, 4096,
+                                  _lib.KVC_SWAP_DIRECT, None, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_thread_release() == _lib.KVC_OK       # nothing held by this thread: a no-op
 
 
 def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):

@@ -70,15 +70,14 @@ def test_copy_blocks_every_launch_shape(gpu, unroll, nt, max_wgs):
     s = wl.LLAMA_3_8B
     L, nb = 2, 64
     _, d = wl.copy_on_write_pairs(nb, 13, seed=unroll)
-    _lib.set_tuning("copy_unroll", unroll)
+    _lib.set_tuning("copy_unroll", unroll)     # the autouse fixture puts the defaults back
     _lib.set_tuning("copy_nt", nt)
     _lib.set_tuning("copy_max_wgs", max_wgs)
-    try:
-        got, want, _ = _run(gpu, (L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), d, seed=8)
-    finally:
-        _lib.set_tuning("copy_unroll", 4)
-        _lib.set_tuning("copy_nt", 1)
-        _lib.set_tuning("copy_max_wgs", 0)
+    got, want, _ = _run(gpu, (L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), d, seed=8)
+    ran = _lib.last_launch()
+    assert ran["kernel"] == _lib.KVC_KERNEL_COPY_TILES and ran["per_lane"] == unroll
+    assert ran["non_temporal"] == nt and ran["vec_bytes"] == 16
+    assert ran["grid"] == (7 if max_wgs else 13 * L * (65536 // (256 * 16 * unroll)))
     assert np.array_equal(got, want)
 
 
@@ -127,11 +126,19 @@ def test_every_launch_shape_the_size_rule_picks_matches_the_oracle(gpu, n):
     want = pool.copy()
     orc.c_copy_blocks(want, flat)
     dpool = to_bf16(pool, gpu)
+    assert _lib.lib().kvc_tuning_modified() == 0 and _lib.get_tuning("copy_unroll") == 0
+    # vectors per lane the size rule must pick on a 256-CU part (2048 resident workgroups):
+    # the smallest depth that fits n * 32 tiles of 64 KiB into 512 workgroups, a whole tile
+    # per workgroup while that stays within 1024, else 2 (copy, scatter) or 1 (gather)
+    small = {1: 1, 2: 2, 4: 4, 8: 8, 16: 16, 32: 16}
     kvc.copy_blocks(dpool, pairs)
+    assert _lib.last_launch()["per_lane"] == small.get(n, 2)
     ids = torch.from_numpy(flat[1::2].copy()).to(gpu)               # the blocks just written
     dense = kvc.gather_blocks(dpool, ids)
+    assert _lib.last_launch()["per_lane"] == small.get(n, 1)
     back = torch.from_numpy(flat[0::2].copy()).to(gpu)              # scatter them over their sources
     kvc.scatter_blocks(dpool, back, dense)
+    assert _lib.last_launch()["per_lane"] == small.get(n, 2)
     torch.cuda.synchronize()
     view = want.reshape(L, nb, -1)
     want_dense = view[:, flat[1::2]].swapaxes(0, 1)

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import lmserve_amd as kvc
+from lmserve_amd import _lib
 from lmserve_amd import workloads as wl
 
 pytestmark = pytest.mark.gpu
@@ -53,7 +54,12 @@ def test_config2_decode_write_full_pool(gpu):
     slots = w.index.slot_mapping
     assert (slots.max() // bs) * s.block_elems >= 2 ** 31 - 2 ** 27   # blocks reach the top of a layer
 
+    assert _lib.lib().kvc_tuning_modified() == 0
     kvc.reshape_and_cache_layers(key, value, pool, idx.slot_mapping)
+    ran = _lib.last_launch()
+    # the headline launch: exactly one resident set of 128-lane workgroups, 4 vectors per lane
+    assert (ran["kernel"], ran["vec_bytes"], ran["per_lane"], ran["threads"], ran["grid"]) == \
+        (_lib.KVC_KERNEL_WRITE_ROWS, 16, 4, 128, 4096)
     assert _check_write(pool, key, value, slots, bs) > 0
     _clear_slots(pool, slots, bs)
     assert int(torch.count_nonzero(pool[L - 1].view(torch.int16))) == 0
@@ -119,7 +125,14 @@ def test_config4_copy_blocks_full_pool(gpu):
     blk_term, elem_term = _pattern_terms(nb, pool3.shape[2], gpu)
     _fill_pattern(pool3, blk_term, elem_term)
     flat, pairs = wl.copy_on_write_pairs(nb, 4096, seed=0)
+    assert _lib.lib().kvc_tuning_modified() == 0     # the launch shape is the library's own choice
     kvc.copy_blocks(pool, pairs, validate=True)
+    ran = _lib.last_launch()
+    # the instantiation the benchmark times for this configuration: 16-byte vectors,
+    # two per lane, non-temporal, one workgroup per 8 KiB chunk
+    assert (ran["kernel"], ran["vec_bytes"], ran["per_lane"], ran["non_temporal"]) == \
+        (_lib.KVC_KERNEL_COPY_TILES, 16, 2, 1)
+    assert ran["grid"] == 4096 * L * 8
     holder = torch.arange(nb, device=gpu)
     holder[torch.from_numpy(flat[1::2]).to(gpu)] = torch.from_numpy(flat[0::2]).to(gpu)
     _check_pattern(pool3, holder, blk_term, elem_term, "copy_blocks")
@@ -159,3 +172,32 @@ def test_config5_swap_round_trip_full(gpu, mode):
     holder = torch.arange(nb, device=gpu)
     holder[torch.from_numpy(new).to(gpu)] = torch.from_numpy(old).to(gpu)
     _check_pattern(pool3, holder, blk_term, elem_term, f"swap round trip ({mode})")
+
+
+def test_config5_swap_layer_by_layer_with_ids_uploaded_once(gpu):
+    """The same round trip issued as the layer-pipelined protocol issues it: the id
+    lists are checked and uploaded once per direction, then one launch per layer
+    (80 + 80 calls of 8192 blocks x 64 KiB)."""
+    s = wl.LLAMA_3_1_70B
+    nb, L, n = 16384, s.num_layers, SWAP_BLOCKS
+    pool = torch.empty(L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16,
+                       device=gpu)
+    pool3 = pool.view(torch.int16).view(L, nb, -1)
+    blk_term, elem_term = _pattern_terms(nb, pool3.shape[2], gpu)
+    _fill_pattern(pool3, blk_term, elem_term)
+    old, host_ids, new = wl.swap_round_trip(nb, n, seed=1)
+    worker = kvc.KVWorker(pool, n, swap_mode="direct")
+    try:
+        out = worker.prepare_swap("out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))])
+        for l in range(L):
+            worker.swap_prepared_layers(out, l, l + 1)
+        worker.dtoh_stream.synchronize()
+        back = worker.prepare_swap("in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))])
+        for l in range(L):
+            worker.swap_prepared_layers(back, l, l + 1)
+        worker.htod_stream.synchronize()
+    finally:
+        worker.close()
+    holder = torch.arange(nb, device=gpu)
+    holder[torch.from_numpy(new).to(gpu)] = torch.from_numpy(old).to(gpu)
+    _check_pattern(pool3, holder, blk_term, elem_term, "layer-by-layer swap round trip")

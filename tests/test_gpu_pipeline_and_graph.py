@@ -10,7 +10,7 @@ import torch
 import lmserve_amd as kvc
 from lmserve_amd import workloads as wl
 from oracle import kvc_oracle as orc
-from tests.helpers import bf16_bits, bits_of, random_pool, sentinel_pool, to_bf16
+from tests.helpers import FifoBlockIds, bf16_bits, bits_of, random_pool, sentinel_pool, to_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -123,15 +123,15 @@ def test_allocator_order_drives_a_realistic_decode_step(gpu):
     the page-table path, equal the oracle."""
     s = wl.LLAMA_3_2_1B
     nb, bs, L = 128, s.block_size, 2
-    alloc = kvc.BlockAllocator(nb)
+    alloc = FifoBlockIds(nb)
     rng = np.random.default_rng(0)
     live = {}
     for step in range(40):                                    # churn: sequences come and go
         sid = step
-        live[sid] = alloc.alloc_blocks(int(rng.integers(1, 6)))
+        live[sid] = alloc.take(int(rng.integers(1, 6)))
         if len(live) > 8:
             victim = list(live)[int(rng.integers(0, len(live)))]
-            alloc.free_blocks(live.pop(victim))
+            alloc.give_back(live.pop(victim))
     reqs = []
     for i, (sid, blocks) in enumerate(live.items()):
         ctx = int(rng.integers((len(blocks) - 1) * bs + 1, len(blocks) * bs + 1))

@@ -98,6 +98,71 @@ def test_swap_layer_ranges_compose_to_the_full_swap(gpu, mode):
 
 
 @pytest.mark.parametrize("mode", MODES)
+def test_prepared_swap_per_layer_equals_the_oracle(gpu, mode):
+    """Ids checked and uploaded once (`kvc_swap_prepare`), then one call per layer
+    range (`kvc_swap_out_prepared` / `kvc_swap_in_prepared`): every intermediate
+    state of the host pool and of the GPU pool equals the oracle's, in both
+    transfer modes; several swaps prepared back to back keep their own id lists."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb, n = 6, 40, 20, 9
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, mode, chunk=2, seed=21)
+    try:
+        rng = np.random.default_rng(22)
+        perm = rng.permutation(nb)
+        old, new = perm[:n].astype(np.int64), perm[n:2 * n].astype(np.int64)
+        host_ids = rng.permutation(nhb)[:n].astype(np.int64)
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        host_np = w.host_kv_caches.copy()
+        out = w.prepare_swap("out", _mappings(old, host_ids))
+        assert out.n == n
+        for lb, le in ((0, 1), (1, 2), (2, 5), (5, 6)):
+            orc.save_blocks_to_host_np(gpu_np, host_np, old, host_ids, lb, le)
+            w.swap_prepared_layers(out, lb, le)
+            w.dtoh_stream.synchronize()
+            assert np.array_equal(w.host_kv_caches, host_np), (lb, le)
+        back = w.prepare_swap("in", _mappings(host_ids, new))
+        for lb, le in ((4, 6), (0, 4)):
+            orc.load_blocks_from_host_np(gpu_np, host_np, host_ids, new, lb, le)
+            w.swap_prepared_layers(back, lb, le)
+            w.htod_stream.synchronize()
+            assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np), (lb, le)
+        assert np.array_equal(w.host_kv_caches, host_np)
+        # empty mappings prepare to nothing and move nothing
+        assert w.prepare_swap("out", []) is None
+        w.swap_prepared_layers(None, 0, L)
+        with pytest.raises(IndexError):
+            w.prepare_swap("out", _mappings(np.asarray([nb]), np.asarray([0]), 1))
+        with pytest.raises(IndexError):
+            w.prepare_swap("in", _mappings(np.asarray([nhb]), np.asarray([0]), 1))
+    finally:
+        w.close()
+
+
+def test_many_swaps_in_flight_keep_their_id_lists(gpu):
+    """More swaps enqueued back to back on one thread than the library has id
+    bounce slots, with growing id counts (so bounce buffers are outgrown while
+    earlier uploads may still be queued): every swap moves its own blocks."""
+    L, nb, nhb = 2, 4200, 4200
+    block_shape = (2, 16, 1, 8)                # 512-byte blocks
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, "direct", seed=31)
+    try:
+        rng = np.random.default_rng(32)
+        gpu_np = pool.reshape(L, nb, -1)
+        host_np = w.host_kv_caches.copy()
+        # call k uses bounce slot k % 4; 2n > 4096 entries outgrows a slot's first buffer
+        for k, n in enumerate([3, 500, 10, 20, 2100, 30, 3000, 40, 4100, 4200, 7]):
+            old = rng.permutation(nb)[:n].astype(np.int64)
+            hid = rng.permutation(nhb)[:n].astype(np.int64)
+            orc.save_blocks_to_host_np(gpu_np, host_np, old, hid, 0, L)
+            w.save_kv_blocks_to_host_nowait(_mappings(old, hid, 2))
+        w.dtoh_stream.synchronize()
+        assert np.array_equal(w.host_kv_caches, host_np)
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
 def test_swap_odd_block_bytes_and_other_dtypes(gpu, mode):
     """Blocks whose byte size is not a multiple of 16, and fp32 / fp16 pools."""
     for dtype, np_dtype, block_shape in ((torch.bfloat16, np.uint16, (2, 3, 1, 5)),

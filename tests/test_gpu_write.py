@@ -76,26 +76,113 @@ def test_fill_key_cache_matches_oracle(gpu, T, H, D, num_slots, dtype, slot_dtyp
 
 @pytest.mark.parametrize("vpt", [1, 2, 4, 8])
 @pytest.mark.parametrize("nt", [0, 1, 2, 3])
-def test_fill_key_cache_every_launch_shape(gpu, vpt, nt):
-    """All vectors-per-lane / store-kind instantiations give the same bits."""
-    T, H, D, num_slots = 301, 8, 128, 512
+@pytest.mark.parametrize("threads", [0, 64, 128])
+def test_write_rows_every_launch_shape(gpu, vpt, nt, threads):
+    """All vectors-per-lane / load-store kind / workgroup-size instantiations give
+    the same bits, and the instantiation asked for is the one that ran (8 layers
+    in one launch, so a token has 2048 vectors and every depth fits)."""
+    T, L, H, D, bs, nb = 301, 8, 8, 128, 16, 32
     rng = np.random.default_rng(7)
-    slots = rng.permutation(num_slots)[:T].astype(np.int64)
-    key, value = bf16_bits((T, H, D), 1), bf16_bits((T, H, D), 2)
-    kc, vc = sentinel_pool((num_slots, H, D), 3), sentinel_pool((num_slots, H, D), 4)
-    want_k, want_v = kc.copy(), vc.copy()
-    orc.fill_key_cache_np(key, value, want_k, want_v, slots)
-    dk, dv = to_bf16(kc, gpu), to_bf16(vc, gpu)
-    _lib.set_tuning("write_vpt", vpt)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    key, value = bf16_bits((L, T, H, D), 1), bf16_bits((L, T, H, D), 2)
+    pool = sentinel_pool((L, nb, 2, bs, H, D), 3)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
+    dpool = to_bf16(pool, gpu)
+    _lib.set_tuning("write_vpt", vpt)     # the autouse fixture puts the defaults back
     _lib.set_tuning("write_nt", nt)
-    try:
-        kvc.fill_key_cache(to_bf16(key, gpu), to_bf16(value, gpu), dk, dv,
-                           torch.from_numpy(slots).to(gpu))
+    _lib.set_tuning("write_threads", threads)
+    kvc.reshape_and_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool,
+                                 torch.from_numpy(slots).to(gpu))
+    torch.cuda.synchronize()
+    ran = _lib.last_launch()
+    assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_ROWS and ran["non_temporal"] == nt
+    assert ran["per_lane"] == vpt and ran["threads"] == (threads or 256) and ran["vec_bytes"] == 16
+    assert np.array_equal(bits_of(dpool), want)
+
+
+NARROW_CASES = [
+    # T, H, D, layers, narrow_vpt   (rows of 16 * H*D/8 ... bytes, all under 1 KiB)
+    (256, 1, 128, 80, 0),    # one KV head of Llama-3.1-70B at tp=8: 256-byte rows
+    (256, 1, 128, 80, 1),
+    (256, 1, 128, 80, 2),
+    (256, 1, 128, 80, 4),
+    (256, 1, 128, 80, 8),
+    (77, 2, 128, 5, 0),      # 512-byte rows, odd token and layer counts
+    (77, 2, 128, 5, 8),
+    (3, 1, 64, 3, 0),        # 128-byte rows, fewer tokens than a wavefront covers
+    (300, 1, 32, 7, 4),      # 64-byte rows
+    (1000, 1, 8, 2, 0),      # 16-byte rows: one vector per row
+    (1, 1, 128, 1, 0),
+]
+
+
+@pytest.mark.parametrize("T,H,D,L,vpt", NARROW_CASES)
+@pytest.mark.parametrize("paged", [False, True])
+def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L, vpt, paged):
+    """Rows under 1 KiB (a tensor-parallel shard's head slice) run the kernel whose
+    lanes walk the tokens of one (layer, K|V) plane; every planes-per-lane
+    instantiation, both addressing modes, whole pool compared."""
+    bs, nb = 16, 96
+    rng = np.random.default_rng(T * 7 + D)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    key, value = bf16_bits((L, T, H, D), 1), bf16_bits((L, T, H, D), 2)
+    pool = sentinel_pool((L, nb, 2, bs, H, D), 3)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
+    dpool = to_bf16(pool, gpu)
+    _lib.set_tuning("write_narrow_vpt", vpt)
+    if paged:
+        # requests of up to three tokens, each token on a page of its own:
+        # page = slot // bs at table entry j, position = j * bs + slot % bs
+        sizes = []
+        while sum(sizes) < T:
+            sizes.append(min(int(rng.integers(1, 4)), T - sum(sizes)))
+        bi = np.repeat(np.arange(len(sizes)), sizes).astype(np.int32)
+        j = np.concatenate([np.arange(n) for n in sizes])
+        pos = (j * bs + slots % bs).astype(np.int32)
+        indptr = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+        indices = (slots // bs).astype(np.int32)
+        last = np.ones(len(sizes), dtype=np.int32)
+        bi, pos, indices, indptr, last = (torch.from_numpy(a).to(gpu) for a in (bi, pos, indices, indptr, last))
+        kvc.append_paged_kv_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), bi, pos, dpool,
+                                         indices, indptr, last)
+    else:
+        kvc.reshape_and_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool,
+                                     torch.from_numpy(slots).to(gpu))
+    torch.cuda.synchronize()
+    ran = _lib.last_launch()
+    assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_ROWS_NARROW and ran["vec_bytes"] == 16
+    if vpt:
+        assert ran["per_lane"] == min(vpt, 1 << (2 * L - 1).bit_length())
+    assert np.array_equal(bits_of(dpool), want)
+
+
+def test_narrow_kernel_switch_and_strided_sources(gpu):
+    """`write_narrow = 0` sends narrow rows through the token-per-workgroup kernel;
+    both kernels agree with the oracle on token-strided sources (slices of a wider
+    projection), where the source side is no longer one run."""
+    T, H, D, bs, nb = 130, 1, 128, 16, 40
+    rng = np.random.default_rng(5)
+    slots = rng.permutation(nb * bs)[:T].astype(np.int64)
+    wide_k, wide_v = bf16_bits((T, 3 * H * D), 1), bf16_bits((T, 3 * H * D), 2)
+    key, value = wide_k[:, H * D:2 * H * D], wide_v[:, 2 * H * D:]
+    pool = sentinel_pool((nb, 2, bs, H, D), 3)
+    want = pool.copy()
+    orc.c_reshape_and_cache(np.ascontiguousarray(key).reshape(T, H, D),
+                            np.ascontiguousarray(value).reshape(T, H, D), want, slots)
+    dk = to_bf16(wide_k, gpu)[:, H * D:2 * H * D].view(T, H, D)
+    dv = to_bf16(wide_v, gpu)[:, 2 * H * D:].view(T, H, D)
+    assert not dk.is_contiguous()
+    for narrow, kernel in ((1, _lib.KVC_KERNEL_WRITE_ROWS_NARROW), (0, _lib.KVC_KERNEL_WRITE_ROWS)):
+        _lib.set_tuning("write_narrow", narrow)
+        dpool = to_bf16(pool, gpu)
+        kvc.reshape_and_cache(dk, dv, dpool, torch.from_numpy(slots).to(gpu))
         torch.cuda.synchronize()
-    finally:
-        _lib.set_tuning("write_vpt", 0)
-        _lib.set_tuning("write_nt", 1)
-    assert np.array_equal(bits_of(dk), want_k) and np.array_equal(bits_of(dv), want_v)
+        assert _lib.last_launch()["kernel"] == kernel
+        assert np.array_equal(bits_of(dpool), want)
 
 
 def test_config1_llama_1b_write_all_layers(gpu):
@@ -217,6 +304,51 @@ def test_append_paged_kv_cache_matches_oracle(gpu, kind):
         plan.append(dkey[0].float(), dval[0], planned[0])
     with pytest.raises(ValueError):
         plan.append(dkey[0], dval[0], planned[0][:, :, :8])
+
+
+def test_write_plan_reads_token_strided_rows_and_outlives_nothing(gpu):
+    """`kvc_write_plan_*` through `PagedKVWritePlan`: K and V read in place from
+    slices of one fused `[T, 3*H*D]` projection (token stride 3 rows), 2-D and 3-D
+    views, against the oracle; overlapping rows and short inputs are refused; a
+    plan of zero tokens does nothing."""
+    rng = np.random.default_rng(3)
+    s = wl.LLAMA_3_2_1B
+    w = wl._write_workload(s, 96, [5, 0, 31, 16], [3, 20, 1, 16], rng)
+    T, H, D, bs, nb = w.num_tokens, s.num_kv_heads, s.head_dim, s.block_size, w.num_blocks
+    row = H * D
+    fused = bf16_bits((T, 3 * row), 4)
+    pool = sentinel_pool((nb, 2, bs, H, D), 5)
+    want = pool.copy()
+    orc.c_append_paged_kv_cache(np.ascontiguousarray(fused[:, row:2 * row]).reshape(T, H, D),
+                                np.ascontiguousarray(fused[:, 2 * row:]).reshape(T, H, D),
+                                w.index.batch_indices, w.index.positions, want,
+                                w.index.kv_block_indices, w.index.kv_block_indptrs)
+    dev = kvc.to_device(w.index, bs, gpu)
+    plan = kvc.PagedKVWritePlan(dev.batch_indices, dev.positions, dev.kv_block_indices,
+                                dev.kv_block_indptrs, dev.kv_last_block_lens, H, D, bs, torch.bfloat16)
+    dfused = to_bf16(fused, gpu)
+    k2, v2 = dfused[:, row:2 * row], dfused[:, 2 * row:]
+    for k, v in ((k2, v2), (k2.view(T, H, D), v2.view(T, H, D))):
+        assert not k.is_contiguous()
+        dpool = to_bf16(pool, gpu)
+        plan.append(k, v, dpool)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits_of(dpool), want)
+    dpool = to_bf16(pool, gpu)
+    with pytest.raises(ValueError):
+        plan.append(k2[:1].expand(T, row), v2, dpool)          # every token reads the same row
+    with pytest.raises(ValueError):
+        plan.append(k2[:-1], v2, dpool)
+    with pytest.raises(ValueError):
+        plan.append(k2, v2, dpool.transpose(1, 2))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), pool)
+    empty = torch.empty(0, dtype=torch.int32, device=gpu)
+    nothing = kvc.PagedKVWritePlan(empty, empty, dev.kv_block_indices, dev.kv_block_indptrs,
+                                   dev.kv_last_block_lens, H, D, bs, torch.bfloat16)
+    nothing.append(k2, v2, dpool)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(dpool), pool)
 
 
 def test_append_paged_skips_tokens_with_bad_indices(gpu):

@@ -9,6 +9,7 @@ import lmserve_amd as kvc
 from lmserve_amd import workloads as wl
 from lmserve_amd.index_prep import InferInput, make_kv_index_inputs
 from oracle import kvc_oracle as orc
+from tests.helpers import FifoBlockIds
 
 
 def test_flatten_block_maps_keeps_dict_order_and_fans_out():
@@ -171,25 +172,25 @@ def test_torch_cpu_statements_agree_with_the_oracle():
     assert np.array_equal(got_gpu.numpy().view(np.uint16), want_gpu)
 
 
-def test_block_allocator_hands_out_ids_in_fifo_order():
-    a = kvc.BlockAllocator(6)
-    assert a.alloc_blocks(4) == [0, 1, 2, 3]
-    a.free_block(1)
-    a.free_block(0)
-    assert a.alloc_blocks(3) == [4, 5, 1]          # freed ids queue up behind the untouched ones
-    assert a.alloc_block() == 0
+def test_fifo_id_source_follows_the_allocator_order():
+    """The test-input generator reproduces the id order of block_manager.rs:62-140:
+    front of the queue on allocation, back of the queue on the last release."""
+    a = FifoBlockIds(6)
+    assert a.take(4) == [0, 1, 2, 3]
+    a.give_back([1])
+    a.give_back([0])
+    assert a.take(3) == [4, 5, 1]                   # released ids queue up behind the untouched ones
+    assert a.take() == [0]
     with pytest.raises(RuntimeError):
-        a.alloc_block()
-    a.alloc_block_by_id(2)                          # shared prefix block: ref count 2
-    a.free_block(2)
-    assert a.get_block_usage() == 1.0
-    a.free_block(2)
-    assert a.alloc_block() == 2
-    assert a.can_alloc_blocks(0) and not a.can_alloc_blocks(1)
-    b = kvc.BlockAllocator(10)
-    assert b.can_alloc_blocks(9, 0.9) and not b.can_alloc_blocks(10, 0.9)
-    b.alloc_block_by_id(7)
-    assert b.alloc_blocks(8) == [0, 1, 2, 3, 4, 5, 6, 8]
+        a.take()
+    a.share(2)                                      # shared prefix block: two users
+    a.give_back([2])
+    assert not a.queue
+    a.give_back([2])
+    assert a.take() == [2]
+    b = FifoBlockIds(10)
+    b.share(7)
+    assert b.take(8) == [0, 1, 2, 3, 4, 5, 6, 8]
 
 
 def test_plan_cache_matches_the_configured_pools():
