@@ -147,6 +147,24 @@ def lib() -> ctypes.CDLL:
     return handle
 
 
+_fast = None
+
+
+def fast():
+    """The `_kvc_fast` extension module (METH_FASTCALL wrappers of the per-layer
+    plan calls), or None when it is not built; callers then go through ctypes to
+    the same entry points."""
+    global _fast
+    if _fast is None:
+        lib()   # the shared library first: the extension binds to the same instance
+        try:
+            from . import _kvc_fast
+            _fast = _kvc_fast if _kvc_fast.abi_version == KVC_ABI_VERSION else False
+        except ImportError:
+            _fast = False
+    return _fast or None
+
+
 def last_error() -> str:
     return lib().kvc_last_error_string().decode("utf-8", "replace")
 

@@ -17,6 +17,8 @@ SOURCES = [os.path.join(PKG_DIR, "csrc", "kvcache.hip"),
            os.path.join(PKG_DIR, "csrc", "disk_tier.cpp")]
 INCLUDE = os.path.join(REPO_ROOT, "include")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcache.so")
+FAST_SRC = os.path.join(PKG_DIR, "csrc", "fastcall.c")
+FAST_PATH = os.path.join(PKG_DIR, "_kvc_fast.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -45,18 +47,39 @@ def build(verbose: bool = False) -> str:
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    build_fastcall(verbose)
     return LIB_PATH
+
+
+def build_fastcall(verbose: bool = False) -> str:
+    """Compile `_kvc_fast`, the CPython entry to the per-layer plan calls (plain
+    C, host compiler; links against libkvcache.so next to it)."""
+    import sysconfig
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        raise RuntimeError("no C compiler for lmserve_amd/csrc/fastcall.c")
+    cmd = [cc, "-O2", "-std=c11", "-fPIC", "-shared", "-Wall", "-I", INCLUDE,
+           "-I", sysconfig.get_paths()["include"], FAST_SRC, "-L", PKG_DIR, "-lkvcache",
+           "-Wl,-rpath,$ORIGIN", "-o", FAST_PATH + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building _kvc_fast failed:\n" + proc.stdout + proc.stderr)
+    os.replace(FAST_PATH + ".tmp", FAST_PATH)
+    return FAST_PATH
 
 
 HEADERS = [os.path.join(PKG_DIR, "csrc", "common.h"), os.path.join(INCLUDE, "kvcache.h")]
 
 
 def is_stale() -> bool:
-    """True when the library is missing or older than one of its sources."""
-    if not os.path.exists(LIB_PATH):
+    """True when a built file is missing or older than one of its sources."""
+    if not os.path.exists(LIB_PATH) or not os.path.exists(FAST_PATH):
         return True
-    built = os.path.getmtime(LIB_PATH)
-    return any(os.path.exists(f) and os.path.getmtime(f) > built for f in SOURCES + HEADERS)
+    built = min(os.path.getmtime(LIB_PATH), os.path.getmtime(FAST_PATH))
+    return any(os.path.exists(f) and os.path.getmtime(f) > built for f in SOURCES + HEADERS + [FAST_SRC])
 
 
 def ensure_built() -> None:

@@ -433,5 +433,10 @@ class KVWorker:
             self.disk_tier = None
         self._host_pool.close()
         self._staging = {"out": None, "in": None}
+        # let go of the pool now: the direction table holds bound methods, so the
+        # worker is part of a reference cycle and would otherwise keep tens of GiB
+        # of HBM alive until the cycle collector runs
+        self.gpu_kv_caches = None
+        self.COPY_KV_OP_MAP = {}
         # events and id bounce buffers the library kept for this thread
         _lib.check(_lib.lib().kvc_thread_release())

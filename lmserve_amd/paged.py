@@ -217,9 +217,11 @@ class PagedKVWritePlan:
             self.kv_indptr.numel() - 1, self.kv_indices.numel(), self.H, self.D, self.page_size,
             self.elem, ctypes.byref(handle)))
         self._plan = handle.value
-        self._append = lib.kvc_write_plan_append
+        fast = _lib.fast()
+        self._append = fast.write_plan_append if fast else lib.kvc_write_plan_append
         self._destroy = lib.kvc_write_plan_destroy
-        self._cache_shape_tail = (2, self.page_size, self.H, self.D)
+        self._cache_shape_tail = torch.Size((2, self.page_size, self.H, self.D))
+        self._k_plane = self.page_size * self.row
         self._dense_page = 2 * self.page_size * self.row
         self._dev_index = self.device.index
         self._get_stream = torch._C._cuda_getCurrentRawStream
@@ -230,7 +232,8 @@ class PagedKVWritePlan:
             self._destroy(plan)
 
     def _row_stride(self, t: torch.Tensor, name: str) -> int:
-        """Token stride of `[nnz, H, D]` / `[nnz, H*D]` rows that are dense inside a token."""
+        """Token stride of `[nnz, H, D]` / `[nnz, H*D]` rows that are dense inside a
+        token; raises with the reason when the tensor does not qualify."""
         if t.dtype != self.dtype or t.device != self.device:
             raise TypeError(f"{name} must have the plan's dtype and device")
         st = t.stride()
@@ -252,19 +255,30 @@ class PagedKVWritePlan:
         place), `paged_kv_cache` `[num_pages, 2, page_size, H, D]` with contiguous
         pages. Launches on the current stream of the plan's device, which must be
         the current device."""
-        if self.nnz == 0:
+        nnz = self.nnz
+        if nnz == 0:
             return
-        k_stride = self._row_stride(append_key, "append_key")
-        v_stride = self._row_stride(append_value, "append_value")
+        row = self.row
+        # the common case in one pass: contiguous [nnz, H, D] / [nnz, H*D] rows; anything
+        # else goes through the checks that name what is wrong
+        k_stride = append_key.stride(0)
+        v_stride = append_value.stride(0)
+        dt, dev = self.dtype, self.device
+        if not (append_key.dtype is dt and append_value.dtype is dt and append_key.device == dev
+                and append_value.device == dev and append_key.is_contiguous()
+                and append_value.is_contiguous() and k_stride == row and v_stride == row
+                and append_key.shape[0] >= nnz and append_value.shape[0] >= nnz):
+            k_stride = self._row_stride(append_key, "append_key")
+            v_stride = self._row_stride(append_value, "append_value")
         shape = paged_kv_cache.shape
-        if paged_kv_cache.dtype != self.dtype or paged_kv_cache.device != self.device:
-            raise TypeError("paged_kv_cache must have the plan's dtype and device")
         num_pages = shape[0]
         if num_pages == 0:
             return
+        if paged_kv_cache.dtype is not dt or paged_kv_cache.device != dev:
+            raise TypeError("paged_kv_cache must have the plan's dtype and device")
         st = paged_kv_cache.stride()
-        if tuple(shape[1:]) != self._cache_shape_tail or st[4] != 1 or st[3] != self.D \
-                or st[2] != self.row or st[1] != self.page_size * self.row:
+        if shape[1:] != self._cache_shape_tail or st[4] != 1 or st[3] != self.D \
+                or st[2] != row or st[1] != self._k_plane:
             raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
         rc = self._append(self._plan, append_key.data_ptr(), append_value.data_ptr(), k_stride,
                           v_stride, paged_kv_cache.data_ptr(),

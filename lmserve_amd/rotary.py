@@ -242,9 +242,11 @@ class PagedRotaryWritePlan:
             kv_indices.data_ptr(), kv_indptr.data_ptr(), kv_indptr.numel() - 1, kv_indices.numel(),
             self.page_size, self.kd, ctypes.byref(handle)))
         self._plan = handle.value
-        self._run = lib.kvc_rotary_plan_run
+        fast = _lib.fast()
+        self._run = fast.rotary_plan_run if fast else lib.kvc_rotary_plan_run
         self._destroy = lib.kvc_rotary_plan_destroy
-        self._cache_shape_tail = (2, self.page_size, self.H, self.D)
+        self._cache_shape_tail = torch.Size((2, self.page_size, self.H, self.D))
+        self._k_plane = self.page_size * self.kv_row
         self._dense_page = 2 * self.page_size * self.kv_row
         self._dev_index = self.device.index
         self._get_stream = torch._C._cuda_getCurrentRawStream
@@ -283,22 +285,40 @@ class PagedRotaryWritePlan:
             key_out = torch.empty((self.nnz, self.kv_row), dtype=self.dtype, device=self.device)
         if self.nnz == 0:
             return query_out, key_out
-        if paged_kv_cache.dtype != self.dtype or paged_kv_cache.device != self.device:
+        dt, dev, nnz = self.dtype, self.device, self.nnz
+        if paged_kv_cache.dtype is not dt or paged_kv_cache.device != dev:
             raise TypeError("paged_kv_cache must have the plan's dtype and device")
         shape, st = paged_kv_cache.shape, paged_kv_cache.stride()
-        if tuple(shape[1:]) != self._cache_shape_tail or st[4] != 1 or st[3] != self.D \
-                or st[2] != self.kv_row or st[1] != self.page_size * self.kv_row:
+        if shape[1:] != self._cache_shape_tail or st[4] != 1 or st[3] != self.D \
+                or st[2] != self.kv_row or st[1] != self._k_plane:
             raise ValueError("paged_kv_cache must be [num_pages, 2, page_size, H, D] with contiguous pages")
         num_pages = shape[0]
         if num_pages == 0:
             raise ValueError("paged_kv_cache has no pages")
-        q_stride = self._rows(query, self.q_row, "query")
-        k_stride = self._rows(key, self.kv_row, "key")
-        v_stride = self._rows(value, self.kv_row, "value")
-        self._rows(query_out, self.q_row, "query_out", dense=True)
+        q_row, kv_row = self.q_row, self.kv_row
+        # the common case in one pass: 2-D [nnz, width] views with unit inner stride (the
+        # slices of a fused projection); anything else goes through the checks that name
+        # what is wrong
+        qs, ks, vs = query.stride(), key.stride(), value.stride()
+        if (query.dtype is dt and key.dtype is dt and value.dtype is dt and len(qs) == 2 and len(ks) == 2
+                and len(vs) == 2 and qs[1] == 1 and ks[1] == 1 and vs[1] == 1
+                and query.shape == (nnz, q_row) and key.shape == (nnz, kv_row)
+                and value.shape == (nnz, kv_row) and qs[0] >= q_row and ks[0] >= kv_row
+                and vs[0] >= kv_row and query.device == dev and key.device == dev
+                and value.device == dev):
+            q_stride, k_stride, v_stride = qs[0], ks[0], vs[0]
+        else:
+            q_stride = self._rows(query, q_row, "query")
+            k_stride = self._rows(key, kv_row, "key")
+            v_stride = self._rows(value, kv_row, "value")
+        if not (query_out.dtype is dt and query_out.is_contiguous() and query_out.device == dev
+                and query_out.numel() == nnz * q_row):
+            self._rows(query_out, q_row, "query_out", dense=True)
         ko_ptr = None
         if key_out is not None:
-            self._rows(key_out, self.kv_row, "key_out", dense=True)
+            if not (key_out.dtype is dt and key_out.is_contiguous() and key_out.device == dev
+                    and key_out.numel() == nnz * kv_row):
+                self._rows(key_out, kv_row, "key_out", dense=True)
             ko_ptr = key_out.data_ptr()
         rc = self._run(self._plan, query.data_ptr(), key.data_ptr(), value.data_ptr(), q_stride,
                        k_stride, v_stride, query_out.data_ptr(), ko_ptr, paged_kv_cache.data_ptr(),

@@ -17,6 +17,17 @@ pytestmark = pytest.mark.gpu
 SWAP_BLOCKS = int(os.environ.get("KVC_TEST_SWAP_BLOCKS", "8192"))
 
 
+@pytest.fixture(autouse=True)
+def release_hbm():
+    """These tests hold 80-128 GiB each: drop what the previous one left behind."""
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    yield
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
 def _check_write(pool, key, value, slots_np, bs):
     """pool [L, nb, 2, bs, H, D] was all-zero before the write."""
     L = pool.shape[0]
