@@ -701,10 +701,11 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     const int64_t token_groups_all = (g.num_tokens + a.tokens_per_wg - 1) / a.tokens_per_wg;
     l.vpt = g_tune.write_narrow_vpt;
     if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8) {
-      // the fewest planes per lane that keep the launch within one resident set
+      // the fewest planes per lane (up to 4) that keep the launch within one resident
+      // set of workgroups; a launch larger than that streams with one plane per lane
       const int64_t resident = resident_workgroups();
-      l.vpt = 8;
-      for (int v = 1; v < 8; v *= 2)
+      l.vpt = 1;
+      for (int v = 1; v <= 4; v *= 2)
         if (token_groups_all * ((a.num_planes + v - 1) / v) <= resident) {
           l.vpt = v;
           break;
