@@ -349,6 +349,31 @@ int kvc_swap_in_prepared(void* pool, const void* host_pool, const int64_t* host_
 
 int kvc_thread_release(void);
 
+/* A direct swap that allocates nothing and needs no workspace. It has no
+ * counterpart in the reference; it is for callers that cannot allocate: code
+ * under HIP graph capture, serving loops and harnesses that forbid hipMalloc.
+ * kvc_swap_out / kvc_swap_in in KVC_SWAP_DIRECT mode with `staging` replaced by
+ * a static device array inside the library (KVC_NOALLOC_MAX_BLOCKS id pairs,
+ * 128 KiB per device, held until the process ends):
+ *   to_host != 0: host[host_ids[i], l, :] = pool[l, gpu_ids[i], :]
+ *   to_host == 0: pool[l, gpu_ids[i], :] = host[host_ids[i], l, :]
+ * for l in [layer_begin, layer_end). gpu_ids / host_ids are HOST int64 arrays,
+ * range-checked before anything is launched; they travel to the device as
+ * kernel arguments, so the call consists of kernel launches on `stream` only:
+ * no hipMalloc, no hipFree, no pinned bounce buffer, no memcpy, no events.
+ * n > KVC_NOALLOC_MAX_BLOCKS: KVC_ERR_UNSUPPORTED, nothing launched. The first
+ * call on a device looks up the array's address there.
+ * Every call on one device shares that device's array: calls on one stream are
+ * ordered by the stream; calls that overlap on different streams of one device
+ * race on the id lists and must be ordered by the caller. */
+#define KVC_NOALLOC_MAX_BLOCKS 8192
+
+int kvc_swap_noalloc(int to_host, void* pool, void* host_pool,
+                     const int64_t* gpu_ids, const int64_t* host_ids, int64_t n,
+                     int64_t num_layers, int64_t layer_stride_bytes, int64_t block_bytes,
+                     int64_t num_gpu_blocks, int64_t num_host_blocks,
+                     int64_t layer_begin, int64_t layer_end, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Rotary position embedding, alone or fused with the K/V write.
  * (Widening beyond the copy path: the rotation runs immediately before the

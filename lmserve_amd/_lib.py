@@ -45,6 +45,7 @@ KVC_LAUNCH_GRID = 4
 KVC_LAUNCH_NON_TEMPORAL = 5
 
 KVC_ABI_VERSION = 2
+KVC_NOALLOC_MAX_BLOCKS = 8192
 
 KVC_DTYPE_BF16 = 0
 KVC_DTYPE_F16 = 1
@@ -76,6 +77,8 @@ SIGNATURES = {
     "kvc_swap_in_prepared": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
                                      _I64, c_int, _P, _P]),
     "kvc_thread_release": (c_int, []),
+    "kvc_swap_noalloc": (c_int, [c_int, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                 _P]),
     "kvc_reshape_and_cache": (c_int, [_P, _P, _P, _P, _P, c_int, _I64, _I64, _I64, _I64, _I64,
                                       _I64, _I64, _I64, c_int, _P]),
     "kvc_reshape_and_cache_layers": (c_int, [_P, _P, _P, _P, _P, c_int, _I64, _I64, _I64, _I64,

@@ -30,6 +30,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "common.h"
@@ -1215,6 +1216,51 @@ int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_
   return KVC_OK;
 }
 
+// --------------------------- swap that allocates nothing ---------------------
+// The id lists of a direct swap live in a static device array instead of a
+// caller-provided workspace, and reach it as kernel arguments instead of through
+// a pinned bounce buffer and a copy: the call is kernel launches only.
+static __device__ __align__(256) int64_t scratch[2 * KVC_NOALLOC_MAX_BLOCKS];  // [gpu ids | host ids]
+
+constexpr int kMaxDevices = 64;
+constexpr int kIdsPerPacket = 448;  // id pairs per staging launch: 3584 bytes of kernel arguments
+
+struct IdPacket {
+  int32_t gpu[kIdsPerPacket];
+  int32_t host[kIdsPerPacket];
+};
+
+// scratch_ptr[first + i] = gpu id, scratch_ptr[n + first + i] = host id, for i in [0, count)
+__global__ __launch_bounds__(kIdsPerPacket) void stage_ids_kernel(IdPacket p, int64_t* scratch_ptr,
+                                                                  int64_t first, int count, int64_t n) {
+  const int i = threadIdx.x;
+  if (i < count) {
+    scratch_ptr[first + i] = p.gpu[i];
+    scratch_ptr[n + first + i] = p.host[i];
+  }
+}
+
+// Device address of `scratch` on the current device. In host code the array's
+// name is only a handle for the runtime; every device holds its own copy at its
+// own address, looked up once per device.
+int scratch_of_current_device(int64_t** out) {
+  static std::mutex mu;
+  static int64_t* ptrs[kMaxDevices] = {};
+  int dev = 0;
+  KVC_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(KVC_ERR_UNSUPPORTED, "device ordinal %d is beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    KVC_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(KVC_ERR_HIP, "hipGetSymbolAddress returned a null address for the id scratch");
+    ptrs[dev] = (int64_t*)p;
+  }
+  *out = ptrs[dev];
+  return KVC_OK;
+}
+
 }  // namespace
 
 // ===========================================================================
@@ -1612,6 +1658,53 @@ int kvc_swap_in_prepared(void* pool, const void* host_pool, const int64_t* host_
 }
 
 int kvc_thread_release(void) { return swap_ctx_release(); }
+
+int kvc_swap_noalloc(int to_host, void* pool, void* host_pool, const int64_t* gpu_ids,
+                     const int64_t* host_ids, int64_t n, int64_t num_layers,
+                     int64_t layer_stride_bytes, int64_t block_bytes, int64_t num_gpu_blocks,
+                     int64_t num_host_blocks, int64_t layer_begin, int64_t layer_end, void* stream) {
+  const char* fn = "kvc_swap_noalloc";
+  if (n < 0 || num_layers < 0 || block_bytes < 0 || layer_stride_bytes < 0 || num_gpu_blocks < 0 ||
+      num_host_blocks < 0)
+    return fail(KVC_ERR_INVALID_ARG, "%s: negative size", fn);
+  if (layer_begin < 0 || layer_end < layer_begin || layer_end > num_layers)
+    return fail(KVC_ERR_INVALID_ARG, "%s: layer range [%lld, %lld) outside [0, %lld)", fn,
+                (long long)layer_begin, (long long)layer_end, (long long)num_layers);
+  if (n > KVC_NOALLOC_MAX_BLOCKS)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: %lld blocks exceed the %d this entry point holds ids for "
+                "(use kvc_swap_out / kvc_swap_in with a workspace)", fn, (long long)n,
+                KVC_NOALLOC_MAX_BLOCKS);
+  const int64_t nl = layer_end - layer_begin;
+  if (n == 0 || nl == 0 || block_bytes == 0) return KVC_OK;
+  if (!pool || !host_pool || !gpu_ids || !host_ids)
+    return fail(KVC_ERR_INVALID_ARG, "%s: null pool/host/id pointer", fn);
+  if (layer_stride_bytes < block_bytes)
+    return fail(KVC_ERR_INVALID_ARG, "%s: layer stride smaller than a block", fn);
+  if (nl > 0xffffffffll) return fail(KVC_ERR_UNSUPPORTED, "%s: too many layers", fn);
+  if (num_gpu_blocks > INT32_MAX || num_host_blocks > INT32_MAX)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: block ids beyond 31 bits", fn);
+  int rc = check_ids(fn, gpu_ids, host_ids, n, num_gpu_blocks, num_host_blocks);
+  if (rc != KVC_OK) return rc;
+  int64_t* ids = nullptr;  // device address of the static id array on this device
+  rc = scratch_of_current_device(&ids);
+  if (rc != KVC_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  IdPacket packet;
+  for (int64_t first = 0; first < n; first += kIdsPerPacket) {
+    const int count = (int)std::min<int64_t>(kIdsPerPacket, n - first);
+    for (int i = 0; i < count; ++i) {
+      packet.gpu[i] = (int32_t)gpu_ids[first + i];
+      packet.host[i] = (int32_t)host_ids[first + i];
+    }
+    hipLaunchKernelGGL(stage_ids_kernel, dim3(1), dim3((count + 63) / 64 * 64), 0, s, packet, ids, first,
+                       count, n);
+    KVC_HIP(hipGetLastError());
+  }
+  const SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
+                   layer_begin, layer_end};
+  const TileArgs t = direct_swap_tiles(to_host != 0, (char*)pool, (char*)host_pool, ids, ids + n, g);
+  return launch_tiles(t, n, g_tune.direct_max_wgs, s);
+}
 
 void* kvc_host_alloc_pinned(size_t bytes) {
   void* p = nullptr;
