@@ -72,7 +72,10 @@ const char* kvc_last_error_string(void);
  *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads
  *   "write_order"                     1 = a token's workgroups are neighbours in the grid
  *   "write_narrow"                    rows under 1 KiB take the kernel whose lanes run over
- *                                     consecutive tokens of one (layer, K|V) plane (0/1)
+ *                                     consecutive tokens of one (layer, K|V) plane: 0 = never,
+ *                                     1 = for launches of "write_narrow_min_bytes" source bytes
+ *                                     and more, 2 = always
+ *   "write_narrow_min_bytes"          that size (default 2 MiB)
  *   "write_narrow_vpt"                planes per lane in that kernel (0 = by size, 1, 2, 4, 8)
  *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
  *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier

@@ -7,7 +7,8 @@
     index_prep  host-side block-table / slot-mapping construction
     rotary      rotary position embedding, alone or fused with the K/V write
     disk_tier   DiskTier (host <-> block file, native positional I/O)
-    kv_pool     pool sizing, layer-sync handle and model-side hooks
+    kv_pool     pool sizing, layer-sync handle and model-side hooks, hand-over to a second process
+    kv_service  the KV worker as a process of its own (pool mapped from an IPC handle)
 
 Every operator runs a hand-written HIP kernel from libkvcache.so through the
 C ABI of include/kvcache.h; the disk tier is host-side file I/O in the same
@@ -20,8 +21,9 @@ from .cache_ops import (check_block_maps, copy_blocks, fill_key_cache, flatten_b
 from .disk_tier import DiskTier
 from .index_prep import (InferInput, KVIndexInputs, make_kv_index_inputs, to_device,
                          to_device_one_launch)
-from .kv_pool import (CachePlan, KVWorkerHandle, LayerSyncHooks,
-                      allocate_kv_caches, plan_cache)
+from .kv_pool import (CachePlan, KVWorkerHandle, KVWorkerParams, LayerSyncHooks,
+                      allocate_kv_caches, make_kv_worker_params, open_kv_worker_params, plan_cache)
+from .kv_service import serve_kv_worker
 from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, PinnedHostPool,
                         flatten_block_mappings)
 from .rotary import (PagedRotaryWritePlan, RotaryEmbedding, make_cos_sin_cache, rotary_pos_emb,
@@ -39,7 +41,8 @@ __all__ = [
     "flatten_block_mappings", "DiskTier",
     "RotaryEmbedding", "make_cos_sin_cache", "rotary_pos_emb", "rotary_pos_emb_and_cache",
     "rotary_pos_emb_and_append_paged", "PagedRotaryWritePlan",
-    "CachePlan", "KVWorkerHandle", "LayerSyncHooks", "allocate_kv_caches",
+    "CachePlan", "KVWorkerHandle", "KVWorkerParams", "LayerSyncHooks", "allocate_kv_caches",
+    "make_kv_worker_params", "open_kv_worker_params", "serve_kv_worker",
     "plan_cache",
     "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device", "to_device_one_launch",
     "build_write_index",

@@ -70,6 +70,8 @@ struct Tuning {
   int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
   int write_narrow = 1;     // rows under 1 KiB: lanes of a wavefront run over consecutive tokens of
                             // one (layer, K|V) plane instead of over one token's planes
+                            // (0 = never, 1 = for launches of write_narrow_min_bytes and more, 2 = always)
+  int write_narrow_min_bytes = 2 << 20;  // source bytes of a launch from which that kernel runs
   int write_narrow_vpt = 0; // planes per lane in that kernel (1, 2, 4, 8), 0 = by size
   int direct_max_wgs = 64;  // grid cap of the direct swap kernel: PCIe saturates with a few
                             // dozen workgroups, the rest of the GPU stays free for the model
@@ -95,6 +97,7 @@ Knob* knobs(int* count) {
       {"write_threads", &g_tune.write_threads, 0},
       {"write_narrow", &g_tune.write_narrow, 1},
       {"write_narrow_vpt", &g_tune.write_narrow_vpt, 0},
+      {"write_narrow_min_bytes", &g_tune.write_narrow_min_bytes, 2 << 20},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 64},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
@@ -692,8 +695,16 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
   a.items_per_token = (uint32_t)items64;
 
-  // Rows under 1 KiB: lanes run over consecutive tokens of one plane.
-  if (g_tune.write_narrow && vec == 16 && a.vpr_shift >= 0 && a.vecs_per_row < 64) {
+  // Rows under 1 KiB: lanes run over consecutive tokens of one plane, once the
+  // launch is large enough for bandwidth to matter. Below about 2 MiB of source
+  // rows a launch is latency-bound and many small token-per-workgroup workgroups
+  // with a scalar slot lookup finish first (one layer of a 2048-token chunk at
+  // 256-byte rows: 2.53 against 2.80 us; 80 layers of a 64-token step: 4.04
+  // against 3.67 us).
+  const bool narrow_rows = vec == 16 && a.vpr_shift >= 0 && a.vecs_per_row < 64;
+  const bool narrow_pays = g_tune.write_narrow >= 2 ||
+                           g.num_tokens * 2 * g.num_layers * g.row_elems * E >= g_tune.write_narrow_min_bytes;
+  if (g_tune.write_narrow && narrow_rows && narrow_pays) {
     WriteLaunch l{};
     const int64_t lanes_all = g.num_tokens * (int64_t)a.vecs_per_row;
     l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes_all + 63) / 64 * 64);

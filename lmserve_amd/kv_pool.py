@@ -1,4 +1,4 @@
-"""Pool sizing and the layer-sync handle.
+"""Pool sizing, the layer-sync handle and its hand-over to a second process.
 
 Host-side mirrors of the pieces that decide what the data-movement kernels are
 handed:
@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import queue
 from dataclasses import dataclass, field
-from typing import Any, Iterable, List, Optional
+from typing import Any, Iterable, List, Optional, Tuple
 
 import torch
 
@@ -58,18 +58,83 @@ class KVWorkerHandle:
                    layer l.
     A queue token accompanies every record, so the waiting side only looks at
     an event that has been recorded for this step.
+
+    sync = "events" (the reference's protocol): both sides hold the SAME events
+    (one process, or interprocess events opened from IPC handles) and order
+    their streams with GPU-side event waits; a token only says "the event has
+    been recorded".
+    sync = "host": for two processes on machines whose HIP runtime cannot export
+    event handles (it builds them on `hipHostRegister`). Events stay local to
+    the process that records them; a token is sent only once the recorded work
+    has COMPLETED (a notifier thread waits for the local event first), so
+    receiving the token is the ordering and no cross-process event wait exists.
+    `pre_events` / `post_events` are then this process's own events.
     """
     pre_events: List[Any]
     post_events: List[Any]
     model_queue: Any = field(default_factory=queue.Queue)
     kv_queue: Any = field(default_factory=queue.Queue)
+    sync: str = "events"
+    _notifier: Any = field(default=None, repr=False, compare=False)
 
     @classmethod
-    def create(cls, num_layers: int, interprocess: bool = False) -> "KVWorkerHandle":
+    def create(cls, num_layers: int, interprocess: bool = False, mp_context=None,
+               sync: str = "events") -> "KVWorkerHandle":
+        """Events and doorbells for one process (threads: `queue.Queue`) or, with
+        `interprocess=True`, for two (`multiprocessing` queues of `mp_context`,
+        default the spawn context, model_worker.py:232-252). With sync="events"
+        the events are created exportable as IPC handles; with sync="host" they
+        are ordinary events of this process."""
+        if sync not in ("events", "host"):
+            raise ValueError("sync must be 'events' or 'host'")
+
         def events():
-            return [torch.cuda.Event(enable_timing=False, interprocess=interprocess)
+            return [torch.cuda.Event(enable_timing=False, interprocess=interprocess and sync == "events")
                     for _ in range(num_layers)]
-        return cls(events(), events())
+        if not interprocess:
+            return cls(events(), events(), sync=sync)
+        import multiprocessing
+        ctx = mp_context or multiprocessing.get_context("spawn")
+        return cls(events(), events(), ctx.Queue(), ctx.Queue(), sync)
+
+    def ring_when_done(self, event, doorbell) -> None:
+        """sync="host": put a token on `doorbell` once `event` has completed, in
+        the order of the calls (one notifier thread per handle and process)."""
+        if self._notifier is None:
+            self._notifier = _Notifier()
+        self._notifier.submit(event, doorbell)
+
+    def close(self) -> None:
+        if self._notifier is not None:
+            self._notifier.stop()
+            self._notifier = None
+
+
+class _Notifier:
+    """A thread that waits for events in submission order and rings a doorbell
+    after each (host-signalled layer protocol)."""
+
+    def __init__(self):
+        import threading
+        self.jobs: "queue.Queue" = queue.Queue()
+        self.thread = threading.Thread(target=self._run, name="kvc-layer-doorbell", daemon=True)
+        self.thread.start()
+
+    def submit(self, event, doorbell) -> None:
+        self.jobs.put((event, doorbell))
+
+    def _run(self) -> None:
+        while True:
+            job = self.jobs.get()
+            if job is None:
+                return
+            event, doorbell = job
+            event.synchronize()
+            doorbell.put(b"")
+
+    def stop(self) -> None:
+        self.jobs.put(None)
+        self.thread.join(timeout=10)
 
 
 class LayerSyncHooks:
@@ -90,14 +155,82 @@ class LayerSyncHooks:
     def pre(self, layer_idx: int, stream: Optional[torch.cuda.Stream] = None) -> None:
         if self.enable_wait_before_execute:
             self.handle.model_queue.get(timeout=self.timeout)
-            (stream or torch.cuda.current_stream()).wait_event(self.handle.pre_events[layer_idx])
+            if self.handle.sync == "events":
+                (stream or torch.cuda.current_stream()).wait_event(self.handle.pre_events[layer_idx])
+            # sync == "host": the token was sent after the layer's load had completed
 
     def post(self, layer_idx: int, stream: Optional[torch.cuda.Stream] = None) -> None:
         if self.enable_record_after_execute:
-            self.handle.post_events[layer_idx].record(stream or torch.cuda.current_stream())
-            self.handle.kv_queue.put(b"")   # doorbell: layer's K/V may be saved
+            event = self.handle.post_events[layer_idx]
+            event.record(stream or torch.cuda.current_stream())
+            if self.handle.sync == "events":
+                self.handle.kv_queue.put(b"")   # doorbell: layer's K/V may be saved
+            else:
+                self.handle.ring_when_done(event, self.handle.kv_queue)
 
     def attach(self, attention_layers: Iterable[torch.nn.Module]) -> None:
         for i, layer in enumerate(attention_layers):
             layer.register_forward_pre_hook(lambda mod, inp, i=i: self.pre(i))
             layer.register_forward_hook(lambda mod, inp, out, i=i: self.post(i))
+
+
+@dataclass
+class KVWorkerParams:
+    """What the model worker hands to the KV-worker process it starts: the pool
+    as an IPC storage handle, its geometry, the per-layer events as IPC handles
+    and the two doorbell queues (kv_worker.py:33-45 of the reference; built at
+    model_worker.py:278-306, consumed at kv_worker.py:97-153). Picklable, so it
+    travels as an argument of `multiprocessing.Process` (spawn start method, as
+    cli.py:115-121 and :282 of the reference use)."""
+    kv_cache_metadata: Tuple[Any, ...]
+    num_layers: int
+    num_gpu_blocks: int
+    num_host_blocks: int
+    num_disk_blocks: int
+    disk_kv_cache_file: str
+    dtype: torch.dtype
+    pre_event_handles: List[bytes]
+    post_event_handles: List[bytes]
+    model_queue: Any
+    kv_queue: Any
+    sync: str = "events"   # "host": no event handles travel (see KVWorkerHandle)
+
+
+def make_kv_worker_params(kv_caches: torch.Tensor, handle: KVWorkerHandle, num_host_blocks: int,
+                          num_disk_blocks: int = 0, disk_kv_cache_file: str = "") -> KVWorkerParams:
+    """Export the pool and the handle's events for another process on the same GPU
+    (model_worker.py:278-306). `handle` must hold interprocess events and queues
+    that cross processes (`multiprocessing` queues). The pool tensor must stay
+    alive in this process for as long as the other process maps it."""
+    if not kv_caches.is_cuda or not kv_caches.is_contiguous() or kv_caches.dim() < 3:
+        raise ValueError("kv_caches must be a contiguous [L, num_gpu_blocks, ...] tensor on the GPU")
+    if kv_caches.storage_offset() != 0 or \
+            kv_caches.untyped_storage().nbytes() != kv_caches.numel() * kv_caches.element_size():
+        raise ValueError("kv_caches must own its storage (the other process maps the whole storage)")
+    return KVWorkerParams(
+        kv_cache_metadata=kv_caches.untyped_storage()._share_cuda_(),
+        num_layers=kv_caches.shape[0], num_gpu_blocks=kv_caches.shape[1],
+        num_host_blocks=int(num_host_blocks), num_disk_blocks=int(num_disk_blocks),
+        disk_kv_cache_file=disk_kv_cache_file, dtype=kv_caches.dtype,
+        pre_event_handles=[e.ipc_handle() for e in handle.pre_events] if handle.sync == "events" else [],
+        post_event_handles=[e.ipc_handle() for e in handle.post_events] if handle.sync == "events" else [],
+        model_queue=handle.model_queue, kv_queue=handle.kv_queue, sync=handle.sync)
+
+
+def open_kv_worker_params(params: KVWorkerParams, device: int = 0):
+    """The receiving side (kv_worker.py:104-108, :140-153): map the pool from its
+    IPC handle as `[L, num_gpu_blocks, block_elems]` and open the events. Returns
+    `(gpu_kv_caches, KVWorkerHandle)`."""
+    device = torch.device("cuda", device) if isinstance(device, int) else torch.device(device)
+    with torch.cuda.device(device):
+        storage = torch.UntypedStorage._new_shared_cuda(*params.kv_cache_metadata)
+        gpu_kv_caches = torch.empty(0, dtype=params.dtype, device=device)
+        gpu_kv_caches.set_(storage)
+        gpu_kv_caches = gpu_kv_caches.view(params.num_layers, params.num_gpu_blocks, -1)
+        if params.sync == "events":
+            pre = [torch.cuda.Event.from_ipc_handle(device, h) for h in params.pre_event_handles]
+            post = [torch.cuda.Event.from_ipc_handle(device, h) for h in params.post_event_handles]
+        else:   # host-signalled: this process records events of its own
+            pre = [torch.cuda.Event(enable_timing=False) for _ in range(params.num_layers)]
+            post = [torch.cuda.Event(enable_timing=False) for _ in range(params.num_layers)]
+    return gpu_kv_caches, KVWorkerHandle(pre, post, params.model_queue, params.kv_queue, params.sync)

@@ -344,7 +344,9 @@ class KVWorker:
                 while handle.kv_queue.empty():
                     await asyncio.sleep(1e-5)
                 handle.kv_queue.get()
-                stream.wait_event(handle.post_events[layer_idx])
+                if handle.sync == "events":
+                    stream.wait_event(handle.post_events[layer_idx])
+                # sync == "host": the token was sent after the layer's write had completed
                 self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
                 await asyncio.sleep(0)  # let other tasks of the loop run
         await asyncio.to_thread(stream.synchronize)
@@ -363,7 +365,10 @@ class KVWorker:
                 self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
                 await asyncio.sleep(0)
                 handle.pre_events[layer_idx].record(stream)
-                handle.model_queue.put(b"")
+                if handle.sync == "events":
+                    handle.model_queue.put(b"")
+                else:
+                    handle.ring_when_done(handle.pre_events[layer_idx], handle.model_queue)
         await asyncio.to_thread(stream.synchronize)
 
     # ----------------------------------------------------------------- disk legs

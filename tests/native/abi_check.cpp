@@ -159,9 +159,9 @@ int main() {
     HIP_OK(hipStreamSynchronize(stream));
     HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
     expect_equal("kvc_write_plan_append == oracle", got.data(), want_paged.data(), pool_bytes);
-    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS_NARROW ||
+    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS ||
         kvc_last_launch_info(KVC_LAUNCH_VEC_BYTES) != 16) {
-      std::fprintf(stderr, "256-byte rows did not take the narrow-row kernel\n");
+      std::fprintf(stderr, "a small launch of 256-byte rows did not take the token-per-workgroup kernel\n");
       ++fails;
     }
     // host cost of one planned launch (informational)
@@ -191,9 +191,9 @@ int main() {
     }
     // tuning knobs: set, read back, reset
     int v = -1;
-    KVC_OK_OR_DIE(kvc_set_tuning("write_narrow", 0));
+    KVC_OK_OR_DIE(kvc_set_tuning("write_narrow", 2));
     KVC_OK_OR_DIE(kvc_get_tuning("write_narrow", &v));
-    if (v != 0 || kvc_tuning_modified() != 1) { std::fprintf(stderr, "tuning read-back failed\n"); ++fails; }
+    if (v != 2 || kvc_tuning_modified() != 1) { std::fprintf(stderr, "tuning read-back failed\n"); ++fails; }
     HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
     for (int64_t l = 0; l < L; ++l)
       KVC_OK_OR_DIE(kvc_reshape_and_cache((char*)d_key + l * T * row * E, (char*)d_value + l * T * row * E,
@@ -202,9 +202,9 @@ int main() {
                                           row, row, row, bs, blk_elems, row, nb, (int)E, stream));
     HIP_OK(hipStreamSynchronize(stream));
     HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
-    expect_equal("token-per-workgroup kernel on 256-byte rows == oracle", got.data(), want.data(), pool_bytes);
-    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS) {
-      std::fprintf(stderr, "write_narrow = 0 did not select the token-per-workgroup kernel\n");
+    expect_equal("plane kernel on 256-byte rows == oracle", got.data(), want.data(), pool_bytes);
+    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS_NARROW) {
+      std::fprintf(stderr, "write_narrow = 2 did not select the plane kernel\n");
       ++fails;
     }
     KVC_OK_OR_DIE(kvc_reset_tuning());

@@ -24,15 +24,18 @@ def _busy(dev, n=3):
 
 
 @pytest.mark.parametrize("mode", ["direct", "staged"])
-def test_write_through_waits_for_each_layers_kv_write(gpu, mode):
+@pytest.mark.parametrize("sync", ["events", "host"])
+def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync):
     """GPU->Host runs concurrently with the forward pass; layer l may be saved
-    only after the model recorded post_events[l], so the host copy must hold
-    the K/V written in THIS step for every layer."""
+    only after the model recorded post_events[l] (sync="events": the worker's
+    stream waits for the event; sync="host": the doorbell itself is rung only
+    once the event has completed), so the host copy must hold the K/V written
+    in THIS step for every layer."""
     s = wl.LLAMA_3_2_1B
     L, nb, nhb, bs, H, D = 6, 32, 8, s.block_size, s.num_kv_heads, s.head_dim
     pool_np = random_pool((L, nb, 2, bs, H, D), 1)
     dpool = to_bf16(pool_np, gpu)
-    handle = kvc.KVWorkerHandle.create(L)
+    handle = kvc.KVWorkerHandle.create(L, sync=sync)
     worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle)
     hooks = kvc.LayerSyncHooks(handle)
     hooks.enable_record_after_execute = True
@@ -76,17 +79,20 @@ def test_write_through_waits_for_each_layers_kv_write(gpu, mode):
         assert handle.kv_queue.empty()
     finally:
         worker.close()
+        handle.close()
 
 
 @pytest.mark.parametrize("mode", ["direct", "staged"])
-def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode):
-    """Host->GPU: the model waits per layer on pre_events[l] (after the doorbell)
+@pytest.mark.parametrize("sync", ["events", "host"])
+def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode, sync):
+    """Host->GPU: the model waits per layer on pre_events[l] (after the doorbell;
+    with sync="host" the doorbell alone, rung after the layer's load completed)
     and must then see that layer's fetched blocks."""
     s = wl.LLAMA_3_2_1B
     L, nb, nhb = 5, 24, 8
     pool_np = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), 5)
     dpool = to_bf16(pool_np, gpu)
-    handle = kvc.KVWorkerHandle.create(L)
+    handle = kvc.KVWorkerHandle.create(L, sync=sync)
     worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle)
     hooks = kvc.LayerSyncHooks(handle)
     hooks.enable_wait_before_execute = True
@@ -116,6 +122,7 @@ def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode):
         assert handle.model_queue.empty()
     finally:
         worker.close()
+        handle.close()
 
 
 def test_allocator_order_drives_a_realistic_decode_step(gpu):

@@ -134,6 +134,7 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
         orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
     dpool = to_bf16(pool, gpu)
     _lib.set_tuning("write_narrow_vpt", vpt)
+    _lib.set_tuning("write_narrow", 2)          # whatever the launch size
     if paged:
         # requests of up to three tokens, each token on a page of its own:
         # page = slot // bs at table entry j, position = j * bs + slot % bs
@@ -161,9 +162,10 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
 
 
 def test_narrow_kernel_switch_and_strided_sources(gpu):
-    """`write_narrow = 0` sends narrow rows through the token-per-workgroup kernel;
-    both kernels agree with the oracle on token-strided sources (slices of a wider
-    projection), where the source side is no longer one run."""
+    """`write_narrow = 0` sends narrow rows through the token-per-workgroup kernel,
+    `2` through the plane kernel whatever the size; both agree with the oracle on
+    token-strided sources (slices of a wider projection), where the source side
+    is no longer one run. By default the launch size decides."""
     T, H, D, bs, nb = 130, 1, 128, 16, 40
     rng = np.random.default_rng(5)
     slots = rng.permutation(nb * bs)[:T].astype(np.int64)
@@ -176,13 +178,30 @@ def test_narrow_kernel_switch_and_strided_sources(gpu):
     dk = to_bf16(wide_k, gpu)[:, H * D:2 * H * D].view(T, H, D)
     dv = to_bf16(wide_v, gpu)[:, 2 * H * D:].view(T, H, D)
     assert not dk.is_contiguous()
-    for narrow, kernel in ((1, _lib.KVC_KERNEL_WRITE_ROWS_NARROW), (0, _lib.KVC_KERNEL_WRITE_ROWS)):
+    for narrow, kernel in ((2, _lib.KVC_KERNEL_WRITE_ROWS_NARROW), (0, _lib.KVC_KERNEL_WRITE_ROWS)):
         _lib.set_tuning("write_narrow", narrow)
         dpool = to_bf16(pool, gpu)
         kvc.reshape_and_cache(dk, dv, dpool, torch.from_numpy(slots).to(gpu))
         torch.cuda.synchronize()
         assert _lib.last_launch()["kernel"] == kernel
         assert np.array_equal(bits_of(dpool), want)
+    _lib.reset_tuning()
+    # by size: 130 tokens x 2 planes x 256 bytes stay with the token kernel, 16 layers of
+    # 512 tokens (4 MiB of source rows) take the plane kernel
+    kvc.reshape_and_cache(dk, dv, to_bf16(pool, gpu), torch.from_numpy(slots).to(gpu))
+    assert _lib.last_launch()["kernel"] == _lib.KVC_KERNEL_WRITE_ROWS
+    Lb, Tb = 16, 512
+    big_slots = np.random.default_rng(6).permutation(nb * bs)[:Tb].astype(np.int64)
+    bk, bv = bf16_bits((Lb, Tb, H, D), 7), bf16_bits((Lb, Tb, H, D), 8)
+    big_pool = sentinel_pool((Lb, nb, 2, bs, H, D), 9)
+    big_want = big_pool.copy()
+    for l in range(Lb):
+        orc.c_reshape_and_cache(bk[l], bv[l], big_want[l], big_slots)
+    dbig = to_bf16(big_pool, gpu)
+    kvc.reshape_and_cache_layers(to_bf16(bk, gpu), to_bf16(bv, gpu), dbig, torch.from_numpy(big_slots).to(gpu))
+    torch.cuda.synchronize()
+    assert _lib.last_launch()["kernel"] == _lib.KVC_KERNEL_WRITE_ROWS_NARROW
+    assert np.array_equal(bits_of(dbig), big_want)
 
 
 def test_config1_llama_1b_write_all_layers(gpu):
