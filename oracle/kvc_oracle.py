@@ -82,6 +82,60 @@ def get_batch_indices_positions_np(append_indptr, seq_lens, nnz) -> Tuple[np.nda
     return batch.astype(np.int32), pos.astype(np.int32)
 
 
+def build_write_index_np(input_lens, context_lens, num_blocks, kv_indices, page_size):
+    """The whole index of a step from the per-request scalars the scheduler sends
+    (proto/worker.proto:40-47), as `ModelWorker._make_inputs` builds it piecewise
+    on the host (model_worker.py:346 position_ids, :362-365 cu_seqlens_q, :399-423
+    page table and last-page fill), the two flashinfer calls derive it
+    (model_worker.py:425-433) and the scheduler's slot rule places it
+    (scheduler.rs:453-541, block_manager.rs:241-273):
+        cu_seqlens_q = [0, cumsum(input_lens)], kv_indptr = [0, cumsum(num_blocks)],
+        last_page_len[b] = (context_lens[b] - 1) % page_size + 1,
+        for the j-th new token of request b:
+            batch_indices = b, position = context_lens[b] - input_lens[b] + j,
+            slot = kv_indices[kv_indptr[b] + position // page_size] * page_size + position % page_size
+    A position outside its request's own table yields slot -1. Requests are taken in
+    the order given (the caller has sorted them, model_worker.py:326-328). Returns
+    (cu_seqlens_q, kv_indptr, last_page_len, batch_indices, positions, slot_mapping):
+    int32 except the int64 slot mapping."""
+    q = np.asarray(input_lens, dtype=np.int64)
+    ctx = np.asarray(context_lens, dtype=np.int64)
+    nblk = np.asarray(num_blocks, dtype=np.int64)
+    table = np.asarray(kv_indices, dtype=np.int64)
+    cu = np.concatenate([[0], np.cumsum(q)])
+    indptr = np.concatenate([[0], np.cumsum(nblk)])
+    last = np.where(ctx > 0, (ctx - 1) % page_size + 1, 0)
+    batch = np.repeat(np.arange(len(q), dtype=np.int64), q)
+    within = np.arange(int(cu[-1]), dtype=np.int64) - cu[:-1][batch]
+    pos = ctx[batch] - q[batch] + within
+    entry = indptr[:-1][batch] + pos // page_size
+    ok = (pos >= 0) & (entry >= 0) & (entry < np.minimum(indptr[1:][batch], len(table)))
+    slots = np.full(len(batch), -1, dtype=np.int64)
+    slots[ok] = table[entry[ok]] * page_size + pos[ok] % page_size
+    i32 = np.int32
+    return (cu.astype(i32), indptr.astype(i32), last.astype(i32), batch.astype(i32), pos.astype(i32), slots)
+
+
+def build_write_index_loops(input_lens, context_lens, num_blocks, kv_indices, page_size):
+    """`build_write_index_np` request by request and token by token."""
+    cu, indptr, last, batch, pos, slots = [0], [0], [], [], [], []
+    for b, (q, ctx, nblk) in enumerate(zip(input_lens, context_lens, num_blocks)):
+        q, ctx, nblk = int(q), int(ctx), int(nblk)
+        table = [int(x) for x in kv_indices[indptr[-1]:indptr[-1] + nblk]]
+        cu.append(cu[-1] + q)
+        indptr.append(indptr[-1] + nblk)
+        last.append((ctx - 1) % page_size + 1 if ctx > 0 else 0)
+        for j in range(q):
+            p = ctx - q + j
+            batch.append(b)
+            pos.append(p)
+            page = p // page_size
+            slots.append(table[page] * page_size + p % page_size if p >= 0 and page < len(table) else -1)
+    i32 = np.int32
+    return (np.asarray(cu, dtype=i32), np.asarray(indptr, dtype=i32), np.asarray(last, dtype=i32),
+            np.asarray(batch, dtype=i32), np.asarray(pos, dtype=i32), np.asarray(slots, dtype=np.int64))
+
+
 def copy_blocks_np(kv_caches, block_maps) -> None:
     """ops/cache_ops.py:8-36 + ops/triton/cache_kernels.py:5-36 on the pool
     viewed as [L, nb, block_elems]; NumPy evaluates the right-hand side first,

@@ -11,6 +11,10 @@ ops/rotary_embedding_ops.py:8-35) and of its cos/sin table
                           storage dtype (what the HIP kernel implements)
   rotary_pos_emb_per_op   every product and sum rounded to the storage dtype,
                           the way a bf16-typed Triton expression evaluates
+                          (three roundings per lane)
+  rotary_pos_emb_fma      the same expression with one product contracted into
+                          a fused multiply-add: two roundings per lane, either
+                          product being the one that is rounded on its own
 
 Pinned in tests/test_rope_oracle.py against complex multiplication
 (x + iy)(cos + i sin), the identity at position 0, norm preservation and
@@ -81,6 +85,40 @@ def rotary_pos_emb_per_op(query, key, positions, cos_sin_cache, head_dim):
     cos, sin = cs[:, :rd], cs[:, rd:]
     return (_rotate_torch(query, cos, sin, head_dim, rd, query.dtype, query.dtype),
             _rotate_torch(key, cos, sin, head_dim, rd, key.dtype, key.dtype))
+
+
+def rotary_pos_emb_fma(query, key, positions, cos_sin_cache, head_dim, rounded="second"):
+    """`a*b - c*d` evaluated as a fused multiply-add over ONE product rounded to the
+    storage dtype: `rounded="second"` is fma(a, b, -rn(c*d)), `"first"` is
+    fma(-c, d, rn(a*b)); the sum is rounded once. The exact products of two
+    16-bit-or-narrower operands fit float64, so float64 stands in for the
+    unrounded fma. Storage dtypes bf16 / fp16."""
+    if rounded not in ("first", "second"):
+        raise ValueError("rounded must be 'first' or 'second'")
+    rd = cos_sin_cache.shape[1] // 2
+    half = rd // 2
+    cs = cos_sin_cache[positions.long()]
+    cos, sin = cs[:, None, :rd].double(), cs[:, None, rd:].double()
+
+    def rotate(x):
+        dt = x.dtype
+        T = x.shape[0]
+        xh = x.reshape(T, -1, head_dim)
+        a, b = xh[:, :, :half].double(), xh[:, :, half:rd].double()
+
+        def rn(t):
+            return t.to(dt).double()
+
+        def fused(p1, p2):          # p1 - p2 (or p1 + p2 below) with one of them pre-rounded
+            return (rn(p1) - p2) if rounded == "first" else (p1 - rn(p2))
+
+        out = xh.clone()
+        out[:, :, :half] = fused(a * cos[:, :, :half], b * sin[:, :, :half]).to(dt)
+        # y*cos + x*sin = y*cos - (-(x*sin))
+        out[:, :, half:rd] = fused(b * cos[:, :, half:], -(a * sin[:, :, half:])).to(dt)
+        return out.reshape(x.shape)
+
+    return rotate(query), rotate(key)
 
 
 def cos_sin_table_f64(rotary_dim, max_position, base=10000.0, rope_scaling=None):

@@ -85,6 +85,14 @@ def test_one_launch_index_build_matches_the_host_construction(gpu, kind):
     host = kvc.make_kv_index_inputs(reqs, bs)
     dev = kvc.to_device_one_launch(reqs, bs, gpu)
     torch.cuda.synchronize()
+    # the oracle's statement of the same index, from the per-request scalars in batch order
+    ordered = [reqs[i] for i in host.order]
+    want = orc.build_write_index_np([r.input_len for r in ordered], [r.context_len for r in ordered],
+                                    [len(r.block_ids) for r in ordered],
+                                    [b for r in ordered for b in r.block_ids], bs)
+    for got, exp in zip((dev.cu_seqlens_q, dev.kv_block_indptrs, dev.kv_last_block_lens,
+                         dev.batch_indices, dev.positions, dev.slot_mapping), want):
+        assert np.array_equal(got.cpu().numpy(), exp)
     assert np.array_equal(dev.cu_seqlens_q.cpu().numpy(), host.cu_seqlens_q)
     assert np.array_equal(dev.kv_block_indptrs.cpu().numpy(), host.kv_block_indptrs)
     assert np.array_equal(dev.kv_last_block_lens.cpu().numpy(), host.kv_last_block_lens)

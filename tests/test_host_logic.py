@@ -66,6 +66,57 @@ def test_make_kv_index_inputs_orders_prefill_first_and_builds_the_page_table():
     assert bi.tolist() == idx.batch_indices.tolist() and pos.tolist() == idx.positions.tolist()
 
 
+def test_index_oracle_reproduces_the_hand_case_and_its_own_loops():
+    """`oracle.build_write_index_*` on the step written out by hand above (requests
+    already in batch order), then NumPy against loops on random steps, and against
+    the two pinned page-table functions."""
+    bs = 4
+    #            prefill 5   continuation 3   decode      decode
+    input_lens, context_lens, tables = [5, 3, 1, 1], [5, 11, 7, 4], [[4, 2], [1, 5, 6], [3, 9], [7]]
+    flat = [b for t in tables for b in t]
+    for build in (orc.build_write_index_np, orc.build_write_index_loops):
+        cu, indptr, last, bi, pos, slots = build(input_lens, context_lens, [len(t) for t in tables], flat, bs)
+        assert cu.tolist() == [0, 5, 8, 9, 10]
+        assert indptr.tolist() == [0, 2, 5, 7, 8]
+        assert last.tolist() == [1, 3, 3, 4]
+        assert bi.tolist() == [0] * 5 + [1] * 3 + [2, 3]
+        assert pos.tolist() == [0, 1, 2, 3, 4, 8, 9, 10, 6, 3]
+        assert slots.tolist() == [16, 17, 18, 19, 8, 24, 25, 26, 9 * 4 + 2, 7 * 4 + 3]
+        assert slots.dtype == np.int64 and pos.dtype == np.int32
+    # a request whose table is too short for its context: slot -1, never the next request's block
+    _, _, _, _, pos, slots = orc.build_write_index_np([1, 1], [20, 5], [1, 1], [7, 3], 16)
+    assert pos.tolist() == [19, 4] and slots.tolist() == [-1, 3 * 16 + 4]
+    assert orc.build_write_index_loops([1, 1], [20, 5], [1, 1], [7, 3], 16)[5].tolist() == [-1, 52]
+    rng = np.random.default_rng(3)
+    for _ in range(20):
+        B = int(rng.integers(0, 9))
+        q = rng.integers(0, 40, size=B)
+        ctx = q + rng.integers(0, 100, size=B)
+        extra = rng.integers(0, 3, size=B)             # tables may hold blocks beyond the context
+        nblk = (ctx + bs - 1) // bs + extra
+        table = rng.permutation(int(nblk.sum()) + 5)[:int(nblk.sum())]
+        a = orc.build_write_index_np(q, ctx, nblk, table, bs)
+        b = orc.build_write_index_loops(q, ctx, nblk, table, bs)
+        for x, y in zip(a, b):
+            assert np.array_equal(x, y) and x.dtype == y.dtype
+        seq_lens = orc.get_seq_lens_np(a[1], a[2], bs)
+        keep = (ctx > 0) & (extra == 0)
+        # model_worker.py:399-408 passes exactly the blocks of [0, context_len): seq_len == context_len
+        assert np.array_equal(seq_lens[keep], ctx[keep])
+        bi, pos = orc.get_batch_indices_positions_np(a[0], ctx.astype(np.int32), int(q.sum()))
+        assert np.array_equal(bi, a[3]) and np.array_equal(pos, a[4])
+    # and the host-side construction of the package agrees with the oracle on a mixed step
+    w = wl._write_workload(wl.LLAMA_3_2_1B, 256, [0, 37, 5, 64], [70, 1, 1, 33], np.random.default_rng(1))
+    host = make_kv_index_inputs(w.inputs, 16)
+    reqs = [w.inputs[i] for i in host.order]
+    got = orc.build_write_index_np([r.input_len for r in reqs], [r.context_len for r in reqs],
+                                   [len(r.block_ids) for r in reqs],
+                                   [b for r in reqs for b in r.block_ids], 16)
+    for x, y in zip(got, (host.cu_seqlens_q, host.kv_block_indptrs, host.kv_last_block_lens,
+                          host.batch_indices, host.positions, host.slot_mapping)):
+        assert np.array_equal(x, y)
+
+
 def test_make_kv_index_inputs_rejects_inconsistent_requests():
     with pytest.raises(ValueError):
         make_kv_index_inputs([InferInput(0, [1, 1], 2, 0, 3, [0])], 4)   # len mismatch

@@ -125,3 +125,37 @@ def test_llama3_scaling_bands():
     # and the product's table follows the same bands
     got = make_cos_sin_cache(rd, 2, base, LLAMA3_SCALING, dtype=torch.float32).double().numpy()
     assert np.abs(got - scaled).max() < 1e-6
+
+
+def test_fma_variants_sit_between_one_and_three_roundings():
+    """The two-rounding variants: within u*|rounded product| + u*|result| of the float64
+    formula (u = 2^-8 for bf16: half an ulp of 8 significant bits), i.e. tighter than the three-rounding bound and
+    looser than a single rounding; at position 0 (cos = 1, sin = 0) they are the
+    identity like the others."""
+    import torch
+    from lmserve_amd import rotary
+    g = torch.Generator().manual_seed(5)
+    T, H, D = 64, 4, 64
+    q = torch.randn(T, H * D, generator=g).to(torch.bfloat16)
+    k = torch.randn(T, H * D, generator=g).to(torch.bfloat16)
+    pos = torch.randint(0, 512, (T,), generator=g)
+    cs = rotary.make_cos_sin_cache(D, 512, 10000.0, dtype=torch.bfloat16)
+    exact_q, _ = ro.rotary_pos_emb_f64(q.double().numpy(), k.double().numpy(), pos.numpy(), cs.double().numpy(), D)
+    u = 2.0 ** -8
+    xh = q.double().numpy().reshape(T, H, D)
+    c = cs[pos].double().numpy()
+    cos, sin = c[:, None, :D], c[:, None, D:]
+    half = D // 2
+    a, b = xh[:, :, :half], xh[:, :, half:]
+    prods = {"first": np.concatenate([np.abs(a * cos[:, :, :half]), np.abs(b * cos[:, :, half:])], axis=2),
+             "second": np.concatenate([np.abs(b * sin[:, :, :half]), np.abs(a * sin[:, :, half:])], axis=2)}
+    for which in ("first", "second"):
+        got, _ = ro.rotary_pos_emb_fma(q, k, pos, cs, D, rounded=which)
+        err = np.abs(got.double().numpy() - exact_q)
+        bound = u * prods[which].reshape(T, -1) + u * np.abs(exact_q) * 1.001 + 1e-30
+        assert (err <= bound).all(), which
+        zero = torch.zeros(T, dtype=torch.long)
+        same_q, same_k = ro.rotary_pos_emb_fma(q, k, zero, cs, D, rounded=which)
+        assert torch.equal(same_q, q) and torch.equal(same_k, k)
+    with pytest.raises(ValueError):
+        ro.rotary_pos_emb_fma(q, k, pos, cs, D, rounded="both")
