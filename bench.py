@@ -62,6 +62,8 @@ def parse_args():
                         "index (index preparation of a step: host construction vs one launch), "
                         "sweep (write / copy_blocks / plain kernel over launch sizes; not in the default), "
                         "calib (a plain elementwise kernel of known size, for counter calibration); "
+                        "translation (the config 3 launch with dense, block-run and random slots, for "
+                        "address-translation counter runs; not in the default); "
                         "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=8192,
                    help="blocks per swap direction; 8192 (40 GiB pinned) is config 5 at its stated size")
@@ -712,6 +714,53 @@ def main():
                                    calls_per_step=L3, launch="hipGraph replay"))
             del q3, k3, v3, plans3, qo3
         del sets3, pool3
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------ config 3 launch, three slot patterns
+    # (for counter runs: the same 2048-token x 28-layer launch writing one dense run per
+    # layer, the workload's scattered 16-token block runs, and fully random rows; the
+    # write_rows_kernel dispatches appear in that order, `reps` + 2 of each)
+    if "translation" in ops:
+        sq = wl.QWEN_2_5_7B
+        nbq = 16384
+        poolq, Lq = alloc_pool(torch, sq, nbq, dev)
+        Tq, Rq, reps = 2048, ROTATE_PREFILL, max(2, min(args.steps, 64))
+        srcs = []
+        for r in range(Rq):
+            kq = torch.randn(Lq, Tq, sq.num_kv_heads, sq.head_dim, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            srcs.append((kq, torch.randn_like(kq)))
+        patterns = (
+            ("one dense run per layer (slots 0..2047)",
+             [torch.arange(Tq, dtype=torch.int64, device=dev) for _ in range(Rq)]),
+            ("the workload's block runs (4 sequences x 32 scattered blocks of 16 tokens)",
+             [torch.from_numpy(wl.chunked_prefill(sq, num_blocks=nbq, seed=r).index.slot_mapping).to(dev)
+              for r in range(Rq)]),
+            ("random rows (2048 distinct random slots)",
+             [torch.from_numpy(wl.random_free_slots(sq, nbq, Tq, seed=r)).to(dev) for r in range(Rq)]),
+        )
+        nbytes = 2 * 2 * Tq * sq.row_bytes * Lq + 8 * Tq
+        rounds = 3                      # patterns interleaved, so drift hits all of them alike
+        per_pattern = {label: [] for label, _ in patterns}
+        for rnd in range(rounds):
+            for label, slot_sets in patterns:
+                for i in range(2):
+                    kvc.reshape_and_cache_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, slot_sets[i % Rq])
+                torch.cuda.synchronize()
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for i in range(reps):
+                    kvc.reshape_and_cache_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, slot_sets[i % Rq])
+                end.record()
+                torch.cuda.synchronize()
+                per_pattern[label].append(start.elapsed_time(end) / reps)
+                log(f"translation: round {rnd}: {reps + 2} write_rows_kernel dispatches, {label}, "
+                    f"{per_pattern[label][-1] * 1e3:.2f} us each")
+        for label, _ in patterns:
+            ms = sorted(per_pattern[label])[rounds // 2]
+            extra.append(entry(f"cfg3 launch, slot pattern: {label}", nbytes, ms, ms, launch="eager",
+                               launches_per_round=reps + 2, rounds=rounds,
+                               us_per_round=[round(x * 1e3, 2) for x in per_pattern[label]]))
+        del poolq, srcs
         torch.cuda.empty_cache()
 
     # ------------------------------------------------ config 5: swap round trip

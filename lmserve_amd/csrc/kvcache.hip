@@ -68,10 +68,14 @@ struct Tuning {
   int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
   int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
-  int write_narrow = 1;     // rows under 1 KiB: lanes of a wavefront run over consecutive tokens of
-                            // one (layer, K|V) plane instead of over one token's planes
-                            // (0 = never, 1 = for launches of write_narrow_min_bytes and more, 2 = always)
-  int write_narrow_min_bytes = 2 << 20;  // source bytes of a launch from which that kernel runs
+  int write_narrow = 1;     // the plane kernel (lanes of a workgroup run over consecutive tokens of
+                            // one (layer, K|V) plane): 0 = never, 1 = by row width and launch size,
+                            // 2 = whenever the row shape allows
+  int write_narrow_min_bytes = 2 << 20;  // rows under 1 KiB: source bytes of a launch from which it runs
+  int write_narrow_max_vpr = 256;        // widest row (in 16-byte vectors) that kernel takes
+  int write_narrow_threads = 0;          // lanes per workgroup of that kernel (256, 512, 1024), 0 = by rule
+  int write_pipe = -1;                   // 1 = a lane waits for each load before issuing its next,
+                                         // 0 = loads back to back, -1 = by rule
   int write_narrow_vpt = 0; // planes per lane in that kernel (1, 2, 4, 8), 0 = by size
   int direct_max_wgs = 64;  // grid cap of the direct swap kernel: PCIe saturates with a few
                             // dozen workgroups, the rest of the GPU stays free for the model
@@ -98,6 +102,9 @@ Knob* knobs(int* count) {
       {"write_narrow", &g_tune.write_narrow, 1},
       {"write_narrow_vpt", &g_tune.write_narrow_vpt, 0},
       {"write_narrow_min_bytes", &g_tune.write_narrow_min_bytes, 2 << 20},
+      {"write_narrow_max_vpr", &g_tune.write_narrow_max_vpr, 256},
+      {"write_narrow_threads", &g_tune.write_narrow_threads, 0},
+      {"write_pipe", &g_tune.write_pipe, -1},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 64},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
@@ -167,6 +174,9 @@ struct WriteArgs {
   uint32_t items_per_token;  // 2 * num_layers * vecs_per_row; item = (layer, K|V, vec)
   uint32_t num_groups;       // workgroups per token
   int groups_fastest;        // blockIdx.x = token * num_groups + group (else group * T + token)
+  int pipe;                  // 1 = a lane waits for each of its loads before issuing the next one,
+                             // so that the lanes of a launch that is resident all at once drift
+                             // apart and reads overlap writes
   int64_t key_token_stride, value_token_stride;
   int64_t key_layer_stride, value_layer_stride;
   int64_t block_size;
@@ -203,31 +213,30 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   const char* key_row = a.key + (int64_t)t * a.key_token_stride;
   const char* value_row = a.value + (int64_t)t * a.value_token_stride;
   const uint32_t first = group * (VPT * blockDim.x) + threadIdx.x;
+  // item -> (row r = 2*layer + K|V, vector inside the row)
+  const auto split = [&](uint32_t item, uint32_t& r, uint32_t& vec) {
+    if (a.vpr_shift >= 0) {
+      r = item >> a.vpr_shift;
+      vec = item & (a.vecs_per_row - 1u);
+    } else {
+      r = item / a.vecs_per_row;
+      vec = item - r * a.vecs_per_row;
+    }
+  };
+  // Loads are unconditional (an item index past the token's last vector is
+  // clamped to it and its store skipped): straight-line code keeps the register
+  // count at the data registers plus a few addresses, whatever VPT.
   V data[VPT];
-  int64_t dst_off[VPT];  // offset from the slot's K (or V) row, < 0 = no item
-  bool to_v[VPT];
+  const uint32_t last_item = a.items_per_token - 1u;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    const uint32_t item = first + j * blockDim.x;
-    dst_off[j] = -1;
-    to_v[j] = false;
-    if (item < a.items_per_token) {
-      uint32_t r, vec;
-      if (a.vpr_shift >= 0) {
-        r = item >> a.vpr_shift;
-        vec = item & (a.vecs_per_row - 1u);
-      } else {
-        r = item / a.vecs_per_row;
-        vec = item - r * a.vecs_per_row;
-      }
-      const int64_t layer = r >> 1;
-      const bool is_v = r & 1u;
-      const char* src = (is_v ? value_row + layer * a.value_layer_stride
-                              : key_row + layer * a.key_layer_stride) + (int64_t)vec * VEC;
-      data[j] = ld<NTL>(reinterpret_cast<const V*>(src));
-      dst_off[j] = layer * a.cache_layer_stride + (int64_t)vec * VEC;
-      to_v[j] = is_v;
-    }
+    uint32_t r, vec;
+    split(min(first + j * blockDim.x, last_item), r, vec);
+    const int64_t layer = r >> 1;
+    const char* src = ((r & 1u) ? value_row + layer * a.value_layer_stride
+                                : key_row + layer * a.key_layer_stride) + (int64_t)vec * VEC;
+    data[j] = ld<NTL>(reinterpret_cast<const V*>(src));
+    if (VPT > 1 && a.pipe == 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
 
   int64_t blk, off;
@@ -266,8 +275,13 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   char* vc_row = a.value_cache + slot_off;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    if (dst_off[j] >= 0)
-      st<NT>(reinterpret_cast<V*>((to_v[j] ? vc_row : kc_row) + dst_off[j]), data[j]);
+    const uint32_t item = first + j * blockDim.x;
+    if (item <= last_item) {
+      uint32_t r, vec;
+      split(item, r, vec);
+      char* dst = ((r & 1u) ? vc_row : kc_row) + (int64_t)(r >> 1) * a.cache_layer_stride + (int64_t)vec * VEC;
+      st<NT>(reinterpret_cast<V*>(dst), data[j]);
+    }
   }
 }
 
@@ -282,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
 // number of them per row only; blockIdx.x = plane_group * num_token_groups +
 // token_group.
 template <int VPT, bool PAGED, bool NT>
-__global__ __launch_bounds__(kThreads) void write_rows_narrow_kernel(WriteArgs a) {
+__global__ __launch_bounds__(1024) void write_rows_narrow_kernel(WriteArgs a) {
   using V = u32x4;
   const uint32_t pg = blockIdx.x / a.num_token_groups;
   const uint32_t tg = blockIdx.x - pg * a.num_token_groups;
@@ -291,16 +305,22 @@ __global__ __launch_bounds__(kThreads) void write_rows_narrow_kernel(WriteArgs a
   const int64_t vec_off = (int64_t)(threadIdx.x & (a.vecs_per_row - 1u)) * 16;
   const char* key_row = a.key + (int64_t)t * a.key_token_stride + vec_off;
   const char* value_row = a.value + (int64_t)t * a.value_token_stride + vec_off;
+  // Loads are unconditional (a plane index past the end is clamped to the last
+  // plane and its store skipped): straight-line code keeps the register count
+  // at the data registers plus a few addresses.
   V data[VPT];
+  const uint32_t last_plane = a.num_planes - 1u;
+  const auto load_plane = [&](int j) {
+    const uint32_t plane = min(pg * VPT + j, last_plane);
+    const int64_t layer = plane >> 1;
+    const char* src = (plane & 1u) ? value_row + layer * a.value_layer_stride
+                                   : key_row + layer * a.key_layer_stride;
+    return *reinterpret_cast<const V*>(src);
+  };
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
-    const uint32_t plane = pg * VPT + j;
-    if (plane < a.num_planes) {
-      const int64_t layer = plane >> 1;
-      const char* src = (plane & 1u) ? value_row + layer * a.value_layer_stride
-                                     : key_row + layer * a.key_layer_stride;
-      data[j] = *reinterpret_cast<const V*>(src);
-    }
+    data[j] = load_plane(j);
+    if (VPT > 1 && a.pipe == 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   int64_t blk, off;
   if constexpr (PAGED) {
@@ -689,41 +709,69 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
   a.cache_slot_stride = g.cache_slot_stride * E;
   a.cache_layer_stride = g.cache_layer_stride * E;
   a.num_cache_blocks = g.num_cache_blocks;
-
   const int64_t items64 = 2 * g.num_layers * (int64_t)a.vecs_per_row;
   if (items64 > 0x7fffffffll)
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per token exceed 2^31", fn, (long long)items64);
   a.items_per_token = (uint32_t)items64;
 
-  // Rows under 1 KiB: lanes run over consecutive tokens of one plane, once the
-  // launch is large enough for bandwidth to matter. Below about 2 MiB of source
-  // rows a launch is latency-bound and many small token-per-workgroup workgroups
-  // with a scalar slot lookup finish first (one layer of a 2048-token chunk at
-  // 256-byte rows: 2.53 against 2.80 us; 80 layers of a 64-token step: 4.04
-  // against 3.67 us).
-  const bool narrow_rows = vec == 16 && a.vpr_shift >= 0 && a.vecs_per_row < 64;
-  const bool narrow_pays = g_tune.write_narrow >= 2 ||
-                           g.num_tokens * 2 * g.num_layers * g.row_elems * E >= g_tune.write_narrow_min_bytes;
-  if (g_tune.write_narrow && narrow_rows && narrow_pays) {
+  // The plane kernel (lanes over consecutive tokens of one (layer, K|V) plane)
+  // takes rows of a power-of-two number of 16-byte vectors up to 4 KiB. From
+  // sweeps on MI355X (rows of 256 B to 2 KiB, 5 MiB to 512 MiB per launch):
+  //   - rows under 1 KiB: from about 2 MiB of source rows per launch; below that a
+  //     launch is latency-bound and many small token-per-workgroup workgroups with
+  //     a scalar slot lookup finish first (one layer of a 2048-token chunk at
+  //     256-byte rows: 2.53 against 2.80 us; 80 layers of a 64-token step: 4.04
+  //     against 3.67 us);
+  //   - wider rows: when the launch is at least one resident set of lanes at one
+  //     vector per lane and 2, 4 or 8 planes per lane bring it down to one resident
+  //     set (2048 lanes per CU); then no second round of workgroups is dispatched
+  //     and every lane has several loads in flight (Llama-3-8B decode step, 64 MiB:
+  //     12.3-12.5 us against 13.0-13.6 for the token kernel; 128 MiB: 24.8 against
+  //     26.1). Larger launches stream best through the token kernel.
+  // In the one-resident-set regime every lane of the GPU is resident at once;
+  // if all of them issue all their loads and then all their stores, the launch
+  // splits into a read phase and a write phase and loses 15 % (14.4 against
+  // 12.4 us). A lane that waits for each load before issuing the next drifts
+  // apart from its neighbours and the two directions overlap; the page-table
+  // lookup, a chain of dependent loads per lane, has the same effect by itself.
+  const int64_t resident_lanes = (int64_t)resident_workgroups() * kThreads;
+  const bool plane_rows = vec == 16 && a.vpr_shift >= 0 &&
+                          (int64_t)a.vecs_per_row <= std::min(g_tune.write_narrow_max_vpr, 256);
+  const int64_t num_planes = 2 * g.num_layers;
+  const auto plane_lanes = [&](int v) {  // lanes of the launch at v planes per lane, 256-lane workgroups
+    const int64_t tpw = kThreads / (int64_t)a.vecs_per_row;
+    return (g.num_tokens + tpw - 1) / tpw * ((num_planes + v - 1) / v) * kThreads;
+  };
+  int fit_vpt = 0;  // fewest planes per lane that bring the launch within one resident set
+  if (plane_rows)
+    for (int v = 1; v <= 8 && !fit_vpt; v *= 2)
+      if (plane_lanes(v) <= resident_lanes) fit_vpt = v;
+  bool plane_pays = false;
+  if (plane_rows) {
+    if (g_tune.write_narrow >= 2) plane_pays = true;
+    else if (a.vecs_per_row < 64)
+      plane_pays = g.num_tokens * num_planes * g.row_elems * E >= g_tune.write_narrow_min_bytes;
+    else plane_pays = fit_vpt > 0 && plane_lanes(1) >= resident_lanes;
+  }
+  if (g_tune.write_narrow && plane_pays) {
     WriteLaunch l{};
-    const int64_t lanes_all = g.num_tokens * (int64_t)a.vecs_per_row;
-    l.threads = (unsigned)std::min<int64_t>(kThreads, (lanes_all + 63) / 64 * 64);
-    a.tokens_per_wg = l.threads / a.vecs_per_row;
-    a.num_planes = (uint32_t)(2 * g.num_layers);
-    const int64_t token_groups_all = (g.num_tokens + a.tokens_per_wg - 1) / a.tokens_per_wg;
     l.vpt = g_tune.write_narrow_vpt;
-    if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8) {
-      // the fewest planes per lane (up to 4) that keep the launch within one resident
-      // set of workgroups; a launch larger than that streams with one plane per lane
-      const int64_t resident = resident_workgroups();
-      l.vpt = 1;
-      for (int v = 1; v <= 4; v *= 2)
-        if (token_groups_all * ((a.num_planes + v - 1) / v) <= resident) {
-          l.vpt = v;
-          break;
-        }
-    }
-    while (l.vpt > 1 && (uint32_t)(l.vpt / 2) >= a.num_planes) l.vpt /= 2;
+    if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8)
+      l.vpt = fit_vpt ? fit_vpt : 1;  // beyond one set: stream
+    // a page-table lookup per lane wants at least two planes to pay for itself
+    if (paged && l.vpt == 1 && g_tune.write_narrow_vpt != 1) l.vpt = 2;
+    while (l.vpt > 1 && (int64_t)(l.vpt / 2) >= num_planes) l.vpt /= 2;
+    // slot-mapped launches of 4 or 8 planes per lane: 512-lane workgroups whose lanes
+    // wait for each load (see above); everything else 256 lanes, loads back to back
+    const bool deep_slot = !paged && l.vpt >= 4;
+    int wg_lanes = g_tune.write_narrow_threads;
+    if (wg_lanes != 256 && wg_lanes != 512 && wg_lanes != 1024) wg_lanes = deep_slot ? 512 : 256;
+    a.pipe = g_tune.write_pipe >= 0 ? g_tune.write_pipe : (deep_slot ? 1 : 0);
+    const int64_t lanes_all = g.num_tokens * (int64_t)a.vecs_per_row;
+    l.threads = (unsigned)std::min<int64_t>(wg_lanes, (lanes_all + 63) / 64 * 64);
+    if (l.threads < a.vecs_per_row) l.threads = a.vecs_per_row;  // a row never splits over workgroups
+    a.tokens_per_wg = l.threads / a.vecs_per_row;
+    a.num_planes = (uint32_t)num_planes;
     l.nt = (g_tune.write_nt & 1) != 0;
     const int64_t plane_groups = (a.num_planes + l.vpt - 1) / l.vpt;
     const int64_t max_groups = std::max<int64_t>(1, 0x7fffffffll / plane_groups);
@@ -785,6 +833,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
   l.threads = (unsigned)std::min<int64_t>(wg, (lanes + 63) / 64 * 64);
   l.nt = (g_tune.write_nt & 1) != 0;
   l.ntl = (g_tune.write_nt & 2) != 0;
+  a.pipe = g_tune.write_pipe >= 0 ? g_tune.write_pipe : (l.vpt > 1 ? 1 : 0);
   const int64_t groups = (items64 + (int64_t)l.vpt * l.threads - 1) / ((int64_t)l.vpt * l.threads);
 
   a.num_groups = (uint32_t)groups;

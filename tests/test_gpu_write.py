@@ -90,9 +90,11 @@ def test_write_rows_every_launch_shape(gpu, vpt, nt, threads):
     for l in range(L):
         orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
     dpool = to_bf16(pool, gpu)
+    _lib.set_tuning("write_narrow", 0)    # the token kernel, whatever the size
     _lib.set_tuning("write_vpt", vpt)     # the autouse fixture puts the defaults back
     _lib.set_tuning("write_nt", nt)
     _lib.set_tuning("write_threads", threads)
+    _lib.set_tuning("write_pipe", nt & 1)  # both load orders over the sweep
     kvc.reshape_and_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool,
                                  torch.from_numpy(slots).to(gpu))
     torch.cuda.synchronize()
@@ -115,6 +117,10 @@ NARROW_CASES = [
     (300, 1, 32, 7, 4),      # 64-byte rows
     (1000, 1, 8, 2, 0),      # 16-byte rows: one vector per row
     (1, 1, 128, 1, 0),
+    (70, 8, 128, 6, 4),      # 2 KiB rows (Llama-3-8B): two tokens per 256-lane workgroup
+    (70, 8, 128, 6, 8),
+    (33, 16, 128, 3, 2),     # 4 KiB rows: one token per workgroup, the widest the kernel takes
+    (90, 4, 128, 9, 0),      # 1 KiB rows (Qwen2.5-7B), depth by rule
 ]
 
 
@@ -135,6 +141,9 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
     dpool = to_bf16(pool, gpu)
     _lib.set_tuning("write_narrow_vpt", vpt)
     _lib.set_tuning("write_narrow", 2)          # whatever the launch size
+    # workgroup size and load order vary over the cases (both are by rule otherwise)
+    _lib.set_tuning("write_narrow_threads", (0, 256, 512, 1024)[(T + L) % 4])
+    _lib.set_tuning("write_pipe", (-1, 0, 1)[(T + vpt) % 3])
     if paged:
         # requests of up to three tokens, each token on a page of its own:
         # page = slot // bs at table entry j, position = j * bs + slot % bs
@@ -438,12 +447,29 @@ def test_dtype_mismatch_raises(gpu):
                                   torch.zeros(1, dtype=torch.int32, device=gpu))
 
 
-@pytest.mark.parametrize("T", [40, 64, 100, 128, 200, 256, 300])
+# token count -> what the launch rule must pick on a 256-CU part for 32 layers of 2 KiB rows:
+# (kernel, planes or vectors per lane, lanes per workgroup) slot-mapped / page-table addressed
+_TOKEN, _PLANE = _lib.KVC_KERNEL_WRITE_ROWS, _lib.KVC_KERNEL_WRITE_ROWS_NARROW
+SIZE_RULE = {
+    40: ((_TOKEN, 1, 256), (_TOKEN, 1, 256)),      # under one resident set of lanes: token kernel
+    64: ((_PLANE, 1, 256), (_PLANE, 2, 256)),      # exactly one set at one plane per lane
+    100: ((_PLANE, 2, 256), (_PLANE, 2, 256)),
+    128: ((_PLANE, 2, 256), (_PLANE, 2, 256)),
+    200: ((_PLANE, 4, 512), (_PLANE, 4, 256)),     # deep slot-mapped lanes: 512-lane workgroups
+    256: ((_PLANE, 4, 512), (_PLANE, 4, 256)),     # the decode step of the benchmark
+    300: ((_PLANE, 8, 512), (_PLANE, 8, 256)),
+    600: ((_TOKEN, 1, 256), (_TOKEN, 1, 256)),     # no depth fits one set: stream through the token kernel
+}
+
+
+@pytest.mark.parametrize("T", sorted(SIZE_RULE))
 @pytest.mark.parametrize("paged", [False, True])
 def test_one_launch_write_through_every_shape_the_size_rule_picks(gpu, T, paged):
     """32 layers of the Llama-3-8B row in one launch, at token counts on both sides
-    of each switch of the launch-shape rule (256 lanes x 1 vector; 128 lanes x 2;
-    128 lanes x 4; back to 256 x 1), slot-mapped and page-table addressed."""
+    of each switch of the launch-shape rule (token kernel below one resident set of
+    lanes; plane kernel with 1, 2, 4 or 8 planes per lane while that brings the
+    launch within one set; token kernel again beyond), slot-mapped and page-table
+    addressed; the shape that ran is asserted as well as the bits."""
     s = wl.LLAMA_3_8B
     L, nb, bs = 32, 96, s.block_size
     w = wl.decode_step(s, num_blocks=nb, batch=T, max_context=4, seed=T) if T <= nb else \
@@ -465,4 +491,7 @@ def test_one_launch_write_through_every_shape_the_size_rule_picks(gpu, T, paged)
     else:
         kvc.reshape_and_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool, dev.slot_mapping)
     torch.cuda.synchronize()
+    ran = _lib.last_launch()
+    assert _lib.lib().kvc_tuning_modified() == 0
+    assert (ran["kernel"], ran["per_lane"], ran["threads"]) == SIZE_RULE[T][1 if paged else 0]
     assert np.array_equal(bits_of(dpool), want)
