@@ -17,7 +17,7 @@ SOURCES = [os.path.join(PKG_DIR, "csrc", "kvcache.hip"),
            os.path.join(PKG_DIR, "csrc", "disk_tier.cpp")]
 INCLUDE = os.path.join(REPO_ROOT, "include")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcache.so")
-FAST_SRC = os.path.join(PKG_DIR, "csrc", "fastcall.c")
+FAST_SRC = os.path.join(PKG_DIR, "csrc", "fastcall.cpp")
 FAST_PATH = os.path.join(PKG_DIR, "_kvc_fast.so")
 
 HIPCC_FLAGS = [
@@ -52,16 +52,25 @@ def build(verbose: bool = False) -> str:
 
 
 def build_fastcall(verbose: bool = False) -> str:
-    """Compile `_kvc_fast`, the CPython entry to the per-layer plan calls (plain
-    C, host compiler; links against libkvcache.so next to it)."""
+    """Compile `_kvc_fast`, the CPython entry to the per-layer plan calls (host C++
+    against torch's tensor headers; links against libkvcache.so next to it and
+    torch's Python library)."""
     import sysconfig
 
-    cc = shutil.which("gcc") or shutil.which("cc")
-    if cc is None:
-        raise RuntimeError("no C compiler for lmserve_amd/csrc/fastcall.c")
-    cmd = [cc, "-O2", "-std=c11", "-fPIC", "-shared", "-Wall", "-I", INCLUDE,
-           "-I", sysconfig.get_paths()["include"], FAST_SRC, "-L", PKG_DIR, "-lkvcache",
-           "-Wl,-rpath,$ORIGIN", "-o", FAST_PATH + ".tmp"]
+    import torch
+    from torch.utils import cpp_extension
+
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("no C++ compiler for lmserve_amd/csrc/fastcall.cpp")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-I", INCLUDE]
+    for inc in cpp_extension.include_paths():
+        cmd += ["-isystem", inc]
+    cmd += ["-I", sysconfig.get_paths()["include"], FAST_SRC, "-L", PKG_DIR, "-lkvcache",
+            "-L", torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10",
+            f"-Wl,-rpath,$ORIGIN,-rpath,{torch_lib}", "-o", FAST_PATH + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -218,7 +218,9 @@ class PagedKVWritePlan:
             self.elem, ctypes.byref(handle)))
         self._plan = handle.value
         fast = _lib.fast()
-        self._append = fast.write_plan_append if fast else lib.kvc_write_plan_append
+        self._fast_append = fast.write_plan_append if fast else None
+        self._dtype_code = fast.scalar_type_code(torch.empty(0, dtype=dtype)) if fast else -1
+        self._append = lib.kvc_write_plan_append
         self._destroy = lib.kvc_write_plan_destroy
         self._cache_shape_tail = torch.Size((2, self.page_size, self.H, self.D))
         self._k_plane = self.page_size * self.row
@@ -258,9 +260,18 @@ class PagedKVWritePlan:
         nnz = self.nnz
         if nnz == 0:
             return
+        fast = self._fast_append
+        if fast is not None:
+            # layouts checked and pointers read in C++; 1 = not a layout it knows: fall through
+            # to the checks below, which name what is wrong (or handle the rare case)
+            rc = fast(self._plan, nnz, self.H, self.D, self.page_size, self._dtype_code,
+                      self._dev_index, append_key, append_value, paged_kv_cache,
+                      self._get_stream(self._dev_index))
+            if rc == 0:
+                return
+            if rc < 0:
+                _lib.check(rc)
         row = self.row
-        # the common case in one pass: contiguous [nnz, H, D] / [nnz, H*D] rows; anything
-        # else goes through the checks that name what is wrong
         k_stride = append_key.stride(0)
         v_stride = append_value.stride(0)
         dt, dev = self.dtype, self.device

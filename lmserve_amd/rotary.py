@@ -243,7 +243,9 @@ class PagedRotaryWritePlan:
             self.page_size, self.kd, ctypes.byref(handle)))
         self._plan = handle.value
         fast = _lib.fast()
-        self._run = fast.rotary_plan_run if fast else lib.kvc_rotary_plan_run
+        self._fast_run = fast.rotary_plan_run if fast else None
+        self._dtype_code = fast.scalar_type_code(cos_sin_cache) if fast else -1
+        self._run = lib.kvc_rotary_plan_run
         self._destroy = lib.kvc_rotary_plan_destroy
         self._cache_shape_tail = torch.Size((2, self.page_size, self.H, self.D))
         self._k_plane = self.page_size * self.kv_row
@@ -285,6 +287,17 @@ class PagedRotaryWritePlan:
             key_out = torch.empty((self.nnz, self.kv_row), dtype=self.dtype, device=self.device)
         if self.nnz == 0:
             return query_out, key_out
+        fast = self._fast_run
+        if fast is not None:
+            # layouts checked and pointers read in C++; 1 = not a layout it knows: fall through
+            # to the checks below, which name what is wrong (or handle the rare case)
+            rc = fast(self._plan, self.nnz, self.Hq, self.H, self.D, self.page_size, self._dtype_code,
+                      self._dev_index, query, key, value, query_out, key_out, paged_kv_cache,
+                      self._get_stream(self._dev_index))
+            if rc == 0:
+                return query_out, key_out
+            if rc < 0:
+                _lib.check(rc)
         dt, dev, nnz = self.dtype, self.device, self.nnz
         if paged_kv_cache.dtype is not dt or paged_kv_cache.device != dev:
             raise TypeError("paged_kv_cache must have the plan's dtype and device")
