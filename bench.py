@@ -37,11 +37,11 @@ PREWARM_S = 0.15     # seconds of untimed launches ahead of every timed region
 ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 
 # HBM bytes per launch of the headline kernel (config 2, all layers in one launch)
-# from two rocprofv3 --pmc runs: FETCH_SIZE 16438.9 KiB x 2.0000 + WRITE_SIZE
-# 32810.8 KiB x 1.0000, the factors being what the same counters read for a
+# from two rocprofv3 --pmc runs: FETCH_SIZE 16410.8 KiB x 2.0000 + WRITE_SIZE
+# 32813.8 KiB x 1.0000, the factors being what the same counters read for a
 # plain elementwise kernel of known size (1 GiB read, 1 GiB written); summary in
 # profiles/hbm_traffic_fetch_size_write_size.txt. Only valid for the default workload.
-MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67264347
+MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67209930
 
 
 def log(*a):
@@ -958,7 +958,9 @@ def main():
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_CFG2_ONE_LAUNCH
                      if (L == 32 and args.pool_blocks == 65536) else None,
-                     "kernel": "write_rows_kernel", "bytes_per_launch": int(bytes_step),
+                     "kernel": "write_planes_kernel<4 planes per lane, slot-mapped, non-temporal stores>, "
+                               "1024 workgroups of 512 lanes",
+                     "bytes_per_launch": int(bytes_step),
                      "us_per_launch": round(ms_event * 1e3, 3),
                      "plain_kernel_of_same_size": same_size,
                      "frac_of_plain_kernel_of_same_size":

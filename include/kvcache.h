@@ -71,12 +71,15 @@ const char* kvc_last_error_string(void);
  *   "write_threads"                   lanes per workgroup in the write kernel (0 = by size, 64, 128, 256)
  *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads
  *   "write_order"                     1 = a token's workgroups are neighbours in the grid
- *   "write_narrow"                    rows under 1 KiB take the kernel whose lanes run over
- *                                     consecutive tokens of one (layer, K|V) plane: 0 = never,
- *                                     1 = for launches of "write_narrow_min_bytes" source bytes
- *                                     and more, 2 = always
- *   "write_narrow_min_bytes"          that size (default 2 MiB)
- *   "write_narrow_vpt"                planes per lane in that kernel (0 = by size, 1, 2, 4, 8)
+ *   "write_planes"                    the plane kernel (lanes of a workgroup run over consecutive
+ *                                     tokens of one (layer, K|V) plane): 0 = never, 1 = by row
+ *                                     width and launch size, 2 = whenever the row shape allows
+ *   "write_planes_vpt"                planes per lane in that kernel (0 = by size, 1, 2, 4, 8)
+ *   "write_planes_threads"            lanes per workgroup in that kernel (0 = by rule, 256, 512, 1024)
+ *   "write_planes_min_bytes"          rows under 1 KiB: source bytes per launch from which it runs
+ *   "write_planes_max_vpr"            widest row it takes, in 16-byte vectors (at most 256)
+ *   "write_pipe"                      1 = a lane waits for each of its loads before issuing the
+ *                                     next, 0 = loads back to back, -1 = by rule
  *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
  *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier
  * Unknown key: KVC_ERR_INVALID_ARG. kvc_reset_tuning puts every knob back to its
@@ -93,7 +96,7 @@ enum {
   KVC_KERNEL_NONE = 0,
   KVC_KERNEL_WRITE_ROWS = 1,        /* token per workgroup                          */
   KVC_KERNEL_COPY_TILES = 2,        /* block copy, gather, scatter, direct swap     */
-  KVC_KERNEL_WRITE_ROWS_NARROW = 3  /* rows under 1 KiB: lanes over tokens of a plane */
+  KVC_KERNEL_WRITE_PLANES = 3       /* lanes over consecutive tokens of one plane   */
 };
 enum {
   KVC_LAUNCH_KERNEL = 0,       /* one of KVC_KERNEL_*                               */

@@ -36,7 +36,7 @@ KVC_SWAP_DIRECT = 1
 KVC_KERNEL_NONE = 0
 KVC_KERNEL_WRITE_ROWS = 1
 KVC_KERNEL_COPY_TILES = 2
-KVC_KERNEL_WRITE_ROWS_NARROW = 3
+KVC_KERNEL_WRITE_PLANES = 3
 KVC_LAUNCH_KERNEL = 0
 KVC_LAUNCH_VEC_BYTES = 1
 KVC_LAUNCH_PER_LANE = 2

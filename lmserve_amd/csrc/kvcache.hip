@@ -1,15 +1,20 @@
 // libkvcache: paged KV-cache data movement for MI355X (gfx950, CDNA4).
 //
-// Three kernels carry the whole path; all are HBM-bound byte movers, so the
+// Four kernels carry the whole path; all are HBM-bound byte movers, so the
 // design is about coalescing and bytes in flight, not arithmetic:
 //
 //   write_rows_kernel   a workgroup owns ONE token and a run of 16-byte vectors
 //                       out of that token's rows (K and V of every layer in
 //                       the launch). The slot lookup is workgroup-uniform, so
 //                       the index chain is resolved once on the scalar unit and
-//                       each lane only streams: VPT loads issued back to back,
-//                       then VPT stores; lanes of a wavefront cover consecutive
-//                       vectors of a row on both sides.
+//                       each lane only streams: VPT loads, then VPT stores;
+//                       lanes of a wavefront cover consecutive vectors of a row
+//                       on both sides. Small launches and launches of many
+//                       resident sets.
+//   write_planes_kernel the lanes of a workgroup run over consecutive tokens of
+//                       one (layer, K|V) plane, 1-8 planes per lane: rows under
+//                       1 KiB, and launches that fit one resident set of lanes
+//                       that way (the decode step of all layers at once).
 //   copy_tiles_kernel   a "tile" is one block of one layer (block_bytes
 //                       contiguous on both sides). A workgroup owns a chunk of
 //                       256 lanes x UNROLL x 16 bytes, issues all its loads
@@ -68,15 +73,15 @@ struct Tuning {
   int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
   int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
-  int write_narrow = 1;     // the plane kernel (lanes of a workgroup run over consecutive tokens of
+  int write_planes = 1;     // the plane kernel (lanes of a workgroup run over consecutive tokens of
                             // one (layer, K|V) plane): 0 = never, 1 = by row width and launch size,
                             // 2 = whenever the row shape allows
-  int write_narrow_min_bytes = 2 << 20;  // rows under 1 KiB: source bytes of a launch from which it runs
-  int write_narrow_max_vpr = 256;        // widest row (in 16-byte vectors) that kernel takes
-  int write_narrow_threads = 0;          // lanes per workgroup of that kernel (256, 512, 1024), 0 = by rule
+  int write_planes_min_bytes = 2 << 20;  // rows under 1 KiB: source bytes of a launch from which it runs
+  int write_planes_max_vpr = 256;        // widest row (in 16-byte vectors) that kernel takes
+  int write_planes_threads = 0;          // lanes per workgroup of that kernel (256, 512, 1024), 0 = by rule
   int write_pipe = -1;                   // 1 = a lane waits for each load before issuing its next,
                                          // 0 = loads back to back, -1 = by rule
-  int write_narrow_vpt = 0; // planes per lane in that kernel (1, 2, 4, 8), 0 = by size
+  int write_planes_vpt = 0; // planes per lane in that kernel (1, 2, 4, 8), 0 = by size
   int direct_max_wgs = 64;  // grid cap of the direct swap kernel: PCIe saturates with a few
                             // dozen workgroups, the rest of the GPU stays free for the model
 };
@@ -99,11 +104,11 @@ Knob* knobs(int* count) {
       {"write_nt", &g_tune.write_nt, 1},
       {"write_order", &g_tune.write_order, 0},
       {"write_threads", &g_tune.write_threads, 0},
-      {"write_narrow", &g_tune.write_narrow, 1},
-      {"write_narrow_vpt", &g_tune.write_narrow_vpt, 0},
-      {"write_narrow_min_bytes", &g_tune.write_narrow_min_bytes, 2 << 20},
-      {"write_narrow_max_vpr", &g_tune.write_narrow_max_vpr, 256},
-      {"write_narrow_threads", &g_tune.write_narrow_threads, 0},
+      {"write_planes", &g_tune.write_planes, 1},
+      {"write_planes_vpt", &g_tune.write_planes_vpt, 0},
+      {"write_planes_min_bytes", &g_tune.write_planes_min_bytes, 2 << 20},
+      {"write_planes_max_vpr", &g_tune.write_planes_max_vpr, 256},
+      {"write_planes_threads", &g_tune.write_planes_threads, 0},
       {"write_pipe", &g_tune.write_pipe, -1},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 64},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
@@ -183,7 +188,7 @@ struct WriteArgs {
   int bs_shift;              // log2(block_size) or -1
   int64_t cache_block_stride, cache_slot_stride, cache_layer_stride;
   int64_t num_cache_blocks;
-  // narrow-row kernel only
+  // plane kernel only
   uint32_t num_planes;        // 2 * num_layers; plane = (layer, K|V)
   uint32_t tokens_per_wg;     // blockDim.x / vecs_per_row
   uint32_t num_token_groups;  // ceil(num_tokens / tokens_per_wg)
@@ -285,18 +290,22 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
   }
 }
 
-// Rows shorter than the 1 KiB a wavefront moves per instruction (one KV head of a
-// tensor-parallel shard: 256-byte rows). With a token per workgroup a wavefront
-// would span several rows of several layers and neither side would be one run.
-// Here the lanes of a workgroup run over consecutive TOKENS of one (layer, K|V)
+// The lanes of a workgroup run over consecutive TOKENS of one (layer, K|V)
 // plane: the source side is one contiguous run of blockDim.x * 16 bytes, the
 // cache side one row per token. Each lane looks up its own token's slot (lanes
 // of one row read the same index words) and reuses it for its VPT planes, whose
-// loads are all issued before the lookup. 16-byte vectors and a power-of-two
-// number of them per row only; blockIdx.x = plane_group * num_token_groups +
-// token_group.
+// loads are issued before the lookup. Two regimes use it:
+//   - rows shorter than the 1 KiB a wavefront moves per instruction (one KV head
+//     of a tensor-parallel shard: 256-byte rows), where a token per workgroup
+//     leaves a wavefront spanning several rows of several layers and neither
+//     side is one run;
+//   - launches that a few planes per lane bring down to one resident set of
+//     lanes (a decode step of every layer at once): no second round of workgroups,
+//     several loads in flight per lane.
+// 16-byte vectors and a power-of-two number of them per row (up to 256) only;
+// blockIdx.x = plane_group * num_token_groups + token_group.
 template <int VPT, bool PAGED, bool NT>
-__global__ __launch_bounds__(1024) void write_rows_narrow_kernel(WriteArgs a) {
+__global__ __launch_bounds__(1024) void write_planes_kernel(WriteArgs a) {
   using V = u32x4;
   const uint32_t pg = blockIdx.x / a.num_token_groups;
   const uint32_t tg = blockIdx.x - pg * a.num_token_groups;
@@ -609,19 +618,19 @@ void launch_write(const WriteArgs& a, int vec, const WriteLaunch& l, hipStream_t
 }
 
 template <int VPT, bool PAGED>
-void launch_narrow_nt(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
+void launch_planes_nt(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
   const dim3 grid(l.grid), block(l.threads);
-  if (l.nt) hipLaunchKernelGGL((write_rows_narrow_kernel<VPT, PAGED, true>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((write_rows_narrow_kernel<VPT, PAGED, false>), grid, block, 0, s, a);
+  if (l.nt) hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, true>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, false>), grid, block, 0, s, a);
 }
 
 template <bool PAGED>
-void launch_narrow(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
+void launch_planes(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
   switch (l.vpt) {
-    case 1: launch_narrow_nt<1, PAGED>(a, l, s); break;
-    case 2: launch_narrow_nt<2, PAGED>(a, l, s); break;
-    case 4: launch_narrow_nt<4, PAGED>(a, l, s); break;
-    default: launch_narrow_nt<8, PAGED>(a, l, s); break;
+    case 1: launch_planes_nt<1, PAGED>(a, l, s); break;
+    case 2: launch_planes_nt<2, PAGED>(a, l, s); break;
+    case 4: launch_planes_nt<4, PAGED>(a, l, s); break;
+    default: launch_planes_nt<8, PAGED>(a, l, s); break;
   }
 }
 
@@ -736,7 +745,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
   // lookup, a chain of dependent loads per lane, has the same effect by itself.
   const int64_t resident_lanes = (int64_t)resident_workgroups() * kThreads;
   const bool plane_rows = vec == 16 && a.vpr_shift >= 0 &&
-                          (int64_t)a.vecs_per_row <= std::min(g_tune.write_narrow_max_vpr, 256);
+                          (int64_t)a.vecs_per_row <= std::min(g_tune.write_planes_max_vpr, 256);
   const int64_t num_planes = 2 * g.num_layers;
   const auto plane_lanes = [&](int v) {  // lanes of the launch at v planes per lane, 256-lane workgroups
     const int64_t tpw = kThreads / (int64_t)a.vecs_per_row;
@@ -748,23 +757,23 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
       if (plane_lanes(v) <= resident_lanes) fit_vpt = v;
   bool plane_pays = false;
   if (plane_rows) {
-    if (g_tune.write_narrow >= 2) plane_pays = true;
+    if (g_tune.write_planes >= 2) plane_pays = true;
     else if (a.vecs_per_row < 64)
-      plane_pays = g.num_tokens * num_planes * g.row_elems * E >= g_tune.write_narrow_min_bytes;
+      plane_pays = g.num_tokens * num_planes * g.row_elems * E >= g_tune.write_planes_min_bytes;
     else plane_pays = fit_vpt > 0 && plane_lanes(1) >= resident_lanes;
   }
-  if (g_tune.write_narrow && plane_pays) {
+  if (g_tune.write_planes && plane_pays) {
     WriteLaunch l{};
-    l.vpt = g_tune.write_narrow_vpt;
+    l.vpt = g_tune.write_planes_vpt;
     if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8)
       l.vpt = fit_vpt ? fit_vpt : 1;  // beyond one set: stream
     // a page-table lookup per lane wants at least two planes to pay for itself
-    if (paged && l.vpt == 1 && g_tune.write_narrow_vpt != 1) l.vpt = 2;
+    if (paged && l.vpt == 1 && g_tune.write_planes_vpt != 1) l.vpt = 2;
     while (l.vpt > 1 && (int64_t)(l.vpt / 2) >= num_planes) l.vpt /= 2;
     // slot-mapped launches of 4 or 8 planes per lane: 512-lane workgroups whose lanes
     // wait for each load (see above); everything else 256 lanes, loads back to back
     const bool deep_slot = !paged && l.vpt >= 4;
-    int wg_lanes = g_tune.write_narrow_threads;
+    int wg_lanes = g_tune.write_planes_threads;
     if (wg_lanes != 256 && wg_lanes != 512 && wg_lanes != 1024) wg_lanes = deep_slot ? 512 : 256;
     a.pipe = g_tune.write_pipe >= 0 ? g_tune.write_pipe : (deep_slot ? 1 : 0);
     const int64_t lanes_all = g.num_tokens * (int64_t)a.vecs_per_row;
@@ -786,14 +795,14 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
       if (paged) {
         a.batch_indices = batch_indices + t0;
         a.positions = positions + t0;
-        launch_narrow<true>(a, l, (hipStream_t)stream);
+        launch_planes<true>(a, l, (hipStream_t)stream);
       } else {
         a.slot_mapping = (const char*)slot_mapping + t0 * slot_bytes;
-        launch_narrow<false>(a, l, (hipStream_t)stream);
+        launch_planes<false>(a, l, (hipStream_t)stream);
       }
       KVC_HIP(hipGetLastError());
     }
-    g_last = LastLaunch{KVC_KERNEL_WRITE_ROWS_NARROW, 16, l.vpt, l.threads, l.grid, l.nt};
+    g_last = LastLaunch{KVC_KERNEL_WRITE_PLANES, 16, l.vpt, l.threads, l.grid, l.nt};
     return KVC_OK;
   }
 

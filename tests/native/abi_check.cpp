@@ -191,8 +191,8 @@ int main() {
     }
     // tuning knobs: set, read back, reset
     int v = -1;
-    KVC_OK_OR_DIE(kvc_set_tuning("write_narrow", 2));
-    KVC_OK_OR_DIE(kvc_get_tuning("write_narrow", &v));
+    KVC_OK_OR_DIE(kvc_set_tuning("write_planes", 2));
+    KVC_OK_OR_DIE(kvc_get_tuning("write_planes", &v));
     if (v != 2 || kvc_tuning_modified() != 1) { std::fprintf(stderr, "tuning read-back failed\n"); ++fails; }
     HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
     for (int64_t l = 0; l < L; ++l)
@@ -203,12 +203,12 @@ int main() {
     HIP_OK(hipStreamSynchronize(stream));
     HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
     expect_equal("plane kernel on 256-byte rows == oracle", got.data(), want.data(), pool_bytes);
-    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_ROWS_NARROW) {
-      std::fprintf(stderr, "write_narrow = 2 did not select the plane kernel\n");
+    if (kvc_last_launch_info(KVC_LAUNCH_KERNEL) != KVC_KERNEL_WRITE_PLANES) {
+      std::fprintf(stderr, "write_planes = 2 did not select the plane kernel\n");
       ++fails;
     }
     KVC_OK_OR_DIE(kvc_reset_tuning());
-    KVC_OK_OR_DIE(kvc_get_tuning("write_narrow", &v));
+    KVC_OK_OR_DIE(kvc_get_tuning("write_planes", &v));
     if (v != 1 || kvc_tuning_modified() != 0) { std::fprintf(stderr, "tuning reset failed\n"); ++fails; }
   }
 

@@ -71,7 +71,7 @@ def test_config2_decode_write_full_pool(gpu):
     # the headline launch: the plane kernel, exactly one resident set of lanes in 512-lane
     # workgroups, 4 planes per lane
     assert (ran["kernel"], ran["vec_bytes"], ran["per_lane"], ran["threads"], ran["grid"]) == \
-        (_lib.KVC_KERNEL_WRITE_ROWS_NARROW, 16, 4, 512, 1024)
+        (_lib.KVC_KERNEL_WRITE_PLANES, 16, 4, 512, 1024)
     assert _check_write(pool, key, value, slots, bs) > 0
     _clear_slots(pool, slots, bs)
     assert int(torch.count_nonzero(pool[L - 1].view(torch.int16))) == 0
@@ -80,7 +80,7 @@ def test_config2_decode_write_full_pool(gpu):
                                      idx.kv_block_indices, idx.kv_block_indptrs, idx.kv_last_block_lens)
     ran = _lib.last_launch()
     assert (ran["kernel"], ran["per_lane"], ran["threads"], ran["grid"]) == \
-        (_lib.KVC_KERNEL_WRITE_ROWS_NARROW, 4, 256, 2048)
+        (_lib.KVC_KERNEL_WRITE_PLANES, 4, 256, 2048)
     _check_write(pool, key, value, slots, bs)
     _clear_slots(pool, slots, bs)
 

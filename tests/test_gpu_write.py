@@ -90,7 +90,7 @@ def test_write_rows_every_launch_shape(gpu, vpt, nt, threads):
     for l in range(L):
         orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
     dpool = to_bf16(pool, gpu)
-    _lib.set_tuning("write_narrow", 0)    # the token kernel, whatever the size
+    _lib.set_tuning("write_planes", 0)    # the token kernel, whatever the size
     _lib.set_tuning("write_vpt", vpt)     # the autouse fixture puts the defaults back
     _lib.set_tuning("write_nt", nt)
     _lib.set_tuning("write_threads", threads)
@@ -139,10 +139,10 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
     for l in range(L):
         orc.c_reshape_and_cache(key[l], value[l], want[l], slots)
     dpool = to_bf16(pool, gpu)
-    _lib.set_tuning("write_narrow_vpt", vpt)
-    _lib.set_tuning("write_narrow", 2)          # whatever the launch size
+    _lib.set_tuning("write_planes_vpt", vpt)
+    _lib.set_tuning("write_planes", 2)          # whatever the launch size
     # workgroup size and load order vary over the cases (both are by rule otherwise)
-    _lib.set_tuning("write_narrow_threads", (0, 256, 512, 1024)[(T + L) % 4])
+    _lib.set_tuning("write_planes_threads", (0, 256, 512, 1024)[(T + L) % 4])
     _lib.set_tuning("write_pipe", (-1, 0, 1)[(T + vpt) % 3])
     if paged:
         # requests of up to three tokens, each token on a page of its own:
@@ -164,14 +164,14 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
                                      torch.from_numpy(slots).to(gpu))
     torch.cuda.synchronize()
     ran = _lib.last_launch()
-    assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_ROWS_NARROW and ran["vec_bytes"] == 16
+    assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_PLANES and ran["vec_bytes"] == 16
     if vpt:
         assert ran["per_lane"] == min(vpt, 1 << (2 * L - 1).bit_length())
     assert np.array_equal(bits_of(dpool), want)
 
 
 def test_narrow_kernel_switch_and_strided_sources(gpu):
-    """`write_narrow = 0` sends narrow rows through the token-per-workgroup kernel,
+    """`write_planes = 0` sends narrow rows through the token-per-workgroup kernel,
     `2` through the plane kernel whatever the size; both agree with the oracle on
     token-strided sources (slices of a wider projection), where the source side
     is no longer one run. By default the launch size decides."""
@@ -187,8 +187,8 @@ def test_narrow_kernel_switch_and_strided_sources(gpu):
     dk = to_bf16(wide_k, gpu)[:, H * D:2 * H * D].view(T, H, D)
     dv = to_bf16(wide_v, gpu)[:, 2 * H * D:].view(T, H, D)
     assert not dk.is_contiguous()
-    for narrow, kernel in ((2, _lib.KVC_KERNEL_WRITE_ROWS_NARROW), (0, _lib.KVC_KERNEL_WRITE_ROWS)):
-        _lib.set_tuning("write_narrow", narrow)
+    for narrow, kernel in ((2, _lib.KVC_KERNEL_WRITE_PLANES), (0, _lib.KVC_KERNEL_WRITE_ROWS)):
+        _lib.set_tuning("write_planes", narrow)
         dpool = to_bf16(pool, gpu)
         kvc.reshape_and_cache(dk, dv, dpool, torch.from_numpy(slots).to(gpu))
         torch.cuda.synchronize()
@@ -209,7 +209,7 @@ def test_narrow_kernel_switch_and_strided_sources(gpu):
     dbig = to_bf16(big_pool, gpu)
     kvc.reshape_and_cache_layers(to_bf16(bk, gpu), to_bf16(bv, gpu), dbig, torch.from_numpy(big_slots).to(gpu))
     torch.cuda.synchronize()
-    assert _lib.last_launch()["kernel"] == _lib.KVC_KERNEL_WRITE_ROWS_NARROW
+    assert _lib.last_launch()["kernel"] == _lib.KVC_KERNEL_WRITE_PLANES
     assert np.array_equal(bits_of(dbig), big_want)
 
 
@@ -449,7 +449,7 @@ def test_dtype_mismatch_raises(gpu):
 
 # token count -> what the launch rule must pick on a 256-CU part for 32 layers of 2 KiB rows:
 # (kernel, planes or vectors per lane, lanes per workgroup) slot-mapped / page-table addressed
-_TOKEN, _PLANE = _lib.KVC_KERNEL_WRITE_ROWS, _lib.KVC_KERNEL_WRITE_ROWS_NARROW
+_TOKEN, _PLANE = _lib.KVC_KERNEL_WRITE_ROWS, _lib.KVC_KERNEL_WRITE_PLANES
 SIZE_RULE = {
     40: ((_TOKEN, 1, 256), (_TOKEN, 1, 256)),      # under one resident set of lanes: token kernel
     64: ((_PLANE, 1, 256), (_PLANE, 2, 256)),      # exactly one set at one plane per lane
