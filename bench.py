@@ -203,18 +203,25 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
 
     plans = {}
 
-    def per_layer_plan(i):
+    def planned(i, resolve):
         r = i % R
         _, k, v, idx = sets[r]
-        plan = plans.get(r)
+        plan = plans.get((r, resolve))
         if plan is None:
             s = sets[r][0].shape
-            plan = plans[r] = kvc.PagedKVWritePlan(
+            plan = plans[(r, resolve)] = kvc.PagedKVWritePlan(
                 idx.batch_indices, idx.positions, idx.kv_block_indices, idx.kv_block_indptrs,
-                idx.kv_last_block_lens, s.num_kv_heads, s.head_dim, s.block_size, k.dtype)
+                idx.kv_last_block_lens, s.num_kv_heads, s.head_dim, s.block_size, k.dtype,
+                resolve_slots=resolve)
         ks, vs = k_l[r], v_l[r]
         for l in range(L):
             plan.append(ks[l], vs[l], pool_l[l])
+
+    def per_layer_plan(i):
+        planned(i, False)
+
+    def per_layer_plan_resolved(i):
+        planned(i, True)
 
     def per_layer_slot(i):
         r = i % R
@@ -231,6 +238,9 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
                             bytes_layer, L),
         "per_layer_plan": (per_layer_plan, f"PagedKVWritePlan.append (per layer, {L} launches per step)",
                            bytes_layer, L),
+        "per_layer_plan_resolved": (per_layer_plan_resolved,
+                                    f"PagedKVWritePlan(resolve_slots).append (per layer, {L} launches per step)",
+                                    bytes_layer, L),
         "per_layer_slot": (per_layer_slot, f"reshape_and_cache (per layer, {L} launches per step)",
                            bytes_layer, L),
     }
@@ -463,9 +473,13 @@ def per_layer_summary(entries):
         ("eager_full_wrapper_us", "cfg2 decode/append_paged_kv_cache (per layer", "eager"),
         ("eager_plan_us", "cfg2 decode/PagedKVWritePlan.append", "eager"),
         ("graph_replay_us", "cfg2 decode/append_paged_kv_cache (per layer", "hipGraph"),
+        ("eager_plan_resolved_slots_us", "cfg2 decode/PagedKVWritePlan(resolve_slots).append", "eager"),
+        ("graph_replay_plan_resolved_slots_us", "cfg2 decode/PagedKVWritePlan(resolve_slots).append", "hipGraph"),
         ("rotation_fused_eager_full_wrapper_us", "cfg2 decode + rotation/rotary_pos_emb_and_append_paged", "eager"),
         ("rotation_fused_eager_plan_us", "cfg2 decode + rotation/PagedRotaryWritePlan.run", "eager"),
         ("rotation_fused_graph_replay_us", "cfg2 decode + rotation/rotary_pos_emb_and_append_paged", "hipGraph"),
+        ("rotation_fused_graph_replay_plan_resolved_slots_us",
+         "cfg2 decode + rotation/PagedRotaryWritePlan(resolve_slots).run", "hipGraph"),
         ("rotation_then_append_graph_replay_us", "cfg2 decode + rotation/rotary_pos_emb + append_paged_kv_cache", "hipGraph"),
     )
     out = {"workload": "configuration 2, one launch per layer (2 MiB of K/V rows per launch)",
@@ -512,7 +526,8 @@ def main():
     variants = ["fused_slot:eager"]
     if "write" in ops:
         variants += ["fused_slot:graph", "fused_paged:eager", "per_layer_paged:graph",
-                     "per_layer_slot:graph", "per_layer_paged:eager", "per_layer_plan:eager"]
+                     "per_layer_slot:graph", "per_layer_paged:eager", "per_layer_plan:eager",
+                     "per_layer_plan_resolved:eager", "per_layer_plan_resolved:graph"]
     entries, res = bench_write_config(torch, kvc, "cfg2 decode", sets, pool, L, args.steps,
                                       args.warmup, variants)
     extra += entries[1:]
@@ -585,6 +600,15 @@ def main():
             for l in range(L):
                 plans[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
 
+        plans_r = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
+                                            ix.kv_block_indptrs, ix.kv_last_block_lens, cs, Hq, Hkv, D,
+                                            s8.block_size, resolve_slots=True) for ix in idxs]
+
+        def fused_plan_resolved(i):
+            r = i % R
+            for l in range(L):
+                plans_r[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
+
         n = max(R, args.steps // 8 // R * R)
         for fn, label in ((fused, "rotary_pos_emb_and_append_paged (1 launch per layer)"),
                           (fused_plan, "PagedRotaryWritePlan.run (1 launch per layer)")):
@@ -593,7 +617,9 @@ def main():
                                calls_per_step=L, launch="eager (Python + ctypes per call)"))
         for fn, label, extra_b in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
                                     2 * T * Hkv * D * E),   # rotated key written out and read back
-                                   (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0)):
+                                   (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0),
+                                   (fused_plan_resolved,
+                                    "PagedRotaryWritePlan(resolve_slots).run (1 launch per layer)", 0)):
             try:
                 ms_w, ms_e = time_region(fn, n, 2, torch, graph_of=R)
             except Exception as exc:

@@ -218,6 +218,16 @@ int kvc_write_plan_append(const kvc_write_plan* plan, const void* append_key,
                           int64_t page_stride, int64_t num_pages, void* stream);
 int kvc_write_plan_destroy(kvc_write_plan* plan);
 
+/* Optional: walk the page table ONCE per step instead of once per layer. One
+ * small launch on `stream` writes every token's slot (page * page_size + entry,
+ * or -1 for a token the page-table write would skip) into `slots`, nnz int64
+ * entries of device memory that the caller owns and keeps valid while the plan
+ * is used. From then on kvc_write_plan_append addresses the cache through these
+ * slots, exactly as kvc_reshape_and_cache would: the per-layer launch loses its
+ * chain of three dependent index loads. The results are identical. Appends must
+ * be ordered after this call (same stream, or an event). */
+int kvc_write_plan_resolve_slots(kvc_write_plan* plan, int64_t* slots, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Index preparation for the paged write.
  * Replace the flashinfer.get_seq_lens / flashinfer.get_batch_indices_positions
@@ -463,6 +473,10 @@ int kvc_rotary_plan_run(const kvc_rotary_plan* plan, const void* query, const vo
                         void* paged_kv_cache, int64_t page_stride, int64_t num_pages,
                         void* stream);
 int kvc_rotary_plan_destroy(kvc_rotary_plan* plan);
+/* As kvc_write_plan_resolve_slots: the page table is walked once per step and
+ * kvc_rotary_plan_run addresses the cache through `slots` (nnz int64 entries of
+ * caller-owned device memory), as kvc_rotary_pos_emb_and_cache would. */
+int kvc_rotary_plan_resolve_slots(kvc_rotary_plan* plan, int64_t* slots, void* stream);
 
 /* The on-device half of a swap on its own: gather scattered pool blocks into a
  * dense device buffer laid out like the host pool, [n, layer_end-layer_begin,

@@ -67,10 +67,12 @@ SIGNATURES = {
                                       ctypes.POINTER(_P)]),
     "kvc_write_plan_append": (c_int, [_P, _P, _P, _I64, _I64, _P, _I64, _I64, _P]),
     "kvc_write_plan_destroy": (c_int, [_P]),
+    "kvc_write_plan_resolve_slots": (c_int, [_P, _P, _P]),
     "kvc_rotary_plan_create": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _I64,
                                        _I64, _I64, c_int, ctypes.POINTER(_P)]),
     "kvc_rotary_plan_run": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P, _I64, _I64, _P]),
     "kvc_rotary_plan_destroy": (c_int, [_P]),
+    "kvc_rotary_plan_resolve_slots": (c_int, [_P, _P, _P]),
     "kvc_swap_prepare": (c_int, [_P, _P, _I64, _I64, _I64, _P, _I64, _P]),
     "kvc_swap_out_prepared": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
                                       _I64, c_int, _P, _P]),

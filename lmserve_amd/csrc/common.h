@@ -27,6 +27,13 @@ struct RopeTuning {
 };
 extern RopeTuning g_rope_tune;
 
+// One launch on `stream`: slots[t] = page * page_size + entry of token t of a
+// page-table write, or -1 where that write would skip the token.
+int launch_resolve_slots(const char* fn, const int32_t* batch_indices, const int32_t* positions,
+                         const int32_t* kv_indices, const int32_t* kv_indptr, int64_t batch_size,
+                         int64_t num_kv_indices, int64_t page_size, int64_t nnz, int64_t* slots,
+                         hipStream_t stream);
+
 // MiB of aligned staging per thread in the disk tier ("disk_bounce_mib").
 extern int g_disk_bounce_mib;
 

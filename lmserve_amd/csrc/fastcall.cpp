@@ -72,6 +72,7 @@ int64_t page_stride(const at::Tensor& c, int64_t page_size, int64_t heads, int64
   if (strides[4] != 1 || strides[3] != dim || strides[2] != row || strides[1] != page_size * row) return -1;
   *num_pages = sizes[0];
   if (sizes[0] < 1) return -1;
+  if (sizes[0] > 1 && strides[0] < 2 * page_size * row) return -1;  // overlapping pages
   return sizes[0] > 1 ? strides[0] : 2 * page_size * row;
 }
 

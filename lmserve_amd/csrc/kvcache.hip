@@ -458,6 +458,28 @@ __global__ void seq_lens_kernel(const int32_t* kv_indptr, const int32_t* last_pa
   seq_lens[b] = pages * page_size + last_page_len[b];
 }
 
+// slot of every token of a page-table write: page * page_size + entry, or -1
+// where the write would skip the token (the rules of the write kernels)
+__global__ void resolve_slots_kernel(const int32_t* batch_indices, const int32_t* positions,
+                                     const int32_t* kv_indices, const int32_t* kv_indptr,
+                                     int64_t batch_size, int64_t num_kv_indices, int64_t page_size,
+                                     int64_t nnz, int64_t* slots) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nnz) return;
+  int64_t slot = -1;
+  const int64_t b = batch_indices[t];
+  const int64_t p = positions[t];
+  if (b >= 0 && b < batch_size && p >= 0) {
+    const int64_t pg = p / page_size;
+    const int64_t it = (int64_t)kv_indptr[b] + pg;
+    if (it >= 0 && it < (int64_t)kv_indptr[b + 1] && it < num_kv_indices) {
+      const int64_t blk = kv_indices[it];
+      if (blk >= 0) slot = blk * page_size + (p - pg * page_size);
+    }
+  }
+  slots[t] = slot;
+}
+
 __global__ void batch_indices_positions_kernel(const int32_t* append_indptr,
                                                const int32_t* seq_lens, int64_t nnz,
                                                int32_t* batch_indices, int32_t* positions) {
@@ -1001,7 +1023,7 @@ int swap_ctx_prepare() {
   KVC_HIP(hipGetDevice(&dev));
   SwapCtx& c = g_swap;
   if (c.device != dev) {
-    if (c.device >= 0) swap_ctx_drop_events(c);
+    swap_ctx_drop_events(c);  // also what an earlier, failed attempt left behind
     c.device = -1;
     hipEvent_t* evs[kSwapEvents];
     c.all_events(evs);
@@ -1332,6 +1354,22 @@ int scratch_of_current_device(int64_t** out) {
 
 }  // namespace
 
+namespace kvc {
+int launch_resolve_slots(const char* fn, const int32_t* batch_indices, const int32_t* positions,
+                         const int32_t* kv_indices, const int32_t* kv_indptr, int64_t batch_size,
+                         int64_t num_kv_indices, int64_t page_size, int64_t nnz, int64_t* slots,
+                         hipStream_t stream) {
+  if (nnz == 0) return KVC_OK;
+  if (!slots) return fail(KVC_ERR_INVALID_ARG, "%s: null slot array", fn);
+  if (nnz > (int64_t(1) << 40)) return fail(KVC_ERR_UNSUPPORTED, "%s: %lld tokens", fn, (long long)nnz);
+  const unsigned grid = (unsigned)((nnz + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(resolve_slots_kernel, dim3(grid), dim3(kThreads), 0, stream, batch_indices,
+                     positions, kv_indices, kv_indptr, batch_size, num_kv_indices, page_size, nnz, slots);
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+}  // namespace kvc
+
 // ===========================================================================
 // C ABI
 // ===========================================================================
@@ -1464,6 +1502,7 @@ struct kvc_write_plan {
   const int32_t* kv_last_page_len;
   int64_t nnz, batch_size, num_kv_indices, num_kv_heads, head_dim, page_size;
   int elem_bytes;
+  const int64_t* slots;  // resolved by kvc_write_plan_resolve_slots, else null
 };
 
 int kvc_write_plan_create(const int32_t* batch_indices, const int32_t* positions,
@@ -1483,7 +1522,7 @@ int kvc_write_plan_create(const int32_t* batch_indices, const int32_t* positions
     return fail(KVC_ERR_UNSUPPORTED, "kvc_write_plan_create: elem_bytes=%d (need 1, 2, 4 or 8)", elem_bytes);
   kvc_write_plan* p = new (std::nothrow) kvc_write_plan{
       batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len, nnz, batch_size,
-      num_kv_indices, num_kv_heads, head_dim, page_size, elem_bytes};
+      num_kv_indices, num_kv_heads, head_dim, page_size, elem_bytes, nullptr};
   if (!p) return fail(KVC_ERR_HIP, "kvc_write_plan_create: out of host memory");
   *out = p;
   return KVC_OK;
@@ -1494,12 +1533,34 @@ int kvc_write_plan_append(const kvc_write_plan* plan, const void* append_key,
                           int64_t value_token_stride, void* paged_kv_cache, int64_t page_stride,
                           int64_t num_pages, void* stream) {
   if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_append: null plan");
+  if (plan->slots) {
+    const int64_t row = plan->num_kv_heads * plan->head_dim;
+    if (page_stride < 2 * plan->page_size * row)
+      return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_append: page_stride %lld < 2*page_size*H*D",
+                  (long long)page_stride);
+    WriteGeom g{plan->nnz, row, key_token_stride, value_token_stride, plan->page_size, page_stride,
+                row, num_pages, 1, 0, 0, 0, plan->elem_bytes};
+    char* vc = paged_kv_cache ? (char*)paged_kv_cache + plan->page_size * row * (int64_t)plan->elem_bytes
+                              : nullptr;
+    return run_write("kvc_write_plan_append", append_key, append_value, paged_kv_cache, vc,
+                     plan->slots, 8, nullptr, nullptr, nullptr, nullptr, 0, 0, g, stream);
+  }
   return kvc_append_paged_kv_cache(append_key, append_value, plan->batch_indices, plan->positions,
                                    paged_kv_cache, plan->kv_indices, plan->kv_indptr,
                                    plan->kv_last_page_len, plan->nnz, plan->batch_size,
                                    plan->num_kv_indices, plan->num_kv_heads, plan->head_dim,
                                    plan->page_size, key_token_stride, value_token_stride,
                                    page_stride, num_pages, plan->elem_bytes, stream);
+}
+
+int kvc_write_plan_resolve_slots(kvc_write_plan* plan, int64_t* slots, void* stream) {
+  if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_resolve_slots: null plan");
+  const int rc = kvc::launch_resolve_slots("kvc_write_plan_resolve_slots", plan->batch_indices,
+                                           plan->positions, plan->kv_indices, plan->kv_indptr,
+                                           plan->batch_size, plan->num_kv_indices, plan->page_size,
+                                           plan->nnz, slots, (hipStream_t)stream);
+  if (rc == KVC_OK && plan->nnz > 0) plan->slots = slots;
+  return rc;
 }
 
 int kvc_write_plan_destroy(kvc_write_plan* plan) {

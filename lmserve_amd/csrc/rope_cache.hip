@@ -558,6 +558,7 @@ struct kvc_rotary_plan {
   int64_t max_position, nnz, num_heads, num_kv_heads, head_dim, rotary_dim;
   int64_t batch_size, num_kv_indices, page_size;
   int dtype;
+  const int64_t* slots;  // resolved by kvc_rotary_plan_resolve_slots, else null
 };
 
 int kvc_rotary_plan_create(const int32_t* batch_indices, const int32_t* positions,
@@ -583,7 +584,7 @@ int kvc_rotary_plan_create(const int32_t* batch_indices, const int32_t* position
     return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_create: null pointer");
   kvc_rotary_plan* p = new (std::nothrow) kvc_rotary_plan{
       batch_indices, positions, cos_sin_cache, kv_indices, kv_indptr, max_position, nnz, num_heads,
-      num_kv_heads, head_dim, rotary_dim, batch_size, num_kv_indices, page_size, dtype};
+      num_kv_heads, head_dim, rotary_dim, batch_size, num_kv_indices, page_size, dtype, nullptr};
   if (!p) return fail(KVC_ERR_HIP, "kvc_rotary_plan_create: out of host memory");
   *out = p;
   return KVC_OK;
@@ -597,12 +598,34 @@ int kvc_rotary_plan_run(const kvc_rotary_plan* plan, const void* query, const vo
   if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_run: null plan");
   const int64_t q_row = plan->num_heads * plan->head_dim;
   const int64_t k_row = plan->num_kv_heads * plan->head_dim;
+  if (plan->slots) {
+    if (page_stride < 2 * plan->page_size * k_row)
+      return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_run: page_stride %lld < 2*page_size*H*D",
+                  (long long)page_stride);
+    const int E = plan->dtype == KVC_DTYPE_F32 ? 4 : 2;
+    char* vc = paged_kv_cache ? (char*)paged_kv_cache + plan->page_size * k_row * E : nullptr;
+    return kvc_rotary_pos_emb_and_cache(
+        query, key, value, plan->positions, 4, plan->cos_sin_cache, plan->max_position, plan->nnz,
+        plan->num_heads, plan->num_kv_heads, plan->head_dim, plan->rotary_dim, q_token_stride,
+        k_token_stride, v_token_stride, query_out, key_out, q_row, k_row, paged_kv_cache, vc,
+        plan->slots, 8, plan->page_size, page_stride, k_row, num_pages, plan->dtype, stream);
+  }
   return kvc_rotary_pos_emb_and_append_paged(
       query, key, value, plan->batch_indices, plan->positions, plan->cos_sin_cache,
       plan->max_position, plan->nnz, plan->num_heads, plan->num_kv_heads, plan->head_dim,
       plan->rotary_dim, q_token_stride, k_token_stride, v_token_stride, query_out, key_out, q_row,
       k_row, paged_kv_cache, plan->kv_indices, plan->kv_indptr, plan->batch_size,
       plan->num_kv_indices, plan->page_size, page_stride, num_pages, plan->dtype, stream);
+}
+
+int kvc_rotary_plan_resolve_slots(kvc_rotary_plan* plan, int64_t* slots, void* stream) {
+  if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_resolve_slots: null plan");
+  const int rc = kvc::launch_resolve_slots("kvc_rotary_plan_resolve_slots", plan->batch_indices,
+                                           plan->positions, plan->kv_indices, plan->kv_indptr,
+                                           plan->batch_size, plan->num_kv_indices, plan->page_size,
+                                           plan->nnz, slots, (hipStream_t)stream);
+  if (rc == KVC_OK && plan->nnz > 0) plan->slots = slots;
+  return rc;
 }
 
 int kvc_rotary_plan_destroy(kvc_rotary_plan* plan) {

@@ -193,13 +193,19 @@ class PagedKVWritePlan:
     `plan.append(key, value, kv_caches[i])` per layer marshals only the layer's
     three pointers, their strides and the stream (`kvc_write_plan_append`).
 
+    With `resolve_slots=True` the page table is walked once, at construction (one
+    small launch on the current stream, `kvc_write_plan_resolve_slots`), and every
+    layer's launch addresses the cache through the resulting slot per token: its
+    chain of three dependent index loads is gone. Same results; the appends must
+    run on that stream or be ordered after it.
+
     The plan keeps references to the index tensors, so their memory stays valid
     for as long as the plan lives.
     """
 
     def __init__(self, batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len,
                  num_kv_heads: int, head_dim: int, page_size: int, dtype: torch.dtype,
-                 kv_layout: str = "NHD"):
+                 kv_layout: str = "NHD", resolve_slots: bool = False):
         (self.batch_indices, self.positions, self.kv_indices, self.kv_indptr,
          self.kv_last_page_len) = _paged_common(None, None, batch_indices, positions, kv_indices,
                                                 kv_indptr, kv_last_page_len, kv_layout)
@@ -217,6 +223,12 @@ class PagedKVWritePlan:
             self.kv_indptr.numel() - 1, self.kv_indices.numel(), self.H, self.D, self.page_size,
             self.elem, ctypes.byref(handle)))
         self._plan = handle.value
+        self.slots = None
+        if resolve_slots and self.nnz:
+            self.slots = torch.empty(self.nnz, dtype=torch.int64, device=self.device)
+            with _on_device_of(self.batch_indices):
+                _lib.check(lib.kvc_write_plan_resolve_slots(self._plan, self.slots.data_ptr(),
+                                                            _stream_of(self.batch_indices)))
         fast = _lib.fast()
         self._fast_append = fast.write_plan_append if fast else None
         self._dtype_code = fast.scalar_type_code(torch.empty(0, dtype=dtype)) if fast else -1

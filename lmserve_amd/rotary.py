@@ -209,12 +209,16 @@ class PagedRotaryWritePlan:
     reads and the library call; `query_out` / `key_out` may be caller-owned
     buffers reused across layers, so that nothing is allocated either.
 
+    `resolve_slots=True` walks the page table once, at construction (one small
+    launch on the current stream); the per-layer launches then read one slot per
+    token. Same results; the runs must be ordered after the construction.
+
     The plan keeps references to its tensors for as long as it lives.
     """
 
     def __init__(self, batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len,
                  cos_sin_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                 page_size: int):
+                 page_size: int, resolve_slots: bool = False):
         for t, n in ((batch_indices, "batch_indices"), (positions, "positions"),
                      (kv_indices, "kv_indices"), (kv_indptr, "kv_indptr"),
                      (kv_last_page_len, "kv_last_page_len")):
@@ -242,6 +246,14 @@ class PagedRotaryWritePlan:
             kv_indices.data_ptr(), kv_indptr.data_ptr(), kv_indptr.numel() - 1, kv_indices.numel(),
             self.page_size, self.kd, ctypes.byref(handle)))
         self._plan = handle.value
+        self.slots = None
+        if resolve_slots and self.nnz:
+            # the page table is walked once, here; every layer's launch reads one slot per token
+            self.slots = torch.empty(self.nnz, dtype=torch.int64, device=self.device)
+            with torch.cuda.device(self.device):
+                _lib.check(lib.kvc_rotary_plan_resolve_slots(
+                    self._plan, self.slots.data_ptr(),
+                    torch._C._cuda_getCurrentRawStream(self.device.index)))
         fast = _lib.fast()
         self._fast_run = fast.rotary_plan_run if fast else None
         self._dtype_code = fast.scalar_type_code(cos_sin_cache) if fast else -1

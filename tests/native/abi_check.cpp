@@ -164,6 +164,25 @@ int main() {
       std::fprintf(stderr, "a small launch of 256-byte rows did not take the token-per-workgroup kernel\n");
       ++fails;
     }
+    // the same plan with the page table walked once: slots == the scheduler's rule, same pool
+    int64_t* d_resolved = nullptr;  // the plan uses it until it is destroyed
+    {
+      HIP_OK(hipMalloc(&d_resolved, T * sizeof(int64_t)));
+      HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+      KVC_OK_OR_DIE(kvc_write_plan_resolve_slots(plan, d_resolved, stream));
+      for (int64_t l = 0; l < L; ++l)
+        KVC_OK_OR_DIE(kvc_write_plan_append(plan, (char*)d_key + l * T * row * E,
+                                            (char*)d_value + l * T * row * E, row, row,
+                                            (char*)d_pool + l * layer_elems * E, blk_elems, nb, stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      std::vector<int64_t> resolved(T);
+      HIP_OK(hipMemcpy(resolved.data(), d_resolved, T * sizeof(int64_t), hipMemcpyDeviceToHost));
+      expect_equal("kvc_write_plan_resolve_slots == slot rule", resolved.data(), slots.data(),
+                   T * sizeof(int64_t));
+      HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+      expect_equal("kvc_write_plan_append through resolved slots == oracle", got.data(), want_paged.data(),
+                   pool_bytes);
+    }
     // host cost of one planned launch (informational)
     hipEvent_t e0, e1;
     HIP_OK(hipEventCreate(&e0));
@@ -184,6 +203,7 @@ int main() {
     HIP_OK(hipEventDestroy(e0));
     HIP_OK(hipEventDestroy(e1));
     KVC_OK_OR_DIE(kvc_write_plan_destroy(plan));
+    HIP_OK(hipFree(d_resolved));
     if (kvc_write_plan_append(nullptr, d_key, d_value, row, row, d_pool, blk_elems, nb, stream) !=
         KVC_ERR_INVALID_ARG) {
       std::fprintf(stderr, "expected KVC_ERR_INVALID_ARG for a null plan\n");

@@ -180,6 +180,8 @@ def test_plans_and_prepared_swap_validate_before_touching_the_gpu():
     assert L.kvc_write_plan_append(h, None, 1, 1024, 1024, 1, 32768, 4, None) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_write_plan_append(h, 1, 1, 512, 1024, 1, 32768, 4, None) == _lib.KVC_ERR_INVALID_ARG
     assert "stride" in _lib.last_error()
+    assert L.kvc_write_plan_resolve_slots(h, None, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_write_plan_resolve_slots(None, 1, None) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_write_plan_destroy(h) == _lib.KVC_OK
     assert L.kvc_write_plan_destroy(None) == _lib.KVC_OK
     assert create(1, 1, 1, 1, 1, 4, 2, 8, 8, 128, 0, 2, ctypes.byref(h)) == _lib.KVC_ERR_INVALID_ARG
@@ -194,6 +196,8 @@ def test_plans_and_prepared_swap_validate_before_touching_the_gpu():
     assert rcreate(1, 1, 1, 100, 4, 8, 2, 64, 64, 1, 1, 2, 8, 16, 0, ctypes.byref(h)) == _lib.KVC_OK
     assert L.kvc_rotary_plan_run(h, None, 1, 1, 512, 128, 128, 1, None, 1, 4096, 4, None) == \
         _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_rotary_plan_resolve_slots(h, None, None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_rotary_plan_resolve_slots(None, 1, None) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_rotary_plan_destroy(h) == _lib.KVC_OK
     assert rcreate(1, 1, 1, 100, 4, 8, 2, 64, 63, 1, 1, 2, 8, 16, 0, ctypes.byref(h)) == _lib.KVC_ERR_INVALID_ARG
     assert rcreate(1, 1, 1, 100, 4, 8, 2, 64, 64, 1, 1, 2, 8, 16, 9, ctypes.byref(h)) == _lib.KVC_ERR_UNSUPPORTED

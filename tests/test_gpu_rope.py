@@ -177,6 +177,11 @@ def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
     plan = kvc.PagedRotaryWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices,
                                     idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D,
                                     s.block_size)
+    plan_r = kvc.PagedRotaryWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices,
+                                      idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D,
+                                      s.block_size, resolve_slots=True)   # page table walked once
+    torch.cuda.synchronize()
+    assert np.array_equal(plan_r.slots.cpu().numpy(), w.index.slot_mapping)
     q_buf = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=gpu)
     k_buf = torch.empty(T, Hkv * D, dtype=torch.bfloat16, device=gpu)
     g = torch.Generator().manual_seed(23)
@@ -196,6 +201,11 @@ def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
         q_c, k_c = plan.run(q, k, v, pool_b)                           # allocates q_out, no key_out
         torch.cuda.synchronize()
         assert k_c is None and torch.equal(q_c, q_b)
+        pool_r = torch.zeros_like(pool_a)
+        q_r, k_r = plan_r.run(q, k, v, pool_r, key_out=torch.empty_like(k_buf))
+        torch.cuda.synchronize()
+        assert torch.equal(q_r, q_b) and torch.equal(k_r, k_b), layer
+        assert torch.equal(pool_a.view(torch.int16), pool_r.view(torch.int16)), layer
     with pytest.raises(TypeError):
         plan.run(q.float(), k, v, pool_b)
     with pytest.raises(ValueError):

@@ -323,11 +323,21 @@ def test_append_paged_kv_cache_matches_oracle(gpu, kind):
                                 s.head_dim, s.block_size, torch.bfloat16)
     for l in range(L):
         plan.append(dkey[l], dval[l], planned[l])
+    # the same plan with the page table walked once: slots against the scheduler's rule,
+    # then the per-layer launches through them
+    resolved = to_bf16(pool, gpu)
+    plan_r = kvc.PagedKVWritePlan(dev.batch_indices, dev.positions, dev.kv_block_indices,
+                                  dev.kv_block_indptrs, dev.kv_last_block_lens, s.num_kv_heads,
+                                  s.head_dim, s.block_size, torch.bfloat16, resolve_slots=True)
+    for l in range(L):
+        plan_r.append(dkey[l], dval[l], resolved[l])
     torch.cuda.synchronize()
+    assert np.array_equal(plan_r.slots.cpu().numpy(), w.index.slot_mapping)
     assert np.array_equal(bits_of(per_layer), want)
     assert np.array_equal(bits_of(fused), want)
     assert np.array_equal(bits_of(slotted), want)
     assert np.array_equal(bits_of(planned), want)
+    assert np.array_equal(bits_of(resolved), want)
     with pytest.raises(TypeError):
         plan.append(dkey[0].float(), dval[0], planned[0])
     with pytest.raises(ValueError):
@@ -410,6 +420,45 @@ def test_append_paged_skips_tokens_with_bad_indices(gpu):
                               up(idx.kv_last_block_lens))
     torch.cuda.synchronize()
     assert np.array_equal(bits_of(dpool), want)
+    # a plan with resolved slots skips the same tokens (their slot is -1) ...
+    neg = idx.kv_block_indices.copy()
+    plan = kvc.PagedKVWritePlan(up(bi), up(pos), up(neg), up(idx.kv_block_indptrs),
+                                up(idx.kv_last_block_lens), H, D, bs, torch.bfloat16,
+                                resolve_slots=True)
+    dpool2 = to_bf16(pool, gpu)
+    plan.append(to_bf16(key, gpu), to_bf16(value, gpu), dpool2)
+    torch.cuda.synchronize()
+    slots = plan.slots.cpu().numpy()
+    assert (slots[[2, 4, 5, 6]] == -1).all() and (slots[keep] >= 0).all()
+    assert np.array_equal(bits_of(dpool2), want)
+    # ... and a negative page id or a page beyond the layer's pool is skipped too
+    first = int(idx.kv_block_indptrs[bi[0]]) + int(pos[0]) // bs
+    neg[first] = -3
+    plan = kvc.PagedKVWritePlan(up(bi), up(pos), up(neg), up(idx.kv_block_indptrs),
+                                up(idx.kv_last_block_lens), H, D, bs, torch.bfloat16,
+                                resolve_slots=True)
+    want3 = pool.copy()
+    orc.c_append_paged_kv_cache(np.ascontiguousarray(key[keep[1:]]), np.ascontiguousarray(value[keep[1:]]),
+                                bi[keep[1:]], pos[keep[1:]], want3, idx.kv_block_indices,
+                                idx.kv_block_indptrs)
+    dpool3 = to_bf16(pool, gpu)
+    plan.append(to_bf16(key, gpu), to_bf16(value, gpu), dpool3)
+    torch.cuda.synchronize()
+    assert plan.slots.cpu().numpy()[0] == -1
+    assert np.array_equal(bits_of(dpool3), want3)
+    half = to_bf16(pool, gpu)[:nb // 2]
+    want4 = pool[:nb // 2].copy()
+    small = kvc.PagedKVWritePlan(up(idx.batch_indices), up(idx.positions), up(idx.kv_block_indices),
+                                 up(idx.kv_block_indptrs), up(idx.kv_last_block_lens), H, D, bs,
+                                 torch.bfloat16, resolve_slots=True)
+    small.append(to_bf16(key, gpu), to_bf16(value, gpu), half)
+    torch.cuda.synchronize()
+    pages = idx.slot_mapping // bs
+    inside = np.flatnonzero(pages < nb // 2)
+    assert 0 < len(inside) < T
+    orc.reshape_and_cache_np(np.ascontiguousarray(key[inside]), np.ascontiguousarray(value[inside]),
+                             want4, idx.slot_mapping[inside])
+    assert np.array_equal(bits_of(half), want4)
 
 
 def test_write_runs_on_the_current_stream(gpu):
