@@ -104,7 +104,8 @@ enum {
   KVC_LAUNCH_PER_LANE = 2,     /* vectors (or planes) in flight per lane            */
   KVC_LAUNCH_THREADS = 3,      /* lanes per workgroup                               */
   KVC_LAUNCH_GRID = 4,         /* workgroups                                        */
-  KVC_LAUNCH_NON_TEMPORAL = 5  /* bit 0 stores, bit 1 loads (tile kernel: both = 1) */
+  KVC_LAUNCH_NON_TEMPORAL = 5, /* bit 0 stores, bit 1 loads (tile kernel: both = 1) */
+  KVC_LAUNCH_PIPE = 6          /* write kernels: 1 = a lane waits for each of its loads */
 };
 int64_t kvc_last_launch_info(int what);
 

@@ -43,6 +43,7 @@ KVC_LAUNCH_PER_LANE = 2
 KVC_LAUNCH_THREADS = 3
 KVC_LAUNCH_GRID = 4
 KVC_LAUNCH_NON_TEMPORAL = 5
+KVC_LAUNCH_PIPE = 6
 
 KVC_ABI_VERSION = 2
 KVC_NOALLOC_MAX_BLOCKS = 8192
@@ -212,4 +213,5 @@ def last_launch() -> dict:
             "per_lane": L.kvc_last_launch_info(KVC_LAUNCH_PER_LANE),
             "threads": L.kvc_last_launch_info(KVC_LAUNCH_THREADS),
             "grid": L.kvc_last_launch_info(KVC_LAUNCH_GRID),
-            "non_temporal": L.kvc_last_launch_info(KVC_LAUNCH_NON_TEMPORAL)}
+            "non_temporal": L.kvc_last_launch_info(KVC_LAUNCH_NON_TEMPORAL),
+            "pipe": L.kvc_last_launch_info(KVC_LAUNCH_PIPE)}

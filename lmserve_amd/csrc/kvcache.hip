@@ -76,7 +76,7 @@ struct Tuning {
   int write_planes = 1;     // the plane kernel (lanes of a workgroup run over consecutive tokens of
                             // one (layer, K|V) plane): 0 = never, 1 = by row width and launch size,
                             // 2 = whenever the row shape allows
-  int write_planes_min_bytes = 2 << 20;  // rows under 1 KiB: source bytes of a launch from which it runs
+  int write_planes_min_bytes = 256 << 10;  // rows under 1 KiB: source bytes of a launch from which it runs
   int write_planes_max_vpr = 256;        // widest row (in 16-byte vectors) that kernel takes
   int write_planes_threads = 0;          // lanes per workgroup of that kernel (256, 512, 1024), 0 = by rule
   int write_pipe = -1;                   // 1 = a lane waits for each load before issuing its next,
@@ -106,7 +106,7 @@ Knob* knobs(int* count) {
       {"write_threads", &g_tune.write_threads, 0},
       {"write_planes", &g_tune.write_planes, 1},
       {"write_planes_vpt", &g_tune.write_planes_vpt, 0},
-      {"write_planes_min_bytes", &g_tune.write_planes_min_bytes, 2 << 20},
+      {"write_planes_min_bytes", &g_tune.write_planes_min_bytes, 256 << 10},
       {"write_planes_max_vpr", &g_tune.write_planes_max_vpr, 256},
       {"write_planes_threads", &g_tune.write_planes_threads, 0},
       {"write_pipe", &g_tune.write_pipe, -1},
@@ -127,7 +127,7 @@ Knob* find_knob(const char* key) {
 
 // What the most recent kernel launch of this thread looked like (kvc_last_launch_info).
 struct LastLaunch {
-  int64_t kernel = KVC_KERNEL_NONE, vec = 0, per_lane = 0, threads = 0, grid = 0, nt = 0;
+  int64_t kernel = KVC_KERNEL_NONE, vec = 0, per_lane = 0, threads = 0, grid = 0, nt = 0, pipe = 0;
 };
 thread_local LastLaunch g_last;
 
@@ -746,25 +746,36 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
   a.items_per_token = (uint32_t)items64;
 
   // The plane kernel (lanes over consecutive tokens of one (layer, K|V) plane)
-  // takes rows of a power-of-two number of 16-byte vectors up to 4 KiB. From
-  // sweeps on MI355X (rows of 256 B to 2 KiB, 5 MiB to 512 MiB per launch):
-  //   - rows under 1 KiB: from about 2 MiB of source rows per launch; below that a
-  //     launch is latency-bound and many small token-per-workgroup workgroups with
-  //     a scalar slot lookup finish first (one layer of a 2048-token chunk at
-  //     256-byte rows: 2.53 against 2.80 us; 80 layers of a 64-token step: 4.04
-  //     against 3.67 us);
-  //   - wider rows: when the launch is at least one resident set of lanes at one
-  //     vector per lane and 2, 4 or 8 planes per lane bring it down to one resident
-  //     set (2048 lanes per CU); then no second round of workgroups is dispatched
-  //     and every lane has several loads in flight (Llama-3-8B decode step, 64 MiB:
-  //     12.3-12.5 us against 13.0-13.6 for the token kernel; 128 MiB: 24.8 against
-  //     26.1). Larger launches stream best through the token kernel.
-  // In the one-resident-set regime every lane of the GPU is resident at once;
-  // if all of them issue all their loads and then all their stores, the launch
-  // splits into a read phase and a write phase and loses 15 % (14.4 against
-  // 12.4 us). A lane that waits for each load before issuing the next drifts
-  // apart from its neighbours and the two directions overlap; the page-table
-  // lookup, a chain of dependent loads per lane, has the same effect by itself.
+  // takes rows of a power-of-two number of 16-byte vectors up to 4 KiB. The rule
+  // below comes from sweeps on MI355X over rows of 256 B to 2 KiB, one layer and
+  // all layers per launch, 1 MiB to 256 MiB moved, sources rotating through
+  // 512 MiB (nothing cached) and through two sets (everything cached). It is
+  // written in terms of fill(v): the lanes of the launch at v planes per lane
+  // over the lanes the GPU holds at once (2048 per CU).
+  //   - Small launches are latency-bound and go to the token kernel (many small
+  //     workgroups, scalar slot lookup): wide rows below half a resident set at
+  //     one plane per lane (a quarter for page-table launches, whose lookup the
+  //     plane kernel amortises over two planes), rows under 1 KiB below 256 KiB
+  //     of source rows (a token per workgroup leaves their wavefronts spanning
+  //     several rows of several layers, which costs 10-30 % from 1 MiB on).
+  //   - The fewest planes per lane (at most 4; 2 for rows under 1 KiB) that leave
+  //     the GPU at most half full run as they are: 256-lane workgroups, loads
+  //     back to back.
+  //   - Otherwise the fewest planes per lane that fit one resident set: no second
+  //     round of workgroups. There every lane of the GPU is resident at once; if
+  //     all of them issue all their loads and then all their stores, the launch
+  //     splits into a read phase and a write phase and loses 15-20 % (64 MiB
+  //     decode step: 14.4 against 12.2 us; 32 MiB: 8.5 against 7.1). A lane that
+  //     waits for each load before issuing the next drifts apart from its
+  //     neighbours and the two directions overlap: slot-mapped launches do that
+  //     (from 4 planes per lane in 512-lane workgroups; at 2 planes per lane only
+  //     when the GPU is more than three quarters full). The page-table lookup, a
+  //     chain of dependent loads per lane, has the same effect by itself.
+  //   - Launches beyond one resident set at 8 planes per lane stream best through
+  //     the token kernel, with two exceptions: rows under 1 KiB (see above), and
+  //     page-table launches of so few planes that every token-kernel workgroup
+  //     would walk a cold index chain for 4 KiB of work (one layer of a long
+  //     prefill chunk: 15.5 against 17.9 us at 64 MiB).
   const int64_t resident_lanes = (int64_t)resident_workgroups() * kThreads;
   const bool plane_rows = vec == 16 && a.vpr_shift >= 0 &&
                           (int64_t)a.vecs_per_row <= std::min(g_tune.write_planes_max_vpr, 256);
@@ -773,31 +784,39 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     const int64_t tpw = kThreads / (int64_t)a.vecs_per_row;
     return (g.num_tokens + tpw - 1) / tpw * ((num_planes + v - 1) / v) * kThreads;
   };
-  int fit_vpt = 0;  // fewest planes per lane that bring the launch within one resident set
-  if (plane_rows)
-    for (int v = 1; v <= 8 && !fit_vpt; v *= 2)
-      if (plane_lanes(v) <= resident_lanes) fit_vpt = v;
-  bool plane_pays = false;
+  const bool narrow = a.vecs_per_row < 64;
+  int rule_vpt = 0, rule_pipe = 0, rule_lanes = kThreads;  // rule_vpt 0 = token kernel
   if (plane_rows) {
-    if (g_tune.write_planes >= 2) plane_pays = true;
-    else if (a.vecs_per_row < 64)
-      plane_pays = g.num_tokens * num_planes * g.row_elems * E >= g_tune.write_planes_min_bytes;
-    else plane_pays = fit_vpt > 0 && plane_lanes(1) >= resident_lanes;
+    bool pays;
+    if (narrow) pays = g.num_tokens * num_planes * g.row_elems * E >= g_tune.write_planes_min_bytes;
+    else pays = plane_lanes(1) * (paged ? 4 : 2) >= resident_lanes;
+    if (pays) {
+      const int v_first = paged ? 2 : 1;  // a lookup per lane wants two planes to pay for itself
+      const int v_last = (int)std::min<int64_t>(8, num_planes);
+      for (int v = v_first; v <= std::min(v_last, narrow ? 2 : 4) && !rule_vpt; v *= 2)
+        if (2 * plane_lanes(v) <= resident_lanes) rule_vpt = v;
+      for (int v = v_first; v <= v_last && !rule_vpt; v *= 2)
+        if (plane_lanes(v) <= resident_lanes) {
+          rule_vpt = v;
+          if (!paged && v >= 4) { rule_pipe = 1; rule_lanes = 512; }
+          else if (!paged && v == 2 && 4 * plane_lanes(v) > 3 * resident_lanes) rule_pipe = 1;
+        }
+      if (!rule_vpt) {  // beyond one resident set
+        if (narrow) rule_vpt = v_first;
+        else if (paged && num_planes * (int64_t)a.vecs_per_row <= 2 * kThreads) rule_vpt = 2;
+      }
+    }
+    if (g_tune.write_planes >= 2 && !rule_vpt) rule_vpt = paged ? 2 : 1;  // forced
   }
-  if (g_tune.write_planes && plane_pays) {
+  if (g_tune.write_planes && rule_vpt) {
     WriteLaunch l{};
     l.vpt = g_tune.write_planes_vpt;
-    if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8)
-      l.vpt = fit_vpt ? fit_vpt : 1;  // beyond one set: stream
-    // a page-table lookup per lane wants at least two planes to pay for itself
-    if (paged && l.vpt == 1 && g_tune.write_planes_vpt != 1) l.vpt = 2;
+    if (l.vpt != 1 && l.vpt != 2 && l.vpt != 4 && l.vpt != 8) l.vpt = rule_vpt;
+    else if (l.vpt != rule_vpt) { rule_pipe = (!paged && l.vpt >= 4) ? 1 : 0; rule_lanes = rule_pipe ? 512 : kThreads; }
     while (l.vpt > 1 && (int64_t)(l.vpt / 2) >= num_planes) l.vpt /= 2;
-    // slot-mapped launches of 4 or 8 planes per lane: 512-lane workgroups whose lanes
-    // wait for each load (see above); everything else 256 lanes, loads back to back
-    const bool deep_slot = !paged && l.vpt >= 4;
     int wg_lanes = g_tune.write_planes_threads;
-    if (wg_lanes != 256 && wg_lanes != 512 && wg_lanes != 1024) wg_lanes = deep_slot ? 512 : 256;
-    a.pipe = g_tune.write_pipe >= 0 ? g_tune.write_pipe : (deep_slot ? 1 : 0);
+    if (wg_lanes != 256 && wg_lanes != 512 && wg_lanes != 1024) wg_lanes = rule_lanes;
+    a.pipe = g_tune.write_pipe >= 0 ? g_tune.write_pipe : rule_pipe;
     const int64_t lanes_all = g.num_tokens * (int64_t)a.vecs_per_row;
     l.threads = (unsigned)std::min<int64_t>(wg_lanes, (lanes_all + 63) / 64 * 64);
     if (l.threads < a.vecs_per_row) l.threads = a.vecs_per_row;  // a row never splits over workgroups
@@ -824,7 +843,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
       }
       KVC_HIP(hipGetLastError());
     }
-    g_last = LastLaunch{KVC_KERNEL_WRITE_PLANES, 16, l.vpt, l.threads, l.grid, l.nt};
+    g_last = LastLaunch{KVC_KERNEL_WRITE_PLANES, 16, l.vpt, l.threads, l.grid, l.nt, a.pipe};
     return KVC_OK;
   }
 
@@ -888,7 +907,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     }
     KVC_HIP(hipGetLastError());
   }
-  g_last = LastLaunch{KVC_KERNEL_WRITE_ROWS, vec, l.vpt, l.threads, l.grid, (l.nt ? 1 : 0) | (l.ntl ? 2 : 0)};
+  g_last = LastLaunch{KVC_KERNEL_WRITE_ROWS, vec, l.vpt, l.threads, l.grid, (l.nt ? 1 : 0) | (l.ntl ? 2 : 0), a.pipe};
   return KVC_OK;
 }
 
@@ -1419,6 +1438,7 @@ int64_t kvc_last_launch_info(int what) {
     case KVC_LAUNCH_THREADS: return g_last.threads;
     case KVC_LAUNCH_GRID: return g_last.grid;
     case KVC_LAUNCH_NON_TEMPORAL: return g_last.nt;
+    case KVC_LAUNCH_PIPE: return g_last.pipe;
     default: return KVC_ERR_INVALID_ARG;
   }
 }

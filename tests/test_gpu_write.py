@@ -497,17 +497,21 @@ def test_dtype_mismatch_raises(gpu):
 
 
 # token count -> what the launch rule must pick on a 256-CU part for 32 layers of 2 KiB rows:
-# (kernel, planes or vectors per lane, lanes per workgroup) slot-mapped / page-table addressed
+# (kernel, planes or vectors per lane, lanes per workgroup, lanes wait per load) slot-mapped /
+# page-table addressed. fill = lanes of the launch / lanes the GPU holds at once.
 _TOKEN, _PLANE = _lib.KVC_KERNEL_WRITE_ROWS, _lib.KVC_KERNEL_WRITE_PLANES
 SIZE_RULE = {
-    40: ((_TOKEN, 1, 256), (_TOKEN, 1, 256)),      # under one resident set of lanes: token kernel
-    64: ((_PLANE, 1, 256), (_PLANE, 2, 256)),      # exactly one set at one plane per lane
-    100: ((_PLANE, 2, 256), (_PLANE, 2, 256)),
-    128: ((_PLANE, 2, 256), (_PLANE, 2, 256)),
-    200: ((_PLANE, 4, 512), (_PLANE, 4, 256)),     # deep slot-mapped lanes: 512-lane workgroups
-    256: ((_PLANE, 4, 512), (_PLANE, 4, 256)),     # the decode step of the benchmark
-    300: ((_PLANE, 8, 512), (_PLANE, 8, 256)),
-    600: ((_TOKEN, 1, 256), (_TOKEN, 1, 256)),     # no depth fits one set: stream through the token kernel
+    12: ((_TOKEN, 1, 256, 0), (_TOKEN, 1, 256, 0)),     # latency-bound: token kernel
+    16: ((_TOKEN, 1, 256, 0), (_PLANE, 2, 256, 0)),     # fill 1/4 at one plane per lane: page-table launches switch
+    32: ((_PLANE, 1, 256, 0), (_PLANE, 2, 256, 0)),     # fill 1/2: slot-mapped launches switch
+    40: ((_PLANE, 2, 256, 0), (_PLANE, 2, 256, 0)),     # fewest planes per lane that leave the GPU half full
+    64: ((_PLANE, 2, 256, 0), (_PLANE, 2, 256, 0)),
+    100: ((_PLANE, 4, 256, 0), (_PLANE, 4, 256, 0)),
+    128: ((_PLANE, 4, 256, 0), (_PLANE, 4, 256, 0)),
+    200: ((_PLANE, 4, 512, 1), (_PLANE, 4, 256, 0)),    # over half full at 4: one resident set, lanes wait per load
+    256: ((_PLANE, 4, 512, 1), (_PLANE, 4, 256, 0)),    # the decode step of the benchmark
+    300: ((_PLANE, 8, 512, 1), (_PLANE, 8, 256, 0)),
+    600: ((_TOKEN, 1, 256, 0), (_TOKEN, 1, 256, 0)),    # no depth fits one set: stream through the token kernel
 }
 
 
@@ -515,10 +519,10 @@ SIZE_RULE = {
 @pytest.mark.parametrize("paged", [False, True])
 def test_one_launch_write_through_every_shape_the_size_rule_picks(gpu, T, paged):
     """32 layers of the Llama-3-8B row in one launch, at token counts on both sides
-    of each switch of the launch-shape rule (token kernel below one resident set of
-    lanes; plane kernel with 1, 2, 4 or 8 planes per lane while that brings the
-    launch within one set; token kernel again beyond), slot-mapped and page-table
-    addressed; the shape that ran is asserted as well as the bits."""
+    of each switch of the launch-shape rule (token kernel for latency-bound
+    launches; plane kernel with the fewest planes per lane that leave the GPU half
+    full, else that fit one resident set; token kernel again beyond), slot-mapped
+    and page-table addressed; the shape that ran is asserted as well as the bits."""
     s = wl.LLAMA_3_8B
     L, nb, bs = 32, 96, s.block_size
     w = wl.decode_step(s, num_blocks=nb, batch=T, max_context=4, seed=T) if T <= nb else \
@@ -542,5 +546,50 @@ def test_one_launch_write_through_every_shape_the_size_rule_picks(gpu, T, paged)
     torch.cuda.synchronize()
     ran = _lib.last_launch()
     assert _lib.lib().kvc_tuning_modified() == 0
-    assert (ran["kernel"], ran["per_lane"], ran["threads"]) == SIZE_RULE[T][1 if paged else 0]
+    assert (ran["kernel"], ran["per_lane"], ran["threads"], ran["pipe"]) == SIZE_RULE[T][1 if paged else 0]
+    assert np.array_equal(bits_of(dpool), want)
+
+
+# (shape, layers, tokens) -> launch slot-mapped / page-table addressed, for the corners of the
+# rule that 32 layers of wide rows do not reach
+_S8 = wl.LLAMA_3_1_70B.shard(8)          # one KV head: 256-byte rows
+RULE_CORNERS = {
+    "one layer, 1 KiB rows, one resident set at 2 planes per lane":
+        (wl.QWEN_2_5_7B, 1, 8192, (_PLANE, 2, 256, 1), (_PLANE, 2, 256, 0)),
+    "one layer, 1 KiB rows, beyond one set: few planes keep page-table launches on the plane kernel":
+        (wl.QWEN_2_5_7B, 1, 12288, (_TOKEN, 1, 128, 0), (_PLANE, 2, 256, 0)),
+    "256-byte rows, 160 KiB of source rows": (_S8, 80, 4, (_TOKEN, 1, 256, 0), (_TOKEN, 1, 256, 0)),
+    "256-byte rows, 320 KiB of source rows": (_S8, 80, 8, (_PLANE, 1, 128, 0), (_PLANE, 2, 128, 0)),
+    "256-byte rows, over half full at 1 plane per lane": (_S8, 80, 160, (_PLANE, 2, 256, 0), (_PLANE, 2, 256, 0)),
+    "256-byte rows, beyond one set": (_S8, 80, 2048, (_PLANE, 1, 256, 0), (_PLANE, 2, 256, 0)),
+}
+
+
+@pytest.mark.parametrize("case", sorted(RULE_CORNERS))
+@pytest.mark.parametrize("paged", [False, True])
+def test_corners_of_the_launch_rule(gpu, case, paged):
+    s, L, T, want_slot, want_paged = RULE_CORNERS[case]
+    bs = s.block_size
+    nb = T // bs + 16
+    w = wl.chunked_prefill(s, num_blocks=nb, num_seqs=4, chunk_tokens=T, min_context=1, max_context=40, seed=7)
+    idx = w.index
+    n = w.num_tokens
+    assert n == T
+    key, value = bf16_bits((L, n, s.num_kv_heads, s.head_dim), 3), bf16_bits((L, n, s.num_kv_heads, s.head_dim), 4)
+    pool = sentinel_pool((L, nb, 2, bs, s.num_kv_heads, s.head_dim), 5)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_reshape_and_cache(key[l], value[l], want[l], idx.slot_mapping)
+    dev = kvc.to_device(idx, bs, gpu)
+    dpool = to_bf16(pool, gpu)
+    if paged:
+        kvc.append_paged_kv_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dev.batch_indices,
+                                         dev.positions, dpool, dev.kv_block_indices,
+                                         dev.kv_block_indptrs, dev.kv_last_block_lens)
+    else:
+        kvc.reshape_and_cache_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool, dev.slot_mapping)
+    torch.cuda.synchronize()
+    ran = _lib.last_launch()
+    assert _lib.lib().kvc_tuning_modified() == 0
+    assert (ran["kernel"], ran["per_lane"], ran["threads"], ran["pipe"]) == (want_paged if paged else want_slot)
     assert np.array_equal(bits_of(dpool), want)
