@@ -16,7 +16,11 @@ All operate IN PLACE on NumPy arrays of any item size (bf16 is carried as
 uint16, as the reference's host pool does: kv_worker.py:17-22). Citations are
 paths under the reference's runtime/worker/llm_worker/. Pinning status is listed
 in the header of kvc_oracle.c; parity of the three page-table functions with
-the third-party flashinfer binary itself is UNPINNED.
+the third-party flashinfer binary itself is UNPINNED. The two functions that
+exist only here, `build_write_index_*` and `paged_write_slots_np`, are pinned in
+tests/test_host_logic.py: a step written out by hand, NumPy against loops, the
+pinned page-table functions, and (for the slots) the property that a slot-mapped
+write through them equals the page-table write.
 """
 from __future__ import annotations
 
@@ -134,6 +138,33 @@ def build_write_index_loops(input_lens, context_lens, num_blocks, kv_indices, pa
     i32 = np.int32
     return (np.asarray(cu, dtype=i32), np.asarray(indptr, dtype=i32), np.asarray(last, dtype=i32),
             np.asarray(batch, dtype=i32), np.asarray(pos, dtype=i32), np.asarray(slots, dtype=np.int64))
+
+
+def paged_write_slots_np(batch_indices, positions, kv_indices, kv_indptr, page_size) -> np.ndarray:
+    """Slot of every token of a page-table write (the addressing of
+    `append_paged_kv_cache`, models/layers/attention.py:76-85, restated as the
+    slot rule of scheduler.rs:453-541): for token i with b = batch_indices[i],
+    p = positions[i]: `kv_indices[kv_indptr[b] + p // page_size] * page_size +
+    p % page_size`; -1 where the write skips the token (no such request, negative
+    position, a page outside the request's own table or outside the array, a
+    negative page id). int64."""
+    bi = np.asarray(batch_indices, dtype=np.int64)
+    pos = np.asarray(positions, dtype=np.int64)
+    table = np.asarray(kv_indices, dtype=np.int64)
+    indptr = np.asarray(kv_indptr, dtype=np.int64)
+    batch_size = len(indptr) - 1
+    slots = np.full(len(bi), -1, dtype=np.int64)
+    for i in range(len(bi)):
+        b, p = int(bi[i]), int(pos[i])
+        if b < 0 or b >= batch_size or p < 0:
+            continue
+        entry = int(indptr[b]) + p // page_size
+        if entry < 0 or entry >= int(indptr[b + 1]) or entry >= len(table):
+            continue
+        page = int(table[entry])
+        if page >= 0:
+            slots[i] = page * page_size + p % page_size
+    return slots
 
 
 def copy_blocks_np(kv_caches, block_maps) -> None:

@@ -181,7 +181,10 @@ def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
                                       idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D,
                                       s.block_size, resolve_slots=True)   # page table walked once
     torch.cuda.synchronize()
-    assert np.array_equal(plan_r.slots.cpu().numpy(), w.index.slot_mapping)
+    assert np.array_equal(plan_r.slots.cpu().numpy(),
+                          orc.paged_write_slots_np(w.index.batch_indices, w.index.positions,
+                                                       w.index.kv_block_indices, w.index.kv_block_indptrs,
+                                                       s.block_size))
     q_buf = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=gpu)
     k_buf = torch.empty(T, Hkv * D, dtype=torch.bfloat16, device=gpu)
     g = torch.Generator().manual_seed(23)

@@ -332,7 +332,10 @@ def test_append_paged_kv_cache_matches_oracle(gpu, kind):
     for l in range(L):
         plan_r.append(dkey[l], dval[l], resolved[l])
     torch.cuda.synchronize()
-    assert np.array_equal(plan_r.slots.cpu().numpy(), w.index.slot_mapping)
+    assert np.array_equal(plan_r.slots.cpu().numpy(),
+                          orc.paged_write_slots_np(w.index.batch_indices, w.index.positions,
+                                                   w.index.kv_block_indices, w.index.kv_block_indptrs,
+                                                   s.block_size))
     assert np.array_equal(bits_of(per_layer), want)
     assert np.array_equal(bits_of(fused), want)
     assert np.array_equal(bits_of(slotted), want)
@@ -429,6 +432,7 @@ def test_append_paged_skips_tokens_with_bad_indices(gpu):
     plan.append(to_bf16(key, gpu), to_bf16(value, gpu), dpool2)
     torch.cuda.synchronize()
     slots = plan.slots.cpu().numpy()
+    assert np.array_equal(slots, orc.paged_write_slots_np(bi, pos, neg, idx.kv_block_indptrs, bs))
     assert (slots[[2, 4, 5, 6]] == -1).all() and (slots[keep] >= 0).all()
     assert np.array_equal(bits_of(dpool2), want)
     # ... and a negative page id or a page beyond the layer's pool is skipped too
@@ -444,6 +448,8 @@ def test_append_paged_skips_tokens_with_bad_indices(gpu):
     dpool3 = to_bf16(pool, gpu)
     plan.append(to_bf16(key, gpu), to_bf16(value, gpu), dpool3)
     torch.cuda.synchronize()
+    assert np.array_equal(plan.slots.cpu().numpy(),
+                          orc.paged_write_slots_np(bi, pos, neg, idx.kv_block_indptrs, bs))
     assert plan.slots.cpu().numpy()[0] == -1
     assert np.array_equal(bits_of(dpool3), want3)
     half = to_bf16(pool, gpu)[:nb // 2]

@@ -117,6 +117,47 @@ def test_index_oracle_reproduces_the_hand_case_and_its_own_loops():
         assert np.array_equal(x, y)
 
 
+def test_slot_oracle_of_the_page_table_write_is_pinned():
+    """`oracle.paged_write_slots_np`: the hand case, every skip rule on its own, and the
+    property that defines it: writing through its slots with the slot-mapped oracle
+    gives the pool the page-table oracle gives."""
+    bs = 4
+    indptr, table = [0, 2, 5, 7, 8], [4, 2, 1, 5, 6, 3, 9, 7]
+    bi = [0] * 5 + [1] * 3 + [2, 3]
+    pos = [0, 1, 2, 3, 4, 8, 9, 10, 6, 3]
+    assert orc.paged_write_slots_np(bi, pos, table, indptr, bs).tolist() == \
+        [16, 17, 18, 19, 8, 24, 25, 26, 9 * 4 + 2, 7 * 4 + 3]
+    #                        no request   beyond batch   negative pos   beyond own table   page id < 0
+    skip = orc.paged_write_slots_np([-1, 4, 0, 0, 3], [0, 0, -1, 8, 1], [4, 2, 1, 5, 6, 3, 9, -7], indptr, bs)
+    assert skip.tolist() == [-1, -1, -1, -1, -1]
+    # an entry that exists in the array but belongs to the next request is not this request's page
+    assert orc.paged_write_slots_np([0], [2 * bs], table, indptr, bs).tolist() == [-1]
+    # the indptr may promise more entries than the array holds
+    assert orc.paged_write_slots_np([3], [bs], table, [0, 2, 5, 7, 10], bs).tolist() == [-1]
+    rng = np.random.default_rng(11)
+    for seed in range(6):
+        w = wl._write_workload(wl.LLAMA_3_2_1B, 64, rng.integers(0, 60, size=4).tolist(),
+                               rng.integers(1, 20, size=4).tolist(), np.random.default_rng(seed))
+        idx, s = w.index, w.shape
+        T = w.num_tokens
+        key = rng.integers(0, 1 << 16, size=(T, s.num_kv_heads, s.head_dim), dtype=np.uint16)
+        value = rng.integers(0, 1 << 16, size=(T, s.num_kv_heads, s.head_dim), dtype=np.uint16)
+        bad_bi, bad_pos = idx.batch_indices.copy(), idx.positions.copy()
+        bad_bi[0], bad_pos[-1] = -1, 1 << 20
+        pool = rng.integers(0, 1 << 16, size=(64, 2, s.block_size, s.num_kv_heads, s.head_dim), dtype=np.uint16)
+        by_table, by_slots = pool.copy(), pool.copy()
+        # the page-table oracle states the write for valid tokens only: hand it those
+        orc.append_paged_kv_cache_np(key[1:-1], value[1:-1], bad_bi[1:-1], bad_pos[1:-1], by_table,
+                                     idx.kv_block_indices, idx.kv_block_indptrs)
+        slots = orc.paged_write_slots_np(bad_bi, bad_pos, idx.kv_block_indices, idx.kv_block_indptrs, s.block_size)
+        assert slots[0] == -1 and slots[-1] == -1 and (slots[1:-1] >= 0).all()
+        keep = slots >= 0
+        orc.reshape_and_cache_np(key[keep], value[keep], by_slots, slots[keep])
+        assert np.array_equal(by_table, by_slots)
+        assert np.array_equal(orc.paged_write_slots_np(idx.batch_indices, idx.positions, idx.kv_block_indices,
+                                                       idx.kv_block_indptrs, s.block_size), idx.slot_mapping)
+
+
 def test_make_kv_index_inputs_rejects_inconsistent_requests():
     with pytest.raises(ValueError):
         make_kv_index_inputs([InferInput(0, [1, 1], 2, 0, 3, [0])], 4)   # len mismatch
