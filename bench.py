@@ -256,7 +256,7 @@ def bench_write_config(torch, kvc, tag, sets, pool, L, steps, warmup, variants):
             continue
         results[variant] = (ms_w, ms_e)
         out.append(entry(f"{tag}/{label}", nbytes, ms_w, ms_e, calls_per_step=calls,
-                         launch="hipGraph replay" if mode == "graph" else "eager (Python + ctypes per call)"))
+                         launch="hipGraph replay" if mode == "graph" else "eager (one Python call per launch)"))
     return out, results
 
 
@@ -475,6 +475,7 @@ def per_layer_summary(entries):
         ("graph_replay_us", "cfg2 decode/append_paged_kv_cache (per layer", "hipGraph"),
         ("eager_plan_resolved_slots_us", "cfg2 decode/PagedKVWritePlan(resolve_slots).append", "eager"),
         ("graph_replay_plan_resolved_slots_us", "cfg2 decode/PagedKVWritePlan(resolve_slots).append", "hipGraph"),
+        ("rotation_then_append_eager_us", "cfg2 decode + rotation/rotary_pos_emb + append_paged_kv_cache", "eager"),
         ("rotation_fused_eager_full_wrapper_us", "cfg2 decode + rotation/rotary_pos_emb_and_append_paged", "eager"),
         ("rotation_fused_eager_plan_us", "cfg2 decode + rotation/PagedRotaryWritePlan.run", "eager"),
         ("rotation_fused_graph_replay_us", "cfg2 decode + rotation/rotary_pos_emb_and_append_paged", "hipGraph"),
@@ -610,11 +611,12 @@ def main():
                 plans_r[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
 
         n = max(R, args.steps // 8 // R * R)
-        for fn, label in ((fused, "rotary_pos_emb_and_append_paged (1 launch per layer)"),
+        for fn, label in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)"),
+                          (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)"),
                           (fused_plan, "PagedRotaryWritePlan.run (1 launch per layer)")):
             ms_w, ms_e = time_region(fn, n, 2, torch)
             extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes, ms_w, ms_e,
-                               calls_per_step=L, launch="eager (Python + ctypes per call)"))
+                               calls_per_step=L, launch="eager (one Python call per launch)"))
         for fn, label, extra_b in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
                                     2 * T * Hkv * D * E),   # rotated key written out and read back
                                    (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0),

@@ -68,8 +68,11 @@ def build_fastcall(verbose: bool = False) -> str:
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-I", INCLUDE]
     for inc in cpp_extension.include_paths():
         cmd += ["-isystem", inc]
-    cmd += ["-I", sysconfig.get_paths()["include"], FAST_SRC, "-L", PKG_DIR, "-lkvcache",
+    rocm = os.path.dirname(os.path.dirname(os.path.realpath(find_hipcc())))
+    cmd += ["-I", sysconfig.get_paths()["include"], "-D__HIP_PLATFORM_AMD__", "-isystem",
+            os.path.join(rocm, "include"), FAST_SRC, "-L", PKG_DIR, "-lkvcache",
             "-L", torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10",
+            "-L", os.path.join(rocm, "lib"), "-lamdhip64",
             f"-Wl,-rpath,$ORIGIN,-rpath,{torch_lib}", "-o", FAST_PATH + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -21,6 +21,20 @@ from . import _lib
 from .cache_ops import _inner_contiguous, _on_device_of, _require_gpu, _rows, _stream_of
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream
+_fast_entries = {}
+
+
+def _fast_entry(name: str):
+    """A function of the `_kvc_fast` extension, or None when it is not built."""
+    try:
+        return _fast_entries[name]
+    except KeyError:
+        mod = _lib.fast()
+        fn = _fast_entries[name] = getattr(mod, name, None) if mod else None
+        return fn
+
+
 def _i32(t: torch.Tensor, name: str) -> torch.Tensor:
     _require_gpu(t, name)
     if t.dtype != torch.int32:
@@ -101,6 +115,18 @@ def append_paged_kv_cache(
     """
     if isinstance(paged_kv_cache, (tuple, list)):
         raise ValueError("only the single-tensor NHD paged cache is supported")
+    if kv_layout == "NHD" and isinstance(paged_kv_cache, torch.Tensor) and paged_kv_cache.is_cuda:
+        fast = _fast_entry("append_paged")
+        if fast is not None:
+            # the common layouts are checked and launched from C++; 1 = not one of them:
+            # the checks below then name what is wrong, or handle the rare layout
+            dev = paged_kv_cache.device.index
+            rc = fast(append_key, append_value, batch_indices, positions, paged_kv_cache, kv_indices,
+                      kv_indptr, kv_last_page_len, dev, _raw_stream(dev))
+            if rc == 0:
+                return
+            if rc < 0:
+                _lib.check(rc)
     for t, n in ((append_key, "append_key"), (append_value, "append_value"),
                  (paged_kv_cache, "paged_kv_cache")):
         _require_gpu(t, n)

@@ -54,6 +54,20 @@ def make_cos_sin_cache(rotary_dim: int, max_position_embeddings: int, base: floa
     return cos_sin.to(device) if device is not None else cos_sin
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream
+_fast_entries = {}
+
+
+def _fast_entry(name: str):
+    """A function of the `_kvc_fast` extension, or None when it is not built."""
+    try:
+        return _fast_entries[name]
+    except KeyError:
+        mod = _lib.fast()
+        fn = _fast_entries[name] = getattr(mod, name, None) if mod else None
+        return fn
+
+
 def _prep(query, key, positions, cos_sin_cache, head_dim):
     for t, n in ((query, "query"), (key, "key"), (positions, "positions"),
                  (cos_sin_cache, "cos_sin_cache")):
@@ -90,6 +104,18 @@ def rotary_pos_emb(query: torch.Tensor, key: torch.Tensor, positions: torch.Tens
                    cos_sin_cache: torch.Tensor, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """Rotate `query [T, Hq*D]` and `key [T, Hkv*D]`; returns new tensors of the
     inputs' shapes (rotary_embedding_ops.py:8-35)."""
+    fast = _fast_entry("rotary_pos_emb")
+    if fast is not None and isinstance(query, torch.Tensor) and query.is_cuda and query.dim() in (2, 3) \
+            and isinstance(key, torch.Tensor) and key.dim() in (2, 3):
+        # common layouts: checked and launched from C++ (1 = not one of them: fall through)
+        dev = query.device.index
+        q_out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+        k_out = torch.empty(key.shape, dtype=key.dtype, device=key.device)
+        rc = fast(query, key, positions, cos_sin_cache, head_dim, q_out, k_out, dev, _raw_stream(dev))
+        if rc == 0:
+            return q_out, k_out
+        if rc < 0:
+            _lib.check(rc)
     q2, k2, positions, pos_bytes, kd, T = _prep(query, key, positions, cos_sin_cache, head_dim)
     q_out = torch.empty_like(q2, memory_format=torch.contiguous_format)
     k_out = torch.empty_like(k2, memory_format=torch.contiguous_format)
@@ -157,6 +183,18 @@ def rotary_pos_emb_and_append_paged(query: torch.Tensor, key: torch.Tensor, valu
     """`rotary_pos_emb` plus `append_paged_kv_cache` of the rotated key and the
     value in one launch; `positions` (int32) is both the rotation position and
     the KV position of each token, as in the reference."""
+    fast = _fast_entry("rotary_append_paged")
+    if fast is not None and isinstance(query, torch.Tensor) and query.is_cuda and query.dim() in (2, 3) \
+            and isinstance(key, torch.Tensor) and key.dim() in (2, 3):
+        dev = query.device.index
+        q_out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+        k_out = torch.empty(key.shape, dtype=key.dtype, device=key.device) if return_key else None
+        rc = fast(query, key, value, batch_indices, positions, cos_sin_cache, head_dim, paged_kv_cache,
+                  kv_indices, kv_indptr, kv_last_page_len, q_out, k_out, dev, _raw_stream(dev))
+        if rc == 0:
+            return q_out, k_out
+        if rc < 0:
+            _lib.check(rc)
     q2, k2, positions, pos_bytes, kd, T = _prep(query, key, positions, cos_sin_cache, head_dim)
     if pos_bytes != 4:
         raise TypeError("positions must be int32 for page-table addressing")

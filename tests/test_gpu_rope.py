@@ -164,6 +164,51 @@ def test_fused_paged_write_equals_rotation_then_append(gpu):
     assert int(torch.count_nonzero(pool_b.view(torch.int16))) > 0
 
 
+def test_rotation_wrappers_agree_with_and_without_the_call_extension(gpu, monkeypatch):
+    """`rotary_pos_emb` and `rotary_pos_emb_and_append_paged` check and launch the
+    common layouts from the `_kvc_fast` extension; without it the Python checks and
+    ctypes do the same work. Both routes, same bits, 2-D and 3-D inputs and
+    token-strided slices of a fused projection."""
+    from lmserve_amd import _lib
+    assert _lib.fast() is not None
+    s = wl.LLAMA_3_8B
+    w = wl._write_workload(s, 128, [3, 40, 0, 17], [1, 9, 30, 1], np.random.default_rng(23))
+    idx = kvc.to_device(w.index, s.block_size, gpu)
+    T, Hq, Hkv, D = w.num_tokens, 32, s.num_kv_heads, s.head_dim
+    cs = rotary.make_cos_sin_cache(D, 1024, 500000.0, dtype=torch.bfloat16).to(gpu)
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D, generator=torch.Generator().manual_seed(29)).bfloat16().to(gpu)
+    q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    results = {}
+    for route in ("extension", "python"):
+        if route == "python":
+            monkeypatch.setattr(rotary, "_fast_entries", {"rotary_pos_emb": None, "rotary_append_paged": None})
+        out = []
+        for qq, kk in ((q, k), (q.contiguous(), k.contiguous()), (q.reshape(T, Hq, D), k.reshape(T, Hkv, D))):
+            a, b = kvc.rotary_pos_emb(qq, kk, idx.positions, cs, D)
+            assert a.shape == qq.shape and b.shape == kk.shape
+            out += [a.reshape(T, -1).clone(), b.reshape(T, -1).clone()]
+            pool = torch.zeros(128, 2, s.block_size, Hkv, D, dtype=torch.bfloat16, device=gpu)
+            a2, b2 = kvc.rotary_pos_emb_and_append_paged(qq, kk, v, idx.batch_indices, idx.positions, cs, D,
+                                                         pool, idx.kv_block_indices, idx.kv_block_indptrs,
+                                                         idx.kv_last_block_lens)
+            a3, none = kvc.rotary_pos_emb_and_append_paged(qq, kk, v, idx.batch_indices, idx.positions, cs, D,
+                                                           pool, idx.kv_block_indices, idx.kv_block_indptrs,
+                                                           idx.kv_last_block_lens, return_key=False)
+            assert none is None
+            out += [a2.reshape(T, -1).clone(), b2.reshape(T, -1).clone(), a3.reshape(T, -1).clone(), pool.clone()]
+        torch.cuda.synchronize()
+        results[route] = out
+    for x, y in zip(results["extension"], results["python"]):
+        assert torch.equal(x.view(torch.int16), y.view(torch.int16))
+    # int64 positions rotate alike; a float table is refused on both routes
+    monkeypatch.undo()
+    a, b = kvc.rotary_pos_emb(q, k, idx.positions.long(), cs, D)
+    torch.cuda.synchronize()
+    assert torch.equal(a, results["extension"][0]) and torch.equal(b, results["extension"][1])
+    with pytest.raises(TypeError):
+        kvc.rotary_pos_emb(q, k, idx.positions, cs.float(), D)
+
+
 def test_plan_reads_slices_of_a_fused_projection_and_reuses_buffers(gpu):
     """The per-step plan gives the same bits as the full wrapper, reading q/k/v in
     place from one [T, (Hq + 2 Hkv) D] projection output and writing into buffers

@@ -467,6 +467,46 @@ def test_append_paged_skips_tokens_with_bad_indices(gpu):
     assert np.array_equal(bits_of(half), want4)
 
 
+def test_drop_in_writes_agree_with_and_without_the_call_extension(gpu, monkeypatch):
+    """`append_paged_kv_cache` and `reshape_and_cache` check and launch the common
+    layouts from the `_kvc_fast` extension; without it (or for a layout it does not
+    take) the Python checks and ctypes do the same work. Both routes, same bits."""
+    from lmserve_amd import cache_ops, paged
+    assert _lib.fast() is not None, "the call extension is built next to the library"
+    w = wl._write_workload(wl.LLAMA_3_2_1B, 128, [5, 0, 31, 16], [3, 20, 1, 16], np.random.default_rng(5))
+    s = w.shape
+    pool, want, dev, dkey, dval = _paged_case(gpu, w, 1, 60)
+    routes = {}
+    for route in ("extension", "python"):
+        if route == "python":
+            monkeypatch.setattr(paged, "_fast_entries", {"append_paged": None})
+            monkeypatch.setattr(cache_ops, "_fast_reshape", False)
+        a, b, c = to_bf16(pool, gpu), to_bf16(pool, gpu), to_bf16(pool, gpu)
+        kvc.append_paged_kv_cache(dkey[0], dval[0], dev.batch_indices, dev.positions, a[0],
+                                  dev.kv_block_indices, dev.kv_block_indptrs, dev.kv_last_block_lens)
+        kvc.reshape_and_cache(dkey[0], dval[0], b[0], dev.slot_mapping)
+        kvc.reshape_and_cache(dkey[0], dval[0], c[0], dev.slot_mapping.int())       # int32 slots
+        torch.cuda.synchronize()
+        routes[route] = [bits_of(x) for x in (a, b, c)]
+        for got in routes[route]:
+            assert np.array_equal(got, want), route
+    # a layout the extension leaves to Python: index arrays that are strided views
+    strided = torch.stack([dev.batch_indices, dev.batch_indices], dim=1)[:, 0]
+    assert not strided.is_contiguous() or strided.numel() <= 1
+    monkeypatch.undo()
+    d = to_bf16(pool, gpu)
+    kvc.append_paged_kv_cache(dkey[0], dval[0], strided, dev.positions, d[0], dev.kv_block_indices,
+                              dev.kv_block_indptrs, dev.kv_last_block_lens)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits_of(d), want)
+    # errors keep their Python types on both routes
+    with pytest.raises(TypeError):
+        kvc.append_paged_kv_cache(dkey[0], dval[0], dev.batch_indices.long(), dev.positions, d[0],
+                                  dev.kv_block_indices, dev.kv_block_indptrs, dev.kv_last_block_lens)
+    with pytest.raises(ValueError):
+        kvc.reshape_and_cache(dkey[0][:-1], dval[0], d[0], dev.slot_mapping)
+
+
 def test_write_runs_on_the_current_stream(gpu):
     """The op is enqueued on torch's current stream: a copy of the pool taken on
     the same side stream right after the call must already see the write."""
