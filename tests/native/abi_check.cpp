@@ -144,6 +144,35 @@ int main() {
   HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
   expect_equal("kvc_append_paged_kv_cache == oracle", got.data(), want_paged.data(), pool_bytes);
   expect_equal("page-table write == slot-mapped write", want_paged.data(), want.data(), pool_bytes);
+  // all layers in one launch
+  HIP_OK(hipMemcpy(d_pool, pool.data(), pool_bytes, hipMemcpyHostToDevice));
+  KVC_OK_OR_DIE(kvc_append_paged_kv_cache_layers(
+      d_key, d_value, (const int32_t*)d_bi, (const int32_t*)d_pos, d_pool, (const int32_t*)d_ind,
+      (const int32_t*)d_ptr, (const int32_t*)d_last, T, 2, (int64_t)kv_indices.size(), H, D, bs, row, row,
+      blk_elems, nb, L, T * row, T * row, layer_elems, (int)E, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+  expect_equal("kvc_append_paged_kv_cache_layers == oracle", got.data(), want_paged.data(), pool_bytes);
+  // the two index functions of the step: seq_lens = (pages - 1) * bs + last, then (request, position) per token
+  {
+    const std::vector<int32_t> cu = {0, 20, 21}, want_seq = {25, 34};
+    void *d_cu, *d_seq, *d_bi2, *d_pos2;
+    HIP_OK(hipMalloc(&d_cu, 3 * 4)); HIP_OK(hipMalloc(&d_seq, 2 * 4));
+    HIP_OK(hipMalloc(&d_bi2, T * 4)); HIP_OK(hipMalloc(&d_pos2, T * 4));
+    HIP_OK(hipMemcpy(d_cu, cu.data(), 3 * 4, hipMemcpyHostToDevice));
+    KVC_OK_OR_DIE(kvc_get_seq_lens((const int32_t*)d_ptr, (const int32_t*)d_last, 2, bs, (int32_t*)d_seq, stream));
+    KVC_OK_OR_DIE(kvc_get_batch_indices_positions((const int32_t*)d_cu, (const int32_t*)d_seq, 2, T,
+                                                  (int32_t*)d_bi2, (int32_t*)d_pos2, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<int32_t> g_seq(2), g_bi(T), g_pos(T);
+    HIP_OK(hipMemcpy(g_seq.data(), d_seq, 2 * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_bi.data(), d_bi2, T * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(g_pos.data(), d_pos2, T * 4, hipMemcpyDeviceToHost));
+    expect_equal("kvc_get_seq_lens == context lengths", g_seq.data(), want_seq.data(), 2 * 4);
+    expect_equal("kvc_get_batch_indices_positions: requests", g_bi.data(), bi.data(), T * 4);
+    expect_equal("kvc_get_batch_indices_positions: positions", g_pos.data(), pos.data(), T * 4);
+    HIP_OK(hipFree(d_cu)); HIP_OK(hipFree(d_seq)); HIP_OK(hipFree(d_bi2)); HIP_OK(hipFree(d_pos2));
+  }
 
   // 3b. the same page-table write through a per-step plan: three pointers per layer
   {
@@ -315,6 +344,34 @@ int main() {
     HIP_OK(hipStreamSynchronize(copy_stream));
     HIP_OK(hipStreamDestroy(copy_stream));
     HIP_OK(hipFree(staging));
+    KVC_OK_OR_DIE(kvc_host_free_pinned(host));
+  }
+
+  // 5b. the swap that allocates nothing: same result as the direct swap, no workspace argument
+  {
+    uint16_t* host = (uint16_t*)kvc_host_alloc_pinned(host_bytes);
+    if (!host) { std::fprintf(stderr, "pinned alloc failed: %s\n", kvc_last_error_string()); return 4; }
+    std::vector<uint16_t> want_host(host_bytes / 2);
+    for (size_t i = 0; i < want_host.size(); ++i) host[i] = want_host[i] = (uint16_t)(0x1234 + i % 97);
+    KVC_OK_OR_DIE(kvc_swap_noalloc(1, d_pool, host, out_src.data(), out_dst.data(), n, L, layer_elems * E,
+                                   blk_bytes, nb, nhb, 0, L, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    oracle_save_blocks_to_host(want.data(), want_host.data(), out_src.data(), out_dst.data(), n, L, nb,
+                               blk_bytes, 0, L);
+    expect_equal("kvc_swap_noalloc to the host == oracle", host, want_host.data(), host_bytes);
+    std::vector<int64_t> back_host = {2, 9}, back_gpu = {36, 37};   // a second, smaller call: layer 1 only
+    KVC_OK_OR_DIE(kvc_swap_noalloc(0, d_pool, host, back_gpu.data(), back_host.data(), 2, L, layer_elems * E,
+                                   blk_bytes, nb, nhb, 1, 2, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    oracle_load_blocks_from_host(want.data(), want_host.data(), back_host.data(), back_gpu.data(), 2, L, nb,
+                                 blk_bytes, 1, 2);
+    HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
+    expect_equal("kvc_swap_noalloc from the host, one layer == oracle", got.data(), want.data(), pool_bytes);
+    if (kvc_swap_noalloc(1, d_pool, host, out_src.data(), out_dst.data(), KVC_NOALLOC_MAX_BLOCKS + 1, L,
+                         layer_elems * E, blk_bytes, nb, nhb, 0, L, stream) != KVC_ERR_UNSUPPORTED) {
+      std::fprintf(stderr, "expected KVC_ERR_UNSUPPORTED beyond KVC_NOALLOC_MAX_BLOCKS\n");
+      ++fails;
+    }
     KVC_OK_OR_DIE(kvc_host_free_pinned(host));
   }
 
