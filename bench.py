@@ -541,6 +541,22 @@ def main():
     # sixth of the region; it is reported as `wall_ms_per_step`.
     achieved = bytes_step / (ms_event * 1e-3) / 1e9
     value_gbps = achieved
+    # dispersion of the same measurement: eight more regions of K steps each, event-timed
+    # the same way (not part of `value`, which is the first region's mean)
+    fused_fn = lambda i: kvc.reshape_and_cache_layers(sets[i % len(sets)][1], sets[i % len(sets)][2], pool,
+                                                      sets[i % len(sets)][3].slot_mapping)
+    regions = [ms_event]
+    for _ in range(8):
+        a_ev, b_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a_ev.record()
+        for i in range(args.steps):
+            fused_fn(i)
+        b_ev.record()
+        torch.cuda.synchronize()
+        regions.append(a_ev.elapsed_time(b_ev) / args.steps)
+    regions.sort()
+    repeats = {"regions_of_k_steps": len(regions), "median_ms_per_step": round(regions[len(regions) // 2], 6),
+               "min_ms_per_step": round(regions[0], 6), "max_ms_per_step": round(regions[-1], 6)}
 
     # a plain elementwise kernel moving the same bytes per launch as the headline
     # (32 MiB read + 32 MiB written), rotated over as many buffers: what a launch
@@ -967,6 +983,7 @@ def main():
         "wall_ms_per_step": round(ms_wall, 6),
         "timing": "mean over the K timed steps between two events on the launch stream; "
                   "wall_ms_per_step is the host clock around the same synchronised region",
+        "repeats": repeats,
         "us_per_call": round(ms_event * 1e3, 3),
         "pct_of_hbm_peak": round(100.0 * value_gbps / HBM_PEAK_GBPS, 2),
         "higher_is_better": True,
