@@ -171,6 +171,20 @@ def fast():
     return _fast or None
 
 
+_fast_entries: dict = {}
+
+
+def fast_entry(name: str):
+    """A function of the `_kvc_fast` extension by name, or None when the extension
+    is not built (looked up once per name)."""
+    try:
+        return _fast_entries[name]
+    except KeyError:
+        mod = fast()
+        fn = _fast_entries[name] = getattr(mod, name, None) if mod else None
+        return fn
+
+
 def last_error() -> str:
     return lib().kvc_last_error_string().decode("utf-8", "replace")
 

@@ -150,9 +150,6 @@ def _rows(t: torch.Tensor, name: str):
     return t, H * D, stride
 
 
-_fast_reshape = None   # `_kvc_fast.reshape_and_cache`, False when the extension is not built
-
-
 def fill_key_cache(
     key: torch.Tensor,
     value: torch.Tensor,
@@ -219,16 +216,12 @@ def reshape_and_cache(
     `kv_caches[l]` view); token `i` lands in block `slot // block_size`, entry
     `slot % block_size`: `kv_cache[blk, 0, e] = key[i]`, `kv_cache[blk, 1, e] = value[i]`.
     """
-    global _fast_reshape
     if isinstance(kv_cache, torch.Tensor) and kv_cache.is_cuda:
-        if _fast_reshape is None:
-            mod = _lib.fast()
-            _fast_reshape = getattr(mod, "reshape_and_cache", False) if mod else False
-        if _fast_reshape:
+        fast = _lib.fast_entry("reshape_and_cache")
+        if fast is not None:
             # common layouts: checked and launched from C++ (1 = not one of them: fall through)
             dev = kv_cache.device.index
-            rc = _fast_reshape(key, value, kv_cache, slot_mapping, dev,
-                               torch._C._cuda_getCurrentRawStream(dev))
+            rc = fast(key, value, kv_cache, slot_mapping, dev, torch._C._cuda_getCurrentRawStream(dev))
             if rc == 0:
                 return
             if rc < 0:

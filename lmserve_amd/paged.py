@@ -22,17 +22,7 @@ from .cache_ops import _inner_contiguous, _on_device_of, _require_gpu, _rows, _s
 
 
 _raw_stream = torch._C._cuda_getCurrentRawStream
-_fast_entries = {}
-
-
-def _fast_entry(name: str):
-    """A function of the `_kvc_fast` extension, or None when it is not built."""
-    try:
-        return _fast_entries[name]
-    except KeyError:
-        mod = _lib.fast()
-        fn = _fast_entries[name] = getattr(mod, name, None) if mod else None
-        return fn
+_fast_entry = _lib.fast_entry
 
 
 def _i32(t: torch.Tensor, name: str) -> torch.Tensor:

@@ -55,17 +55,7 @@ def make_cos_sin_cache(rotary_dim: int, max_position_embeddings: int, base: floa
 
 
 _raw_stream = torch._C._cuda_getCurrentRawStream
-_fast_entries = {}
-
-
-def _fast_entry(name: str):
-    """A function of the `_kvc_fast` extension, or None when it is not built."""
-    try:
-        return _fast_entries[name]
-    except KeyError:
-        mod = _lib.fast()
-        fn = _fast_entries[name] = getattr(mod, name, None) if mod else None
-        return fn
+_fast_entry = _lib.fast_entry
 
 
 def _prep(query, key, positions, cos_sin_cache, head_dim):

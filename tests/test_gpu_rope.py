@@ -181,7 +181,7 @@ def test_rotation_wrappers_agree_with_and_without_the_call_extension(gpu, monkey
     results = {}
     for route in ("extension", "python"):
         if route == "python":
-            monkeypatch.setattr(rotary, "_fast_entries", {"rotary_pos_emb": None, "rotary_append_paged": None})
+            monkeypatch.setattr(_lib, "_fast_entries", {"rotary_pos_emb": None, "rotary_append_paged": None})
         out = []
         for qq, kk in ((q, k), (q.contiguous(), k.contiguous()), (q.reshape(T, Hq, D), k.reshape(T, Hkv, D))):
             a, b = kvc.rotary_pos_emb(qq, kk, idx.positions, cs, D)

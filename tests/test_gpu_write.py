@@ -471,7 +471,6 @@ def test_drop_in_writes_agree_with_and_without_the_call_extension(gpu, monkeypat
     """`append_paged_kv_cache` and `reshape_and_cache` check and launch the common
     layouts from the `_kvc_fast` extension; without it (or for a layout it does not
     take) the Python checks and ctypes do the same work. Both routes, same bits."""
-    from lmserve_amd import cache_ops, paged
     assert _lib.fast() is not None, "the call extension is built next to the library"
     w = wl._write_workload(wl.LLAMA_3_2_1B, 128, [5, 0, 31, 16], [3, 20, 1, 16], np.random.default_rng(5))
     s = w.shape
@@ -479,8 +478,7 @@ def test_drop_in_writes_agree_with_and_without_the_call_extension(gpu, monkeypat
     routes = {}
     for route in ("extension", "python"):
         if route == "python":
-            monkeypatch.setattr(paged, "_fast_entries", {"append_paged": None})
-            monkeypatch.setattr(cache_ops, "_fast_reshape", False)
+            monkeypatch.setattr(_lib, "_fast_entries", {"append_paged": None, "reshape_and_cache": None})
         a, b, c = to_bf16(pool, gpu), to_bf16(pool, gpu), to_bf16(pool, gpu)
         kvc.append_paged_kv_cache(dkey[0], dval[0], dev.batch_indices, dev.positions, a[0],
                                   dev.kv_block_indices, dev.kv_block_indptrs, dev.kv_last_block_lens)
