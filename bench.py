@@ -465,6 +465,83 @@ def cpu_baseline_others(torch, wl, seconds_each):
     return out
 
 
+def bench_two_process_swap(torch, kvc, wl, dev):
+    """The reference's deployment: the KV worker is a process of its own that maps
+    the pool from an IPC handle (kv_worker.py:97-160, cli.py:115-121). A pool in a
+    segment of its own below 2 GiB, swapped out and back in by the other process;
+    the time is the request's round trip as the model process sees it (queue
+    hand-over included)."""
+    import gc
+    import multiprocessing as mp
+    import queue as queue_mod
+
+    s70 = wl.LLAMA_3_1_70B
+    L, nb, n = 16, 1536, 768                  # 1.5 GiB pool, 0.75 GiB each way
+    gc.collect()
+    torch.cuda.empty_cache()
+    pool = torch.empty(L, nb, 2, s70.block_size, s70.num_kv_heads, s70.head_dim, dtype=torch.bfloat16,
+                       device=dev)
+    ctx = mp.get_context("spawn")
+    handle = kvc.KVWorkerHandle.create(L, interprocess=True, mp_context=ctx, sync="host")
+    params = kvc.make_kv_worker_params(pool, handle, n)
+    requests, replies = ctx.Queue(), ctx.Queue()
+    child = ctx.Process(target=kvc.serve_kv_worker, args=(params, dev.index or 0, requests, replies),
+                        daemon=True)
+    child.start()
+    out = []
+    try:
+        def get(what):
+            try:
+                msg = replies.get(timeout=120)
+            except queue_mod.Empty:
+                raise RuntimeError(f"the KV-worker process did not answer ({what})")
+            if msg[0] == "error":
+                raise RuntimeError(msg[1])
+            return msg
+        get("start-up")
+        hooks = kvc.LayerSyncHooks(handle)
+        hooks.timeout = 60
+        old, host_ids, new = wl.swap_round_trip(nb, n, seed=1)
+        nbytes = n * L * s70.block_bytes
+        for direction, pairs, src, dst in (
+                ("swap_out", list(zip(old.tolist(), host_ids.tolist())), kvc.Device.GPU, kvc.Device.Host),
+                ("swap_in", list(zip(host_ids.tolist(), new.tolist())), kvc.Device.Host, kvc.Device.GPU)):
+            best = None
+            for _ in range(4):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                requests.put(("copy_kv", [pairs], int(src), int(dst)))
+                # the model's half of the layer protocol (model_worker.py:254-276): a save waits
+                # for "layer l written" per layer, a load announces "layer l landed" per layer
+                if direction == "swap_out":
+                    hooks.enable_record_after_execute = True
+                    for l in range(L):
+                        hooks.post(l)
+                    hooks.enable_record_after_execute = False
+                else:
+                    hooks.enable_wait_before_execute = True
+                    for l in range(L):
+                        hooks.pre(l)
+                    hooks.enable_wait_before_execute = False
+                get(direction)
+                t = time.perf_counter() - t0
+                best = t if best is None else min(best, t)
+            out.append({"name": f"two processes: {direction} by a KV-worker process on the IPC-mapped pool "
+                                f"(direct; {n} blocks x {L} layers x 64 KiB, request round trip)",
+                        "ms_per_call": round(best * 1e3, 2), "pcie_gbps": round(nbytes / best / 1e9, 2),
+                        "bytes_per_call": int(nbytes)})
+    finally:
+        handle.close()
+        requests.put(("stop",))
+        child.join(timeout=30)
+        if child.is_alive():
+            child.kill()
+            child.join(timeout=10)
+        del pool
+        torch.cuda.empty_cache()
+    return out
+
+
 def per_layer_summary(entries):
     """The launches a layer-by-layer forward pass can actually issue (one K/V write
     per attention layer, as runtime/worker/llm_worker/models/layers/attention.py:76-85
@@ -918,6 +995,10 @@ def main():
             worker.close()
         del pool5
         torch.cuda.empty_cache()
+        try:
+            extra += bench_two_process_swap(torch, kvc, wl, dev)
+        except Exception as exc:   # a second process is optional equipment of the bench
+            log(f"two-process swap skipped: {exc!r}")
 
     # ------------------------------------------------ one rank's slice of Llama-3.1-70B at tp=8
     if "shard" in ops:
