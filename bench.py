@@ -492,7 +492,7 @@ def bench_two_process_swap(torch, kvc, wl, dev):
     try:
         def get(what):
             try:
-                msg = replies.get(timeout=120)
+                msg = replies.get(timeout=60)
             except queue_mod.Empty:
                 raise RuntimeError(f"the KV-worker process did not answer ({what})")
             if msg[0] == "error":
