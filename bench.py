@@ -53,10 +53,11 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=320)
     p.add_argument("--warmup", type=int, default=32)
-    p.add_argument("--ops", default="write,prefill,copy,swap,rope,shard,disk,index",
+    p.add_argument("--ops", default="write,prefill,copy,swap,twoproc,rope,shard,disk,index",
                    help="comma list of extra measurements: write (per-layer / page-table variants "
                         "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
                         "rope (rotation fused with the write vs two launches), "
+                        "twoproc (a swap carried out by a KV-worker process on the IPC-mapped pool), "
                         "shard (one rank's head slice of Llama-3.1-70B at tp=8), "
                         "disk (host <-> disk tier), "
                         "index (index preparation of a step: host construction vs one launch), "
@@ -995,6 +996,7 @@ def main():
             worker.close()
         del pool5
         torch.cuda.empty_cache()
+    if "twoproc" in ops:
         try:
             extra += bench_two_process_swap(torch, kvc, wl, dev)
         except Exception as exc:   # a second process is optional equipment of the bench

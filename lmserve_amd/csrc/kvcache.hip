@@ -82,8 +82,9 @@ struct Tuning {
   int write_pipe = -1;                   // 1 = a lane waits for each load before issuing its next,
                                          // 0 = loads back to back, -1 = by rule
   int write_planes_vpt = 0; // planes per lane in that kernel (1, 2, 4, 8), 0 = by size
-  int direct_max_wgs = 128; // grid cap of the direct swap kernel: one direction of PCIe saturates
-                            // with 64 workgroups, both at once want 128 each (92 against 87 GB/s
+  int direct_max_wgs = 96;  // grid cap of the direct swap kernel: one direction of PCIe saturates
+                            // with 48-64 workgroups (more cost a 16 MiB one-layer launch 2-4 %),
+                            // both directions at once want 96 or more each (91-92 against 87 GB/s
                             // in sum); the rest of the GPU stays free for the model
 };
 Tuning g_tune;
@@ -111,7 +112,7 @@ Knob* knobs(int* count) {
       {"write_planes_max_vpr", &g_tune.write_planes_max_vpr, 256},
       {"write_planes_threads", &g_tune.write_planes_threads, 0},
       {"write_pipe", &g_tune.write_pipe, -1},
-      {"direct_max_wgs", &g_tune.direct_max_wgs, 128},
+      {"direct_max_wgs", &g_tune.direct_max_wgs, 96},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
   };
