@@ -158,11 +158,14 @@ _fast = None
 
 def fast():
     """The `_kvc_fast` extension module (METH_FASTCALL wrappers of the per-layer
-    plan calls), or None when it is not built; callers then go through ctypes to
-    the same entry points."""
+    calls), or None when it is not built or `KVC_DISABLE_CALL_EXTENSION` is set in
+    the environment; callers then go through ctypes to the same entry points."""
     global _fast
     if _fast is None:
         lib()   # the shared library first: the extension binds to the same instance
+        if os.environ.get("KVC_DISABLE_CALL_EXTENSION"):
+            _fast = False   # everything through ctypes (same entry points, more host time per call)
+            return None
         try:
             from . import _kvc_fast
             _fast = _kvc_fast if _kvc_fast.abi_version == KVC_ABI_VERSION else False

