@@ -259,6 +259,25 @@ def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
     assert out.returncode == 0 and "c ok" in out.stdout, out.stdout + out.stderr
 
 
+def test_call_extension_is_built_and_binds_the_same_library():
+    """`_kvc_fast` (the CPython entry of the per-layer calls) sits next to the library,
+    reports the library's ABI version and exposes one function per call it serves."""
+    if os.environ.get("KVC_DISABLE_CALL_EXTENSION"):
+        pytest.skip("switched off in the environment")
+    mod = _lib.fast()
+    assert mod is not None, "lmserve_amd/_kvc_fast.so is missing: run python -m lmserve_amd.build"
+    assert mod.abi_version == _lib.KVC_ABI_VERSION and mod.NOT_FAST == 1
+    for name in ("write_plan_append", "rotary_plan_run", "append_paged", "reshape_and_cache",
+                 "rotary_pos_emb", "rotary_append_paged", "scalar_type_code"):
+        assert callable(getattr(mod, name)), name
+        assert _lib.fast_entry(name) is getattr(mod, name)
+    # not tensors: every entry hands the call back to Python (1), it never guesses
+    assert mod.append_paged(*([None] * 8), 0, None) == 1
+    assert mod.reshape_and_cache(None, None, None, None, 0, None) == 1
+    with pytest.raises(TypeError):
+        mod.append_paged(None)
+
+
 def test_operators_fail_loudly_without_the_library(monkeypatch, tmp_path):
     """No CPU fallback: with the shared library absent every entry into the
     binding raises, and so do the operators that sit on it."""
