@@ -41,7 +41,7 @@ ROTATE_PREFILL = 8   # 8 x 112 MiB of K/V sources
 # 32813.8 KiB x 1.0000, the factors being what the same counters read for a
 # plain elementwise kernel of known size (1 GiB read, 1 GiB written); summary in
 # profiles/hbm_traffic_fetch_size_write_size.txt. Only valid for the default workload.
-MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67227932
+MEASURED_TRAFFIC_CFG2_ONE_LAUNCH = 67221046
 
 
 def log(*a):
