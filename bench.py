@@ -53,10 +53,11 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=320)
     p.add_argument("--warmup", type=int, default=32)
-    p.add_argument("--ops", default="write,prefill,copy,swap,twoproc,rope,shard,disk,index",
+    p.add_argument("--ops", default="write,prefill,copy,swap,overlap,twoproc,rope,shard,disk,index",
                    help="comma list of extra measurements: write (per-layer / page-table variants "
                         "of config 2), prefill (config 3), copy (config 4), swap (config 5), "
                         "rope (rotation fused with the write vs two launches), "
+                        "overlap (write-through behind a stand-in forward pass), "
                         "twoproc (a swap carried out by a KV-worker process on the IPC-mapped pool), "
                         "shard (one rank's head slice of Llama-3.1-70B at tp=8), "
                         "disk (host <-> disk tier), "
@@ -68,8 +69,6 @@ def parse_args():
                         "'none' for the headline only")
     p.add_argument("--swap-blocks", type=int, default=8192,
                    help="blocks per swap direction; 8192 (40 GiB pinned) is config 5 at its stated size")
-    p.add_argument("--staged-swap-blocks", type=int, default=1024,
-                   help="blocks per direction for the staged-mode comparison rows (a scaled run, labelled)")
     p.add_argument("--pool-blocks", type=int, default=65536)
     p.add_argument("--disk-blocks", type=int, default=256,
                    help="blocks moved by the disk-tier measurement (5 MiB each)")
@@ -466,6 +465,107 @@ def cpu_baseline_others(torch, wl, seconds_each):
     return out
 
 
+def bench_write_through_overlap(torch, kvc, wl, dev):
+    """What the layer-pipelined protocol is for (kv_worker.py:272-295,
+    model_worker.py:254-276): the KV worker saves layer l of the step's blocks to
+    the host pool while the model is already computing layer l+1. A stand-in
+    forward pass (per layer: four bf16 GEMMs of 0.11 ms, then the layer's K/V
+    write through a per-step plan, then the post hook) runs alone, the
+    layer-by-layer swap-out runs alone, and then both run together with the
+    worker (a thread of this process, as the tests run it) following the hooks:
+    once in the default staged mode (DMA engines carry the PCIe leg) and once in
+    the direct mode (a kernel writes to the mapped host pool)."""
+    import asyncio
+    import threading
+
+    import numpy as np
+
+    s8 = wl.LLAMA_3_8B
+    L, nb, n = s8.num_layers, 4096, 512            # 8 GiB pool; 512 blocks x 32 layers x 64 KiB = 1 GiB out
+    pool = torch.empty(L, nb, 2, s8.block_size, s8.num_kv_heads, s8.head_dim, dtype=torch.bfloat16, device=dev)
+    w = wl.decode_step(s8, num_blocks=nb, batch=256, max_context=200, seed=3)
+    idx = kvc.to_device(w.index, s8.block_size, dev)
+    key = torch.randn(L, 256, s8.num_kv_heads, s8.head_dim, device=dev).to(torch.bfloat16)
+    value = torch.randn_like(key)
+    a = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    b = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    c = torch.empty(4096, 4096, dtype=torch.bfloat16, device=dev)
+    plan = kvc.PagedKVWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices, idx.kv_block_indptrs,
+                                idx.kv_last_block_lens, s8.num_kv_heads, s8.head_dim, s8.block_size,
+                                torch.bfloat16, resolve_slots=True)
+    rng_ids = np.random.default_rng(5).permutation(nb)[:n]
+    maps = [kvc.BlockMapping.from_pairs(zip(rng_ids.tolist(), range(n)))]
+    model_stream = torch.cuda.Stream()
+    nbytes = n * L * s8.block_bytes
+    out = []
+    for mode in ("staged", "direct"):
+        handle = kvc.KVWorkerHandle.create(L)
+        worker = kvc.KVWorker(pool, num_host_blocks=n, swap_mode=mode, kv_worker_handle=handle)
+        hooks = kvc.LayerSyncHooks(handle)
+
+        def forward():
+            with torch.cuda.stream(model_stream):
+                for l in range(L):
+                    for _ in range(4):
+                        torch.mm(a, b, out=c)
+                    plan.append(key[l], value[l], pool[l])
+                    hooks.post(l)
+
+        def timed_forward():
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(model_stream)
+            forward()
+            e1.record(model_stream)
+            return e0, e1
+
+        try:
+            forward()                                            # warm up (hooks off: nothing posted)
+            torch.cuda.synchronize()
+            e0, e1 = timed_forward()
+            torch.cuda.synchronize()
+            fwd_alone = e0.elapsed_time(e1)
+            prepared = worker.prepare_swap("out", maps)
+            swap_alone = None
+            for _ in range(4):                                   # the first pass touches the pinned pool
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for l in range(L):
+                    worker.swap_prepared_layers(prepared, l, l + 1)
+                worker.dtoh_stream.synchronize()
+                t = (time.perf_counter() - t0) * 1e3
+                swap_alone = t if swap_alone is None else min(swap_alone, t)
+
+            def kv_thread():
+                asyncio.run(worker.copy_kv(maps, kvc.Device.GPU, kvc.Device.Host))
+
+            hooks.enable_record_after_execute = True
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            th = threading.Thread(target=kv_thread)
+            th.start()
+            e0, e1 = timed_forward()
+            th.join(timeout=120)
+            torch.cuda.synchronize()
+            total = (time.perf_counter() - t0) * 1e3
+            hooks.enable_record_after_execute = False
+            fwd_with = e0.elapsed_time(e1)
+            out.append({"name": f"write-through during a stand-in forward pass ({mode} swap; {L} layers; {n} blocks x "
+                                f"{L} layers x 64 KiB saved layer by layer behind the model's post hooks)",
+                        "forward_alone_ms": round(fwd_alone, 2), "swap_alone_ms": round(swap_alone, 2),
+                        "forward_with_write_through_ms": round(fwd_with, 2),
+                        "forward_slowdown_pct": round(100.0 * (fwd_with / fwd_alone - 1.0), 1),
+                        "both_done_after_ms": round(total, 2),
+                        "one_after_the_other_ms": round(fwd_alone + swap_alone, 2),
+                        "pcie_gbps_alone": round(nbytes / swap_alone / 1e6, 2),
+                        "bytes_per_call": int(nbytes)})
+        finally:
+            worker.close()
+            handle.close()
+    del pool
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_two_process_swap(torch, kvc, wl, dev):
     """The reference's deployment: the KV worker is a process of its own that maps
     the pool from an IPC handle (kv_worker.py:97-160, cli.py:115-121). A pool in a
@@ -486,7 +586,8 @@ def bench_two_process_swap(torch, kvc, wl, dev):
     handle = kvc.KVWorkerHandle.create(L, interprocess=True, mp_context=ctx, sync="host")
     params = kvc.make_kv_worker_params(pool, handle, n)
     requests, replies = ctx.Queue(), ctx.Queue()
-    child = ctx.Process(target=kvc.serve_kv_worker, args=(params, dev.index or 0, requests, replies),
+    mode = "staged"                           # the KV worker's default
+    child = ctx.Process(target=kvc.serve_kv_worker, args=(params, dev.index or 0, requests, replies, mode),
                         daemon=True)
     child.start()
     out = []
@@ -528,7 +629,7 @@ def bench_two_process_swap(torch, kvc, wl, dev):
                 t = time.perf_counter() - t0
                 best = t if best is None else min(best, t)
             out.append({"name": f"two processes: {direction} by a KV-worker process on the IPC-mapped pool "
-                                f"(direct; {n} blocks x {L} layers x 64 KiB, request round trip)",
+                                f"({mode}; {n} blocks x {L} layers x 64 KiB, request round trip)",
                         "ms_per_call": round(best * 1e3, 2), "pcie_gbps": round(nbytes / best / 1e9, 2),
                         "bytes_per_call": int(nbytes)})
     finally:
@@ -913,7 +1014,7 @@ def main():
         extra.append(entry(f"cfg5 scatter stage, HBM only (dense buffer -> {n} blocks x {L5} layers x 64 KiB)",
                            2 * nbytes, ms_w, ms_e, launch="eager"))
         del dense
-        worker = kvc.KVWorker(pool5, n, swap_mode="direct")
+        worker = kvc.KVWorker(pool5, n)      # swap_mode "staged": the default
         try:
             def timed_sync(fn, reps):
                 fn()   # warm-up (first touch of the pinned pool, staging allocation)
@@ -926,34 +1027,55 @@ def main():
                 return sorted(times)[len(times) // 2]
 
             size = f"{n} blocks x {L5} layers x 64 KiB"
-            for direction, maps, src, dst in (
-                    ("swap_out", out_maps, kvc.Device.GPU, kvc.Device.Host),
-                    ("swap_in", in_maps, kvc.Device.Host, kvc.Device.GPU)):
-                t = timed_sync(lambda: worker.copy_kv_sync(maps, src, dst), 3)
-                extra.append({"name": f"cfg5 {direction} (direct; {size})", "ms_per_call": round(t * 1e3, 2),
-                              "pcie_gbps": round(nbytes / t / 1e9, 2), "bytes_per_call": int(nbytes)})
+            host_in = np.arange(n // 2, n, dtype=np.int64)
+            both_out = [kvc.BlockMapping.from_pairs(zip(old[:n // 2].tolist(), range(n // 2)))]
+            both_in = [kvc.BlockMapping.from_pairs(zip(host_in.tolist(), new[n // 2:].tolist()))]
+            # "staged" (default): gather/scatter kernel + DMA extents on a second stream;
+            # "direct": one kernel that addresses the mapped host pool
+            for mode in ("staged", "direct"):
+                worker.swap_mode = mode
+                for direction, maps, src, dst in (
+                        ("swap_out", out_maps, kvc.Device.GPU, kvc.Device.Host),
+                        ("swap_in", in_maps, kvc.Device.Host, kvc.Device.GPU)):
+                    t = timed_sync(lambda: worker.copy_kv_sync(maps, src, dst), 3)
+                    extra.append({"name": f"cfg5 {direction} ({mode}; {size})", "ms_per_call": round(t * 1e3, 2),
+                                  "pcie_gbps": round(nbytes / t / 1e9, 2), "bytes_per_call": int(nbytes)})
 
-            # one call per layer, as the layer-pipelined protocol issues them: ids checked and
-            # uploaded once (kvc_swap_prepare), then one launch per layer
-            enqueue = []
+                # one call per layer, as the layer-pipelined protocol issues them: ids checked and
+                # uploaded once (kvc_swap_prepare), then one call per layer
+                enqueue = []
 
-            def layer_by_layer_prepared():
-                t0 = time.perf_counter()
-                prep = worker.prepare_swap("out", out_maps)
-                t1 = time.perf_counter()
-                for l in range(L5):
-                    worker.swap_prepared_layers(prep, l, l + 1)
-                enqueue.append((t1 - t0, time.perf_counter() - t1))
-                worker.dtoh_stream.synchronize()
+                def layer_by_layer_prepared():
+                    t0 = time.perf_counter()
+                    prep = worker.prepare_swap("out", out_maps)
+                    t1 = time.perf_counter()
+                    for l in range(L5):
+                        worker.swap_prepared_layers(prep, l, l + 1)
+                    enqueue.append((t1 - t0, time.perf_counter() - t1))
+                    worker.dtoh_stream.synchronize()
 
-            t = timed_sync(layer_by_layer_prepared, 3)
-            prep_s, calls_s = sorted(enqueue[1:])[len(enqueue[1:]) // 2]
-            extra.append({"name": f"cfg5 swap_out layer by layer, ids uploaded once (direct; {L5} calls of {n} blocks x 1 layer)",
-                          "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
-                          "bytes_per_call": int(nbytes),
-                          "host_ms_flatten_check_upload_once": round(prep_s * 1e3, 3),
-                          "host_ms_to_enqueue_all_layer_calls": round(calls_s * 1e3, 3),
-                          "host_us_per_layer_call": round(calls_s / L5 * 1e6, 2)})
+                t = timed_sync(layer_by_layer_prepared, 3)
+                prep_s, calls_s = sorted(enqueue[1:])[len(enqueue[1:]) // 2]
+                extra.append({"name": f"cfg5 swap_out layer by layer, ids uploaded once ({mode}; {L5} calls of {n} blocks x 1 layer)",
+                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                              "bytes_per_call": int(nbytes),
+                              "host_ms_flatten_check_upload_once": round(prep_s * 1e3, 3),
+                              "host_ms_to_enqueue_all_layer_calls": round(calls_s * 1e3, 3),
+                              "host_us_per_layer_call": round(calls_s / L5 * 1e6, 2)})
+
+                # both directions at once on the worker's two streams (PCIe is full duplex):
+                # write-through of one set of blocks while another set is fetched
+                def both():
+                    worker.save_kv_blocks_to_host_nowait(both_out)
+                    worker.load_kv_blocks_from_host_nowait(both_in)
+                    worker.dtoh_stream.synchronize()
+                    worker.htod_stream.synchronize()
+
+                t = timed_sync(both, 3)
+                extra.append({"name": f"cfg5 swap_out and swap_in at once ({mode}; {n // 2} blocks each way)",
+                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                              "pcie_gbps_note": "sum of both directions", "bytes_per_call": int(nbytes)})
+
             enqueue2 = []
 
             def layer_by_layer_unprepared():
@@ -968,41 +1090,15 @@ def main():
                           "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
                           "bytes_per_call": int(nbytes),
                           "host_ms_to_enqueue_all_layer_calls": round(enqueue2[-1] * 1e3, 3)})
-
-            # both directions at once on the worker's two streams (PCIe is full duplex):
-            # write-through of one set of blocks while another set is fetched
-            host_in = np.arange(n // 2, n, dtype=np.int64)
-            both_out = [kvc.BlockMapping.from_pairs(zip(old[:n // 2].tolist(), range(n // 2)))]
-            both_in = [kvc.BlockMapping.from_pairs(zip(host_in.tolist(), new[n // 2:].tolist()))]
-
-            def both():
-                worker.save_kv_blocks_to_host_nowait(both_out)
-                worker.load_kv_blocks_from_host_nowait(both_in)
-                worker.dtoh_stream.synchronize()
-                worker.htod_stream.synchronize()
-
-            t = timed_sync(both, 3)
-            extra.append({"name": f"cfg5 swap_out and swap_in at once (direct; {n // 2} blocks each way)",
-                          "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
-                          "pcie_gbps_note": "sum of both directions", "bytes_per_call": int(nbytes)})
-
-            # the staged mode (gather kernel + hipMemcpyAsync extents on a second stream) on a
-            # scaled-down id list, for comparison
-            ns = min(args.staged_swap_blocks, n)
-            worker.swap_mode = "staged"
-            s_out = [kvc.BlockMapping.from_pairs(zip(old[:ns].tolist(), host_ids[:ns].tolist()))]
-            s_in = [kvc.BlockMapping.from_pairs(zip(host_ids[:ns].tolist(), new[:ns].tolist()))]
-            sbytes = ns * L5 * s70.block_bytes
-            for direction, maps, src, dst in (("swap_out", s_out, kvc.Device.GPU, kvc.Device.Host),
-                                              ("swap_in", s_in, kvc.Device.Host, kvc.Device.GPU)):
-                t = timed_sync(lambda: worker.copy_kv_sync(maps, src, dst), 3)
-                extra.append({"name": f"cfg5 {direction} (staged; scaled to {ns} blocks x {L5} layers x 64 KiB)",
-                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
-                              "bytes_per_call": int(sbytes)})
         finally:
             worker.close()
         del pool5
         torch.cuda.empty_cache()
+    if "overlap" in ops:
+        try:
+            extra += bench_write_through_overlap(torch, kvc, wl, dev)
+        except Exception as exc:
+            log(f"write-through overlap skipped: {exc!r}")
     if "twoproc" in ops:
         try:
             extra += bench_two_process_swap(torch, kvc, wl, dev)

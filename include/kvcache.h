@@ -304,7 +304,8 @@ int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pair
  * host_pool must be pinned memory that the device can address (kvc_host_alloc_pinned).
  * staging is a device buffer of staging_bytes >= kvc_swap_staging_bytes(...):
  * its head holds the device copy of the id lists, the rest is the two-slot
- * ring used by KVC_SWAP_STAGED. Kernels run on kernel_stream, PCIe copies on
+ * ring used by KVC_SWAP_STAGED (chunk_blocks blocks per slot; 0 = about 64 MiB
+ * per slot, more when the call would otherwise take over 128 chunks). Kernels run on kernel_stream, PCIe copies on
  * copy_stream (may equal kernel_stream: then nothing overlaps). On return all
  * work is enqueued and kernel_stream has been made to wait for copy_stream's
  * part, so synchronising kernel_stream alone completes the swap.

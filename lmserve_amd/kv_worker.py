@@ -140,9 +140,15 @@ class KVWorker:
       (`[L, nb, 2, bs, H, D]`), contiguous, on the GPU. The reference maps it
       from an IPC handle in a second process (kv_worker.py:104-108); here the
       tensor itself is passed.
-    swap_mode: "direct" (default; one kernel addresses the mapped host pool,
-      no staging traffic) or "staged" (gather/scatter kernel + large DMA extents
-      on a second stream).
+    swap_mode: "staged" (default): a short gather/scatter kernel between the pool
+      and a device ring, the PCIe leg as large DMA extents on a second stream;
+      the copy engines carry the transfer, so a forward pass running on other
+      streams keeps its speed. "direct": one kernel addresses the mapped host
+      pool, no staging traffic and one launch per call; same PCIe rate, but
+      while that kernel runs, kernels of other streams are held back (a stream
+      of short GEMMs stands still beside a direct swap-out and loses a third to
+      all of the swap's duration beside a direct swap-in, measured on MI355X):
+      for an otherwise idle GPU, or when nothing may be allocated.
     kv_worker_handle: a `kv_pool.KVWorkerHandle`; when given, `copy_kv` between
       GPU and Host follows the reference's layer-pipelined protocol
       (kv_worker.py:249-295): a save waits for the model's doorbell and
@@ -161,7 +167,7 @@ class KVWorker:
         num_host_blocks: int,
         num_disk_blocks: int = 0,
         disk_kv_cache_file: Optional[str] = None,
-        swap_mode: str = "direct",
+        swap_mode: str = "staged",
         staging_chunk_blocks: int = 0,
         kv_worker_handle=None,
         disk_direct_io: bool = True,

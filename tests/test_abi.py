@@ -107,10 +107,14 @@ def test_staging_size_arithmetic():
     L = _lib.lib()
     blk, nl = 65536, 80
     ids = 2 * 8192 * 8
-    # default ring slot: as many whole blocks as fit 64 MiB
+    # default ring slot: as many whole blocks as fit 64 MiB, more when that would cut the call
+    # into more than 128 chunks
     per_block = nl * blk
     chunk = (64 << 20) // per_block
-    assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 0) == ids + 2 * chunk * per_block
+    assert chunk == 12
+    assert L.kvc_swap_staging_bytes(1024, nl, blk, _lib.KVC_SWAP_STAGED, 0) == 2 * 1024 * 8 + 2 * chunk * per_block
+    assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 0) == ids + 2 * 64 * per_block
+    assert L.kvc_swap_staging_bytes(8192, 1, blk, _lib.KVC_SWAP_STAGED, 0) == ids + 2 * 1024 * blk
     assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 4) == ids + 8 * per_block
     assert L.kvc_swap_staging_bytes(3, nl, blk, _lib.KVC_SWAP_STAGED, 100) == 256 + 6 * per_block
     assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_DIRECT, 0) == ids
