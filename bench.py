@@ -1122,24 +1122,26 @@ def main():
         n = min(4096, args.swap_blocks * 4, nbs // 2)
         old, host_ids, new = wl.swap_round_trip(nbs, n, seed=0)
         nbytes = n * Ls * sh.block_bytes
-        worker = kvc.KVWorker(pool_s, n, swap_mode="direct")
+        worker = kvc.KVWorker(pool_s, n)
         try:
-            for direction, maps_, src, dst in (
-                    ("swap_out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))],
-                     kvc.Device.GPU, kvc.Device.Host),
-                    ("swap_in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))],
-                     kvc.Device.Host, kvc.Device.GPU)):
-                worker.copy_kv_sync(maps_, src, dst)
-                times = []
-                for _ in range(3):
-                    torch.cuda.synchronize()
-                    t0 = time.perf_counter()
+            for mode in ("staged", "direct"):
+                worker.swap_mode = mode
+                for direction, maps_, src, dst in (
+                        ("swap_out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))],
+                         kvc.Device.GPU, kvc.Device.Host),
+                        ("swap_in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))],
+                         kvc.Device.Host, kvc.Device.GPU)):
                     worker.copy_kv_sync(maps_, src, dst)
-                    times.append(time.perf_counter() - t0)
-                t = sorted(times)[1]
-                extra.append({"name": f"70B/tp8 shard {direction} (direct; {n} blocks x {Ls} layers x 8 KiB)",
-                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
-                              "bytes_per_call": int(nbytes)})
+                    times = []
+                    for _ in range(3):
+                        torch.cuda.synchronize()
+                        t0 = time.perf_counter()
+                        worker.copy_kv_sync(maps_, src, dst)
+                        times.append(time.perf_counter() - t0)
+                    t = sorted(times)[1]
+                    extra.append({"name": f"70B/tp8 shard {direction} ({mode}; {n} blocks x {Ls} layers x 8 KiB)",
+                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                  "bytes_per_call": int(nbytes)})
         finally:
             worker.close()
         del pool_s, sets_s
