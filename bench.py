@@ -586,7 +586,7 @@ def bench_two_process_swap(torch, kvc, wl, dev):
     handle = kvc.KVWorkerHandle.create(L, interprocess=True, mp_context=ctx, sync="host")
     params = kvc.make_kv_worker_params(pool, handle, n)
     requests, replies = ctx.Queue(), ctx.Queue()
-    mode = "staged"                           # the KV worker's default
+    mode = "auto"                             # the KV worker's default; consecutive host blocks: staged
     child = ctx.Process(target=kvc.serve_kv_worker, args=(params, dev.index or 0, requests, replies, mode),
                         daemon=True)
     child.start()
@@ -1014,7 +1014,7 @@ def main():
         extra.append(entry(f"cfg5 scatter stage, HBM only (dense buffer -> {n} blocks x {L5} layers x 64 KiB)",
                            2 * nbytes, ms_w, ms_e, launch="eager"))
         del dense
-        worker = kvc.KVWorker(pool5, n)      # swap_mode "staged": the default
+        worker = kvc.KVWorker(pool5, n)
         try:
             def timed_sync(fn, reps):
                 fn()   # warm-up (first touch of the pinned pool, staging allocation)
@@ -1076,6 +1076,42 @@ def main():
                               "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
                               "pcie_gbps_note": "sum of both directions", "bytes_per_call": int(nbytes)})
 
+            # host blocks that do not neighbour each other (every second block of the host pool:
+            # what an allocator hands out after churn): the staged mode's PCIe leg falls apart into
+            # one copy per block, the direct kernel does not care, "auto" picks per call
+            ns = min(512, n // 2)
+            scat_maps = [kvc.BlockMapping.from_pairs(zip(old[:ns].tolist(), range(0, 2 * ns, 2)))]
+            sbytes = ns * L5 * s70.block_bytes
+            for mode in ("staged", "direct", "auto"):
+                worker.swap_mode = mode
+                picked = {}
+
+                def scattered_layer_by_layer():
+                    prep = worker.prepare_swap("out", scat_maps)
+                    for l in range(L5):
+                        worker.swap_prepared_layers(prep, l, l + 1)
+                    picked["layer"] = _lib.last_swap_mode()
+                    worker.dtoh_stream.synchronize()
+
+                def scattered_one_call():
+                    worker.save_kv_blocks_to_host_nowait(scat_maps)
+                    picked["all"] = _lib.last_swap_mode()
+                    worker.dtoh_stream.synchronize()
+
+                names = {_lib.KVC_SWAP_STAGED: "staged", _lib.KVC_SWAP_DIRECT: "direct"}
+                t = timed_sync(scattered_layer_by_layer, 3)
+                extra.append({"name": f"cfg5 swap_out to scattered host blocks, layer by layer ({mode}"
+                                      f"{' -> ' + names[picked['layer']] if mode == 'auto' else ''}; "
+                                      f"{L5} calls of {ns} blocks x 1 layer, 64 KiB extents)",
+                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
+                              "bytes_per_call": int(sbytes)})
+                t = timed_sync(scattered_one_call, 3)
+                extra.append({"name": f"cfg5 swap_out to scattered host blocks, one call ({mode}"
+                                      f"{' -> ' + names[picked['all']] if mode == 'auto' else ''}; "
+                                      f"{ns} blocks x {L5} layers, 5 MiB extents)",
+                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
+                              "bytes_per_call": int(sbytes)})
+            worker.swap_mode = "direct"
             enqueue2 = []
 
             def layer_by_layer_unprepared():

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define KVC_ABI_VERSION 2
+#define KVC_ABI_VERSION 3
 
 typedef enum kvc_status {
   KVC_OK = 0,
@@ -52,8 +52,12 @@ typedef enum kvc_status {
 typedef enum kvc_swap_mode {
   KVC_SWAP_STAGED = 0, /* gather/scatter kernel <-> device staging ring, large
                           hipMemcpyAsync extents on the copy stream, overlapped */
-  KVC_SWAP_DIRECT = 1  /* one kernel that loads/stores the pinned host pool
+  KVC_SWAP_DIRECT = 1, /* one kernel that loads/stores the pinned host pool
                           through its device mapping (no staging traffic)       */
+  KVC_SWAP_AUTO = 2    /* per call: staged when the host ids of the call form
+                          runs that make the PCIe copies 4 MiB or more in the
+                          mean (knob auto_min_extent_bytes), direct otherwise,
+                          and direct when `staging` holds no ring               */
 } kvc_swap_mode;
 
 int kvc_abi_version(void);
@@ -105,7 +109,8 @@ enum {
   KVC_LAUNCH_THREADS = 3,      /* lanes per workgroup                               */
   KVC_LAUNCH_GRID = 4,         /* workgroups                                        */
   KVC_LAUNCH_NON_TEMPORAL = 5, /* bit 0 stores, bit 1 loads (tile kernel: both = 1) */
-  KVC_LAUNCH_PIPE = 6          /* write kernels: 1 = a lane waits for each of its loads */
+  KVC_LAUNCH_PIPE = 6,         /* write kernels: 1 = a lane waits for each of its loads */
+  KVC_LAUNCH_SWAP_MODE = 7     /* the kvc_swap_mode this thread's last swap call ran in  */
 };
 int64_t kvc_last_launch_info(int what);
 
@@ -305,8 +310,13 @@ int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pair
  * staging is a device buffer of staging_bytes >= kvc_swap_staging_bytes(...):
  * its head holds the device copy of the id lists, the rest is the two-slot
  * ring used by KVC_SWAP_STAGED (chunk_blocks blocks per slot; 0 = about 64 MiB
- * per slot, more when the call would otherwise take over 128 chunks). Kernels run on kernel_stream, PCIe copies on
- * copy_stream (may equal kernel_stream: then nothing overlaps). On return all
+ * per slot, more when the call would otherwise take over 128 chunks).
+ * KVC_SWAP_AUTO wants the staged size and falls back to the direct kernel when
+ * the buffer holds the id lists only. The staged PCIe copies follow the runs of
+ * consecutive host ids in the order given: a caller that sorts the pairs of a
+ * call by host id gets the longest runs. Kernels run on kernel_stream, PCIe
+ * copies on copy_stream (may equal kernel_stream: then nothing overlaps; a
+ * staged call of one chunk uses kernel_stream for both). On return all
  * work is enqueued and kernel_stream has been made to wait for copy_stream's
  * part, so synchronising kernel_stream alone completes the swap.
  * ------------------------------------------------------------------------- */
@@ -341,7 +351,7 @@ int kvc_swap_in(void* pool, const void* host_pool,
  *     destinations of a swap-in). Neither checks nor uploads anything; in
  *     KVC_SWAP_DIRECT mode the call is one kernel launch and host_ids may be
  *     NULL; KVC_SWAP_STAGED still needs the HOST array host_ids for its PCIe
- *     extents. The caller orders these calls after the prepare call (same
+ *     extents, and KVC_SWAP_AUTO reads it to choose (NULL: direct). The caller orders these calls after the prepare call (same
  *     stream, or an event) and keeps `staging` untouched in between.
  * kvc_thread_release frees what the swap entry points keep per calling thread
  * (events, pinned id bounce buffers); it waits for that thread's pending id

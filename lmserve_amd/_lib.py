@@ -32,6 +32,7 @@ KVC_DISK_INFO_BOUNCED = 5
 
 KVC_SWAP_STAGED = 0
 KVC_SWAP_DIRECT = 1
+KVC_SWAP_AUTO = 2
 
 KVC_KERNEL_NONE = 0
 KVC_KERNEL_WRITE_ROWS = 1
@@ -44,8 +45,9 @@ KVC_LAUNCH_THREADS = 3
 KVC_LAUNCH_GRID = 4
 KVC_LAUNCH_NON_TEMPORAL = 5
 KVC_LAUNCH_PIPE = 6
+KVC_LAUNCH_SWAP_MODE = 7
 
-KVC_ABI_VERSION = 2
+KVC_ABI_VERSION = 3
 KVC_NOALLOC_MAX_BLOCKS = 8192
 
 KVC_DTYPE_BF16 = 0
@@ -220,6 +222,12 @@ def get_tuning(key: str) -> int:
 
 def reset_tuning() -> None:
     check(lib().kvc_reset_tuning())
+
+
+def last_swap_mode() -> int:
+    """The KVC_SWAP_* mode the calling thread's most recent swap call ran in
+    (what KVC_SWAP_AUTO chose); -1 before the first."""
+    return int(lib().kvc_last_launch_info(KVC_LAUNCH_SWAP_MODE))
 
 
 def last_launch() -> dict:

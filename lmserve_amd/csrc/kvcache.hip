@@ -86,6 +86,10 @@ struct Tuning {
                             // with 48-64 workgroups (more cost a 16 MiB one-layer launch 2-4 %),
                             // both directions at once want 96 or more each (91-92 against 87 GB/s
                             // in sum); the rest of the GPU stays free for the model
+  int auto_min_extent_bytes = 4 << 20;  // KVC_SWAP_AUTO: mean bytes per PCIe copy from which a call
+                                        // goes through the copy engines (a copy costs about 10 us
+                                        // beyond its transfer time: 88 % of the link rate at 4 MiB,
+                                        // 48 % at 512 KiB, 11 % at 64 KiB)
 };
 Tuning g_tune;
 
@@ -113,6 +117,7 @@ Knob* knobs(int* count) {
       {"write_planes_threads", &g_tune.write_planes_threads, 0},
       {"write_pipe", &g_tune.write_pipe, -1},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 96},
+      {"auto_min_extent_bytes", &g_tune.auto_min_extent_bytes, 4 << 20},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
   };
@@ -132,6 +137,7 @@ struct LastLaunch {
   int64_t kernel = KVC_KERNEL_NONE, vec = 0, per_lane = 0, threads = 0, grid = 0, nt = 0, pipe = 0;
 };
 thread_local LastLaunch g_last;
+thread_local int g_last_swap_mode = -1;  // the mode this thread's most recent swap call ran in
 
 constexpr int kThreads = 256;
 
@@ -1225,9 +1231,30 @@ TileArgs direct_swap_tiles(bool out, char* pool, char* host_pool, const int64_t*
   return t;
 }
 
+// KVC_SWAP_AUTO: the copy engines when the PCIe leg of this call is made of large
+// extents, the direct kernel when it would fall apart into small copies. The
+// engines leave the kernels of other streams alone, but every copy costs about
+// 10 us beyond its transfer time, so scattered host blocks of one layer (64 KiB
+// each) move at a ninth of the link rate; the direct kernel holds the link rate
+// whatever the ids are, but holds back the kernels of other streams while it runs.
+int resolve_auto_mode(const int64_t* host_ids, const SwapGeom& g, const void* staging,
+                      int64_t staging_bytes) {
+  const int64_t nl = g.layer_end - g.layer_begin;
+  if (!host_ids || !staging || g.n <= 0 || nl <= 0 || g.block_bytes <= 0) return KVC_SWAP_DIRECT;
+  const int64_t width = nl * g.block_bytes;
+  if (staging_bytes < ids_region_bytes(g.n) + 2 * round_up(width, kIdAlign)) return KVC_SWAP_DIRECT;
+  int64_t runs = 1;
+  for (int64_t i = 1; i < g.n; ++i) runs += host_ids[i] != host_ids[i - 1] + 1;
+  // mean extent = n * width / runs, compared without the division
+  return (g.n * width >= runs * (int64_t)g_tune.auto_min_extent_bytes) ? KVC_SWAP_STAGED
+                                                                        : KVC_SWAP_DIRECT;
+}
+
 int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_t* gpu_ids,
              const int64_t* host_ids, const SwapGeom& g, void* staging, int64_t staging_bytes,
              int mode, bool prepared, void* kernel_stream, void* copy_stream) {
+  if (mode == KVC_SWAP_AUTO) mode = resolve_auto_mode(host_ids, g, staging, staging_bytes);
+  g_last_swap_mode = mode;
   int64_t chunk_blocks = 0;
   int rc = check_swap(fn, pool, host_pool, gpu_ids, host_ids, g, staging, staging_bytes, mode,
                       prepared, &chunk_blocks);
@@ -1446,6 +1473,7 @@ int64_t kvc_last_launch_info(int what) {
     case KVC_LAUNCH_GRID: return g_last.grid;
     case KVC_LAUNCH_NON_TEMPORAL: return g_last.nt;
     case KVC_LAUNCH_PIPE: return g_last.pipe;
+    case KVC_LAUNCH_SWAP_MODE: return g_last_swap_mode;
     default: return KVC_ERR_INVALID_ARG;
   }
 }
@@ -1737,6 +1765,8 @@ int64_t kvc_swap_staging_bytes(int64_t n, int64_t num_layers_in_range, int64_t b
                                int mode, int64_t chunk_blocks) {
   if (n < 0 || num_layers_in_range < 0 || block_bytes < 0) return KVC_ERR_INVALID_ARG;
   const int64_t ids = std::max<int64_t>(ids_region_bytes(n), kIdAlign);
+  if (mode != KVC_SWAP_STAGED && mode != KVC_SWAP_AUTO && mode != KVC_SWAP_DIRECT)
+    return KVC_ERR_INVALID_ARG;
   if (mode == KVC_SWAP_DIRECT || n == 0) return ids;
   const int64_t per_block = round_up(num_layers_in_range * block_bytes, kIdAlign);
   if (per_block == 0) return ids;

@@ -29,7 +29,7 @@ from .kv_worker import BlockMapping, Device, KVWorker
 
 
 def serve_kv_worker(params: KVWorkerParams, device: int, requests, replies,
-                    swap_mode: str = "staged") -> None:
+                    swap_mode: str = "auto") -> None:
     """Process entry point (target of `multiprocessing.Process`, spawn context)."""
     torch.cuda.set_device(device)
     try:

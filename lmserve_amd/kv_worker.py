@@ -68,7 +68,7 @@ dtype_map = {
     torch.int32: np.int32,
 }
 
-SWAP_MODES = {"staged": _lib.KVC_SWAP_STAGED, "direct": _lib.KVC_SWAP_DIRECT}
+SWAP_MODES = {"staged": _lib.KVC_SWAP_STAGED, "direct": _lib.KVC_SWAP_DIRECT, "auto": _lib.KVC_SWAP_AUTO}
 
 
 def flatten_block_mappings(block_mappings: Sequence[BlockMapping]) -> Tuple[np.ndarray, np.ndarray]:
@@ -82,6 +82,18 @@ def flatten_block_mappings(block_mappings: Sequence[BlockMapping]) -> Tuple[np.n
             src.append(entry.src_block_id)
             dst.append(entry.dst_block_id)
     return np.asarray(src, dtype=np.int64), np.asarray(dst, dtype=np.int64)
+
+
+def order_by_host_id(gpu_ids: np.ndarray, host_ids: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """The pairs of one swap call in ascending order of their host block id
+    (stable), so that host blocks which lie next to each other in the pool are
+    next to each other in the call and leave as one PCIe extent. The result of a
+    swap does not depend on the order of its pairs (the reference copies them
+    one after the other, kv_worker.py:197-227, and they touch distinct blocks)."""
+    if host_ids.size > 1 and bool(np.any(host_ids[1:] < host_ids[:-1])):
+        order = np.argsort(host_ids, kind="stable")
+        return gpu_ids[order], host_ids[order]
+    return gpu_ids, host_ids
 
 
 class PinnedHostPool:
@@ -140,15 +152,20 @@ class KVWorker:
       (`[L, nb, 2, bs, H, D]`), contiguous, on the GPU. The reference maps it
       from an IPC handle in a second process (kv_worker.py:104-108); here the
       tensor itself is passed.
-    swap_mode: "staged" (default): a short gather/scatter kernel between the pool
-      and a device ring, the PCIe leg as large DMA extents on a second stream;
+    swap_mode: "staged": a short gather/scatter kernel between the pool and a
+      device ring, the PCIe leg as DMA extents (runs of consecutive host ids);
       the copy engines carry the transfer, so a forward pass running on other
-      streams keeps its speed. "direct": one kernel addresses the mapped host
-      pool, no staging traffic and one launch per call; same PCIe rate, but
-      while that kernel runs, kernels of other streams are held back (a stream
-      of short GEMMs stands still beside a direct swap-out and loses a third to
-      all of the swap's duration beside a direct swap-in, measured on MI355X):
-      for an otherwise idle GPU, or when nothing may be allocated.
+      streams keeps its speed, but every extent costs about 10 us beyond its
+      transfer time: host blocks scattered over the pool, one layer per call,
+      move at a ninth of the link rate. "direct": one kernel addresses the
+      mapped host pool, no staging traffic, one launch per call and the link
+      rate whatever the ids are; but while that kernel runs, kernels of other
+      streams are held back (a stream of short GEMMs stands still beside a
+      direct swap-out, measured on MI355X). "auto" (default): per call, staged
+      when the call's extents are 4 MiB or more in the mean, else direct. The
+      mappings of a call are sorted by host block id first (their order does not
+      matter to the result), so a call's host blocks form the longest runs they
+      can.
     kv_worker_handle: a `kv_pool.KVWorkerHandle`; when given, `copy_kv` between
       GPU and Host follows the reference's layer-pipelined protocol
       (kv_worker.py:249-295): a save waits for the model's doorbell and
@@ -167,7 +184,7 @@ class KVWorker:
         num_host_blocks: int,
         num_disk_blocks: int = 0,
         disk_kv_cache_file: Optional[str] = None,
-        swap_mode: str = "staged",
+        swap_mode: str = "auto",
         staging_chunk_blocks: int = 0,
         kv_worker_handle=None,
         disk_direct_io: bool = True,
@@ -255,6 +272,10 @@ class KVWorker:
             return
         src = np.ascontiguousarray(src, dtype=np.int64)
         dst = np.ascontiguousarray(dst, dtype=np.int64)
+        if direction == "out":
+            src, dst = order_by_host_id(src, dst)
+        else:
+            dst, src = order_by_host_id(dst, src)
         with torch.cuda.device(self.device):
             # whatever the caller's current stream has queued on the pool comes first
             stream.wait_stream(torch.cuda.current_stream(self.device))
@@ -304,7 +325,7 @@ class KVWorker:
         n = int(src.shape[0])
         if n == 0:
             return None
-        gpu_ids, host_ids = (src, dst) if direction == "out" else (dst, src)
+        gpu_ids, host_ids = order_by_host_id(*((src, dst) if direction == "out" else (dst, src)))
         if stream is None:
             stream = self.dtoh_stream if direction == "out" else self.htod_stream
         copy_stream = self._dtoh_copy_stream if direction == "out" else self._htod_copy_stream

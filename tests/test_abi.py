@@ -118,6 +118,10 @@ def test_staging_size_arithmetic():
     assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 4) == ids + 8 * per_block
     assert L.kvc_swap_staging_bytes(3, nl, blk, _lib.KVC_SWAP_STAGED, 100) == 256 + 6 * per_block
     assert L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_DIRECT, 0) == ids
+    # the per-call choice wants room for the staged path
+    assert (L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_AUTO, 0)
+            == L.kvc_swap_staging_bytes(8192, nl, blk, _lib.KVC_SWAP_STAGED, 0))
+    assert L.kvc_swap_staging_bytes(8192, nl, blk, 3, 0) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_swap_staging_bytes(-1, nl, blk, 0, 0) < 0
 
 
@@ -157,7 +161,7 @@ def test_tuning_knobs_read_back_and_reset():
     defaults = {"copy_unroll": 0, "gather_unroll": 0, "copy_nt": 1, "copy_max_wgs": 0, "copy_order": 0,
                 "write_vpt": 0, "write_nt": 1, "write_order": 0, "write_threads": 0, "write_planes": 1,
                 "write_planes_vpt": 0, "write_planes_min_bytes": 256 << 10, "write_planes_max_vpr": 256, "write_planes_threads": 0,
-                "write_pipe": -1, "direct_max_wgs": 96, "rope_threads": 0, "disk_bounce_mib": 4}
+                "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 4 << 20, "rope_threads": 0, "disk_bounce_mib": 4}
     for key, value in defaults.items():
         assert _lib.get_tuning(key) == value, key
     for i, key in enumerate(defaults):
@@ -229,6 +233,10 @@ def test_plans_and_prepared_swap_validate_before_touching_the_gpu():
                None, None) == _lib.KVC_ERR_STAGING
     assert out(4096, 4096, None, 0, 2, 65536, 1024, 64, 64, 0, 2, None, 0, _lib.KVC_SWAP_DIRECT,
                None, None) == _lib.KVC_OK
+    assert out(4096, 4096, None, 0, 2, 65536, 1024, 64, 64, 0, 2, None, 0, _lib.KVC_SWAP_AUTO,
+               None, None) == _lib.KVC_OK                                        # nothing to move
+    assert out(4096, 4096, None, 3, 2, 65536, 1024, 64, 64, 0, 2, 4096, 4096, 3,
+               None, None) == _lib.KVC_ERR_INVALID_ARG                          # no such mode
     assert L.kvc_swap_in_prepared(None, 4096, None, 3, 2, 65536, 1024, 64, 64, 0, 2, 4096, 4096,
                                   _lib.KVC_SWAP_DIRECT, None, None) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_thread_release() == _lib.KVC_OK       # nothing held by this thread: a no-op

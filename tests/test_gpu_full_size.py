@@ -156,7 +156,7 @@ def test_config4_copy_blocks_full_pool(gpu):
     _check_pattern(pool3, holder, blk_term, elem_term, "copy_blocks twice")
 
 
-@pytest.mark.parametrize("mode", ["direct", "staged"])
+@pytest.mark.parametrize("mode", ["direct", "staged", "auto"])
 def test_config5_swap_round_trip_full(gpu, mode):
     """Llama-3.1-70B shape: scattered blocks -> contiguous pinned host buffer ->
     fresh random blocks; the payload must arrive bit-exact and nothing else may change."""
@@ -201,11 +201,13 @@ def test_config5_swap_layer_by_layer_with_ids_uploaded_once(gpu):
     blk_term, elem_term = _pattern_terms(nb, pool3.shape[2], gpu)
     _fill_pattern(pool3, blk_term, elem_term)
     old, host_ids, new = wl.swap_round_trip(nb, n, seed=1)
-    worker = kvc.KVWorker(pool, n, swap_mode="direct")
+    worker = kvc.KVWorker(pool, n)      # the default mode: decided per call from the host ids
     try:
         out = worker.prepare_swap("out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))])
         for l in range(L):
             worker.swap_prepared_layers(out, l, l + 1)
+        # consecutive host blocks: each layer leaves as one extent through the copy engines
+        assert _lib.last_swap_mode() == _lib.KVC_SWAP_STAGED
         worker.dtoh_stream.synchronize()
         back = worker.prepare_swap("in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))])
         for l in range(L):

@@ -13,7 +13,7 @@ from tests.helpers import bits_of, random_pool, sentinel_pool, to_bf16
 
 pytestmark = pytest.mark.gpu
 
-MODES = ["staged", "direct"]
+MODES = ["staged", "direct", "auto"]
 
 
 def _mappings(src, dst, pieces=3):
@@ -270,6 +270,52 @@ def test_staged_swap_of_a_layer_range_with_runs_of_consecutive_host_ids(gpu, chu
         w.htod_stream.synchronize()
         assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), want)
     finally:
+        w.close()
+
+
+def test_auto_mode_takes_the_copy_engines_for_long_runs_and_the_kernel_for_scattered_blocks(gpu):
+    """"auto" decides per call from the host ids: runs of consecutive host blocks
+    whose PCIe extents reach the threshold go through the staging ring, scattered
+    blocks through the direct kernel; both give the oracle's bytes. The worker
+    sorts a call's pairs by host id, so a shuffled dense range still forms one run."""
+    from lmserve_amd import _lib
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb, n = 4, 64, 32, 12
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)      # 32 KiB per layer and block
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, "auto", seed=41)
+    cases = [
+        ("one run, all layers", np.arange(4, 4 + n), (0, L), 256 << 10, _lib.KVC_SWAP_STAGED),
+        ("one run given in shuffled order", np.random.default_rng(1).permutation(np.arange(4, 4 + n)), (0, L),
+         256 << 10, _lib.KVC_SWAP_STAGED),
+        ("every second host block", np.arange(0, 2 * n, 2), (0, L), 256 << 10, _lib.KVC_SWAP_DIRECT),
+        ("one run, one layer, under the threshold", np.arange(4, 4 + n), (1, 2), 1 << 20, _lib.KVC_SWAP_DIRECT),
+        ("one run, one layer, over the threshold", np.arange(4, 4 + n), (1, 2), 256 << 10, _lib.KVC_SWAP_STAGED),
+        ("the default threshold on a small call", np.arange(4, 4 + n), (0, L), None, _lib.KVC_SWAP_DIRECT),
+    ]
+    try:
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        rng = np.random.default_rng(42)
+        for name, host_ids, (lb, le), threshold, want_mode in cases:
+            _lib.reset_tuning()
+            if threshold is not None:
+                _lib.set_tuning("auto_min_extent_bytes", threshold)
+            host_ids = np.asarray(host_ids, dtype=np.int64)
+            old = rng.permutation(nb)[:n].astype(np.int64)
+            host_np = w.host_kv_caches.copy()
+            orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids, lb, le)
+            w.save_kv_blocks_to_host_nowait(_mappings(old, host_ids), layer_begin=lb, layer_end=le)
+            assert _lib.last_swap_mode() == want_mode, name
+            w.dtoh_stream.synchronize()
+            assert np.array_equal(w.host_kv_caches, host_np), name
+            new = rng.permutation(nb)[:n].astype(np.int64)
+            orc.c_load_blocks_from_host(gpu_np, host_np, host_ids, new, lb, le)
+            prepared = w.prepare_swap("in", _mappings(host_ids, new))
+            w.swap_prepared_layers(prepared, lb, le)
+            assert _lib.last_swap_mode() == want_mode, name
+            w.htod_stream.synchronize()
+            assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np), name
+    finally:
+        _lib.reset_tuning()
         w.close()
 
 

@@ -37,6 +37,22 @@ def test_flatten_block_mappings_concatenates_in_order():
     assert src.shape == (0,)
 
 
+def test_pairs_of_a_swap_call_are_ordered_by_host_block_id():
+    from lmserve_amd.kv_worker import order_by_host_id
+    gpu = np.asarray([70, 71, 72, 73, 74, 75], dtype=np.int64)
+    host = np.asarray([9, 3, 4, 10, 2, 3], dtype=np.int64)
+    g, h = order_by_host_id(gpu, host)
+    assert h.tolist() == [2, 3, 3, 4, 9, 10]
+    assert g.tolist() == [74, 71, 75, 72, 70, 73]            # pairs stay together, ties keep their order
+    assert g.flags["C_CONTIGUOUS"] and h.flags["C_CONTIGUOUS"] and g.dtype == np.int64
+    # an ascending list is handed back as it is
+    asc = np.asarray([1, 2, 5], dtype=np.int64)
+    g2, h2 = order_by_host_id(gpu[:3], asc)
+    assert g2 is not None and h2 is asc
+    e = np.zeros(0, dtype=np.int64)
+    assert order_by_host_id(e, e)[1].size == 0
+
+
 def test_device_enum_matches_the_wire_values():
     assert (int(kvc.Device.GPU), int(kvc.Device.Host), int(kvc.Device.Disk)) == (0, 1, 2)
 
