@@ -13,6 +13,7 @@
 #include <cstring>
 #include <numeric>
 #include <random>
+#include <string>
 #include <vector>
 
 #include "kvcache.h"
@@ -272,12 +273,13 @@ int main() {
   HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
   expect_equal("kvc_copy_blocks == oracle", got.data(), want.data(), pool_bytes);
 
-  // 5. swap out / in, both modes, through library-pinned host memory
+  // 5. swap out / in, every mode, through library-pinned host memory
   const int64_t nhb = 10, n = 6;
   std::vector<int64_t> out_src = {30, 0, 47, 19, 5, 11}, out_dst = {2, 3, 4, 9, 0, 6};
   std::vector<int64_t> in_src = {9, 0, 3}, in_dst = {44, 45, 13};
   const size_t host_bytes = (size_t)(nhb * L * blk_bytes);
-  for (int mode = 0; mode < 2; ++mode) {
+  for (int mode = 0; mode < 3; ++mode) {
+    const std::string tag = mode == KVC_SWAP_STAGED ? " (staged)" : mode == KVC_SWAP_DIRECT ? " (direct)" : " (auto)";
     uint16_t* host = (uint16_t*)kvc_host_alloc_pinned(host_bytes);
     if (!host) { std::fprintf(stderr, "pinned alloc failed: %s\n", kvc_last_error_string()); return 4; }
     std::vector<uint16_t> want_host(host_bytes / 2);
@@ -292,16 +294,27 @@ int main() {
     HIP_OK(hipStreamSynchronize(stream));
     oracle_save_blocks_to_host(want.data(), want_host.data(), out_src.data(), out_dst.data(), n, L, nb,
                                blk_bytes, 0, L);
-    expect_equal(mode ? "kvc_swap_out (direct) == oracle" : "kvc_swap_out (staged) == oracle", host,
-                 want_host.data(), host_bytes);
+    expect_equal(("kvc_swap_out" + tag + " == oracle").c_str(), host, want_host.data(), host_bytes);
+    if (mode == KVC_SWAP_AUTO) {
+      // six scattered blocks of a few KiB: far under the extent size that pays for the copy engines
+      if (kvc_last_launch_info(KVC_LAUNCH_SWAP_MODE) != KVC_SWAP_DIRECT) {
+        std::fprintf(stderr, "KVC_SWAP_AUTO took mode %lld for small scattered extents\n",
+                     (long long)kvc_last_launch_info(KVC_LAUNCH_SWAP_MODE));
+        ++fails;
+      }
+      KVC_OK_OR_DIE(kvc_set_tuning("auto_min_extent_bytes", 1));  // from here on every call is staged
+    }
     KVC_OK_OR_DIE(kvc_swap_in(d_pool, host, in_src.data(), in_dst.data(), 3, L, layer_elems * E,
                               blk_bytes, nb, nhb, 0, L, staging, staging_bytes, mode, stream, copy_stream));
     HIP_OK(hipStreamSynchronize(stream));
     oracle_load_blocks_from_host(want.data(), want_host.data(), in_src.data(), in_dst.data(), 3, L, nb,
                                  blk_bytes, 0, L);
     HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
-    expect_equal(mode ? "kvc_swap_in (direct) == oracle" : "kvc_swap_in (staged) == oracle", got.data(),
-                 want.data(), pool_bytes);
+    expect_equal(("kvc_swap_in" + tag + " == oracle").c_str(), got.data(), want.data(), pool_bytes);
+    if (mode == KVC_SWAP_AUTO && kvc_last_launch_info(KVC_LAUNCH_SWAP_MODE) != KVC_SWAP_STAGED) {
+      std::fprintf(stderr, "KVC_SWAP_AUTO did not take the staged path with the threshold at one byte\n");
+      ++fails;
+    }
     // the same ids checked and uploaded once, then one call per layer
     {
       std::vector<int64_t> p_gpu = {1, 46, 22, 9}, p_host = {1, 5, 7, 8};
@@ -313,9 +326,8 @@ int main() {
       HIP_OK(hipStreamSynchronize(stream));
       oracle_save_blocks_to_host(want.data(), want_host.data(), p_gpu.data(), p_host.data(), 4, L, nb,
                                  blk_bytes, 0, L);
-      expect_equal(mode ? "kvc_swap_out_prepared per layer (direct) == oracle"
-                        : "kvc_swap_out_prepared per layer (staged) == oracle",
-                   host, want_host.data(), host_bytes);
+      expect_equal(("kvc_swap_out_prepared per layer" + tag + " == oracle").c_str(), host, want_host.data(),
+                   host_bytes);
       std::vector<int64_t> q_gpu = {33, 34, 35, 2};
       KVC_OK_OR_DIE(kvc_swap_prepare(q_gpu.data(), p_host.data(), 4, nb, nhb, staging, staging_bytes, stream));
       for (int64_t l = L; l-- > 0;)
@@ -326,9 +338,8 @@ int main() {
       oracle_load_blocks_from_host(want.data(), want_host.data(), p_host.data(), q_gpu.data(), 4, L, nb,
                                    blk_bytes, 0, L);
       HIP_OK(hipMemcpy(got.data(), d_pool, pool_bytes, hipMemcpyDeviceToHost));
-      expect_equal(mode ? "kvc_swap_in_prepared per layer (direct) == oracle"
-                        : "kvc_swap_in_prepared per layer (staged) == oracle",
-                   got.data(), want.data(), pool_bytes);
+      expect_equal(("kvc_swap_in_prepared per layer" + tag + " == oracle").c_str(), got.data(), want.data(),
+                   pool_bytes);
       std::vector<int64_t> bad_gpu = {nb};
       if (kvc_swap_prepare(bad_gpu.data(), p_host.data(), 1, nb, nhb, staging, staging_bytes, stream) !=
           KVC_ERR_OUT_OF_RANGE) {
@@ -345,6 +356,7 @@ int main() {
     HIP_OK(hipStreamDestroy(copy_stream));
     HIP_OK(hipFree(staging));
     KVC_OK_OR_DIE(kvc_host_free_pinned(host));
+    KVC_OK_OR_DIE(kvc_reset_tuning());
   }
 
   // 5b. the swap that allocates nothing: same result as the direct swap, no workspace argument
