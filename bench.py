@@ -143,6 +143,40 @@ def entry(name, bytes_per_call, ms_wall, ms_event, calls_per_step=1, **extra):
     return d
 
 
+def settle_copy_engines(torch, dev, what, quiet_s=8.0, limit_s=20.0):
+    """For some seconds after a large device allocation has been freed (128 GiB:
+    under 8 s on MI355X), transfers that hand over between a kernel and a copy
+    engine several times per call run at half their rate (the staged swap-in at
+    29 instead of 54 GB/s), while kernels and plain back-to-back copies keep
+    theirs; waiting is what ends it, wherever the wait sits, so it is taken to be
+    the driver working through the freed memory. The bench frees pools of tens of
+    GiB between its sections, a serving process does not: let that time pass, then
+    check that plain pinned copies run at a steady rate, before timing anything
+    that uses the engines."""
+    t_start = time.perf_counter()
+    torch.cuda.synchronize()
+    time.sleep(quiet_s)
+    h = torch.empty(128 << 20, dtype=torch.uint8, pin_memory=True)
+    d = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    rates = []
+    while time.perf_counter() - t_start < quiet_s + limit_s:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        h.copy_(d, non_blocking=True)
+        d.copy_(h, non_blocking=True)
+        torch.cuda.synchronize()
+        rates.append(2 * h.numel() / (time.perf_counter() - t0) / 1e9)
+        last = rates[-4:]
+        steady = len(last) == 4 and min(last) >= 0.97 * max(rates)
+        # a PCIe Gen5 x16 link gives 55-57 GB/s; on a slower link, steady for 10 s is enough
+        if steady and (rates[-1] >= 45.0 or time.perf_counter() - t_start >= quiet_s + 10.0):
+            break
+    waited = time.perf_counter() - t_start
+    log(f"waited {waited:.1f} s before {what}; plain pinned copies then: {len(rates)} probes, "
+        f"{min(rates):.1f} -> {rates[-1]:.1f} GB/s")
+    return waited
+
+
 def alloc_pool(torch, shape_cfg, num_blocks, dev):
     """[L, nb, 2, bs, H, D] bf16; drops layers if HBM cannot hold all of them."""
     L = shape_cfg.num_layers
@@ -1014,6 +1048,8 @@ def main():
         extra.append(entry(f"cfg5 scatter stage, HBM only (dense buffer -> {n} blocks x {L5} layers x 64 KiB)",
                            2 * nbytes, ms_w, ms_e, launch="eager"))
         del dense
+        torch.cuda.empty_cache()
+        settle_copy_engines(torch, dev, "the swap rows")
         worker = kvc.KVWorker(pool5, n)
         try:
             def timed_sync(fn, reps):
@@ -1132,11 +1168,13 @@ def main():
         torch.cuda.empty_cache()
     if "overlap" in ops:
         try:
+            settle_copy_engines(torch, dev, "the write-through rows")
             extra += bench_write_through_overlap(torch, kvc, wl, dev)
         except Exception as exc:
             log(f"write-through overlap skipped: {exc!r}")
     if "twoproc" in ops:
         try:
+            settle_copy_engines(torch, dev, "the two-process rows")
             extra += bench_two_process_swap(torch, kvc, wl, dev)
         except Exception as exc:   # a second process is optional equipment of the bench
             log(f"two-process swap skipped: {exc!r}")
@@ -1158,6 +1196,7 @@ def main():
         n = min(4096, args.swap_blocks * 4, nbs // 2)
         old, host_ids, new = wl.swap_round_trip(nbs, n, seed=0)
         nbytes = n * Ls * sh.block_bytes
+        settle_copy_engines(torch, dev, "the shard's swap rows")
         worker = kvc.KVWorker(pool_s, n)
         try:
             for mode in ("staged", "direct"):
