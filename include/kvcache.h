@@ -315,8 +315,12 @@ int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pair
  * the buffer holds the id lists only. The staged PCIe copies follow the runs of
  * consecutive host ids in the order given: a caller that sorts the pairs of a
  * call by host id gets the longest runs. Kernels run on kernel_stream, PCIe
- * copies on copy_stream (may equal kernel_stream: then nothing overlaps; a
- * staged call of one chunk uses kernel_stream for both). On return all
+ * copies on copy_stream. Pass the same stream for both unless measured
+ * otherwise: the gather or scatter of a chunk takes a hundredth of its PCIe
+ * time, so two streams gain 1 % at best, and late in a busy process (graphs
+ * captured, many streams) the event-ordered pipeline fell to a quarter of the
+ * link rate where one stream kept all of it (a staged call of one chunk uses
+ * kernel_stream for both in any case). On return all
  * work is enqueued and kernel_stream has been made to wait for copy_stream's
  * part, so synchronising kernel_stream alone completes the swap.
  * ------------------------------------------------------------------------- */

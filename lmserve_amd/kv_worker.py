@@ -8,8 +8,12 @@ behaviour (kv_worker.py:336-346), and the per-entry semantics
   Host->GPU: gpu[l, dst_block_id] = host[src_block_id, l]   (kv_worker.py:197-211)
 Where the reference issues one driver memcpy per (layer, block), this engine
 hands the whole mapping list to libkvcache (`kvc_swap_out` / `kvc_swap_in`):
-a gather/scatter kernel plus large PCIe extents on a second stream, or one
-kernel that addresses the mapped host pool directly.
+a gather/scatter kernel plus large PCIe extents carried by the copy engines,
+or one kernel that addresses the mapped host pool directly. Both legs of a
+staged call run on the direction's own stream (the reference's two dedicated
+streams, kv_worker.py:159-160): splitting kernel and copy over two streams
+tied by events gained 1 % at best and lost up to three quarters of the rate
+late in a busy process.
 
 A copy that runs layer by layer (the reference's protocol with the model's
 forward pass) flattens, checks and uploads its id lists once
@@ -142,7 +146,6 @@ class PreparedSwap:
     host_ids: np.ndarray           # kept alive: the staged mode reads it per call
     staging: torch.Tensor          # head: [gpu_ids | host_ids] on the device
     stream: torch.cuda.Stream
-    copy_stream: torch.cuda.Stream
 
 
 class KVWorker:
@@ -235,8 +238,6 @@ class KVWorker:
         with torch.cuda.device(self.device):
             self.dtoh_stream = torch.cuda.Stream()
             self.htod_stream = torch.cuda.Stream()
-            self._dtoh_copy_stream = torch.cuda.Stream()
-            self._htod_copy_stream = torch.cuda.Stream()
         self._staging = {"out": None, "in": None}
         self.kv_worker_handle = kv_worker_handle
 
@@ -266,7 +267,7 @@ class KVWorker:
         return buf
 
     def _swap(self, direction: str, src: np.ndarray, dst: np.ndarray, layer_begin: int,
-              layer_end: int, stream: torch.cuda.Stream, copy_stream: torch.cuda.Stream) -> None:
+              layer_end: int, stream: torch.cuda.Stream) -> None:
         n = int(src.shape[0])
         if n == 0 or layer_end <= layer_begin:
             return
@@ -282,13 +283,12 @@ class KVWorker:
             staging = self._staging_for(direction, n, layer_end - layer_begin)
             # the staging buffer may have been allocated on another stream
             staging.record_stream(stream)
-            staging.record_stream(copy_stream)
             fn = _lib.lib().kvc_swap_out if direction == "out" else _lib.lib().kvc_swap_in
             _lib.check(fn(self.gpu_kv_caches.data_ptr(), self._host_pool.ptr,
                           src.ctypes.data, dst.ctypes.data, n, self.num_layers, self.layer_stride,
                           self.block_stride, self.num_gpu_blocks, self.num_host_blocks,
                           layer_begin, layer_end, staging.data_ptr(), staging.numel(),
-                          SWAP_MODES[self.swap_mode], stream.cuda_stream, copy_stream.cuda_stream))
+                          SWAP_MODES[self.swap_mode], stream.cuda_stream, stream.cuda_stream))
 
     def save_kv_blocks_to_host_nowait(self, block_mappings: Sequence[BlockMapping],
                                       stream: Optional[torch.cuda.Stream] = None,
@@ -298,7 +298,7 @@ class KVWorker:
             return
         src, dst = flatten_block_mappings(block_mappings)
         self._swap("out", src, dst, layer_begin, self.num_layers if layer_end is None else layer_end,
-                   stream or self.dtoh_stream, self._dtoh_copy_stream)
+                   stream or self.dtoh_stream)
 
     def load_kv_blocks_from_host_nowait(self, block_mappings: Sequence[BlockMapping],
                                         stream: Optional[torch.cuda.Stream] = None,
@@ -308,7 +308,7 @@ class KVWorker:
             return
         src, dst = flatten_block_mappings(block_mappings)
         self._swap("in", src, dst, layer_begin, self.num_layers if layer_end is None else layer_end,
-                   stream or self.htod_stream, self._htod_copy_stream)
+                   stream or self.htod_stream)
 
     # ------------------------------------------------- layer by layer, ids uploaded once
     def prepare_swap(self, direction: str, block_mappings: Sequence[BlockMapping],
@@ -328,17 +328,15 @@ class KVWorker:
         gpu_ids, host_ids = order_by_host_id(*((src, dst) if direction == "out" else (dst, src)))
         if stream is None:
             stream = self.dtoh_stream if direction == "out" else self.htod_stream
-        copy_stream = self._dtoh_copy_stream if direction == "out" else self._htod_copy_stream
         with torch.cuda.device(self.device):
             stream.wait_stream(torch.cuda.current_stream(self.device))
             # room for one layer per call and for the whole range in one call
             staging = self._staging_for(direction, n, 1, self.num_layers)
             staging.record_stream(stream)
-            staging.record_stream(copy_stream)
             _lib.check(_lib.lib().kvc_swap_prepare(
                 gpu_ids.ctypes.data, host_ids.ctypes.data, n, self.num_gpu_blocks,
                 self.num_host_blocks, staging.data_ptr(), staging.numel(), stream.cuda_stream))
-        return PreparedSwap(direction, n, host_ids, staging, stream, copy_stream)
+        return PreparedSwap(direction, n, host_ids, staging, stream)
 
     def swap_prepared_layers(self, prepared: Optional["PreparedSwap"], layer_begin: int,
                              layer_end: int) -> None:
@@ -354,7 +352,7 @@ class KVWorker:
                           self.layer_stride, self.block_stride, self.num_gpu_blocks,
                           self.num_host_blocks, layer_begin, layer_end, prepared.staging.data_ptr(),
                           prepared.staging.numel(), SWAP_MODES[self.swap_mode],
-                          prepared.stream.cuda_stream, prepared.copy_stream.cuda_stream))
+                          prepared.stream.cuda_stream, prepared.stream.cuda_stream))
 
     async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
                                      stream: torch.cuda.Stream) -> None:
