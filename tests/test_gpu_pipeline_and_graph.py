@@ -23,7 +23,7 @@ def _busy(dev, n=3):
     return a
 
 
-@pytest.mark.parametrize("mode", ["direct", "staged"])
+@pytest.mark.parametrize("mode", ["direct", "staged", "auto"])
 @pytest.mark.parametrize("sync", ["events", "host"])
 def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync):
     """GPU->Host runs concurrently with the forward pass; layer l may be saved
@@ -82,7 +82,7 @@ def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync):
         handle.close()
 
 
-@pytest.mark.parametrize("mode", ["direct", "staged"])
+@pytest.mark.parametrize("mode", ["direct", "staged", "auto"])
 @pytest.mark.parametrize("sync", ["events", "host"])
 def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode, sync):
     """Host->GPU: the model waits per layer on pre_events[l] (after the doorbell;
