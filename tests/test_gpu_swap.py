@@ -273,6 +273,38 @@ def test_staged_swap_of_a_layer_range_with_runs_of_consecutive_host_ids(gpu, chu
         w.close()
 
 
+@pytest.mark.parametrize("mode", MODES)
+def test_both_directions_at_once_on_disjoint_blocks(gpu, mode):
+    """Write-through of one set of blocks while another set is fetched, each on
+    the worker's stream of its direction and both in flight together (the
+    reference's two dedicated streams, kv_worker.py:159-160): every byte of both
+    pools must be what the oracle leaves, whichever transfer runs first."""
+    s = wl.LLAMA_3_8B
+    L, nb, nhb, n = 6, 96, 64, 20
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, mode, chunk=3, seed=51)
+    try:
+        rng = np.random.default_rng(52)
+        perm = rng.permutation(nb)
+        out_gpu, in_gpu = perm[:n].astype(np.int64), perm[n:2 * n].astype(np.int64)
+        hperm = rng.permutation(nhb)
+        out_host = np.sort(hperm[:n]).astype(np.int64)            # the blocks being saved
+        in_host = hperm[n:2 * n].astype(np.int64)                 # the blocks being fetched: disjoint from them
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        host_np = w.host_kv_caches.copy()
+        orc.c_save_blocks_to_host(gpu_np, host_np, out_gpu, out_host)
+        orc.c_load_blocks_from_host(gpu_np, host_np, in_host, in_gpu)
+        for _ in range(3):                                        # again and again onto the same state: idempotent
+            w.save_kv_blocks_to_host_nowait(_mappings(out_gpu, out_host))
+            w.load_kv_blocks_from_host_nowait(_mappings(in_host, in_gpu))
+        w.dtoh_stream.synchronize()
+        w.htod_stream.synchronize()
+        assert np.array_equal(w.host_kv_caches, host_np)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+    finally:
+        w.close()
+
+
 def test_auto_mode_takes_the_copy_engines_for_long_runs_and_the_kernel_for_scattered_blocks(gpu):
     """"auto" decides per call from the host ids: runs of consecutive host blocks
     whose PCIe extents reach the threshold go through the staging ring, scattered
