@@ -305,6 +305,64 @@ def test_both_directions_at_once_on_disjoint_blocks(gpu, mode):
         w.close()
 
 
+def test_seeded_random_swaps_match_the_oracle(gpu):
+    """Forty seeded cases over what a call can vary: number of blocks, layer range,
+    shape of the host id list (runs, singles, shuffled, reversed), ring size and
+    mode, in both directions on the same worker one after the other."""
+    from lmserve_amd import _lib
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb = 5, 80, 48
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    rng = np.random.default_rng(61)
+    pool = random_pool((L, nb) + block_shape, 62)
+    dpool = to_bf16(pool, gpu)
+    gpu_np = pool.reshape(L, nb, -1).copy()
+    try:
+        for case in range(40):
+            mode = MODES[case % 3]
+            chunk = int(rng.choice([0, 1, 2, 5]))
+            w = kvc.KVWorker(dpool, nhb, swap_mode=mode, staging_chunk_blocks=chunk)
+            try:
+                _lib.set_tuning("auto_min_extent_bytes", int(rng.choice([1, 64 << 10, 4 << 20])))
+                w.host_kv_caches[...] = sentinel_pool(w.host_kv_caches.shape, 100 + case)
+                host_np = w.host_kv_caches.copy()
+                n = int(rng.integers(1, 24))
+                lb = int(rng.integers(0, L))
+                le = int(rng.integers(lb + 1, L + 1))
+                kind = case % 4
+                if kind == 0:                                    # one run, somewhere in the pool
+                    start = int(rng.integers(0, nhb - n + 1))
+                    host_ids = np.arange(start, start + n)
+                elif kind == 1:                                  # scattered singles
+                    host_ids = rng.permutation(nhb)[:n]
+                elif kind == 2:                                  # a run handed over in reverse
+                    start = int(rng.integers(0, nhb - n + 1))
+                    host_ids = np.arange(start, start + n)[::-1]
+                else:                                            # runs of three with gaps
+                    host_ids = np.sort(rng.permutation(nhb // 4)[:(n + 2) // 3])[:, None] * 4 + np.arange(3)[None, :]
+                    host_ids = host_ids.reshape(-1)[:n]
+                host_ids = np.ascontiguousarray(host_ids, dtype=np.int64)
+                n = len(host_ids)
+                perm = rng.permutation(nb)
+                old, new = perm[:n].astype(np.int64), perm[n:2 * n].astype(np.int64)
+                tag = f"case {case}: {mode}, chunk {chunk}, n {n}, layers [{lb}, {le}), host ids {host_ids.tolist()}"
+                orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids, lb, le)
+                w.save_kv_blocks_to_host_nowait(_mappings(old, host_ids, pieces=2), layer_begin=lb, layer_end=le)
+                w.dtoh_stream.synchronize()
+                assert np.array_equal(w.host_kv_caches, host_np), tag
+                orc.c_load_blocks_from_host(gpu_np, host_np, host_ids, new, lb, le)
+                prepared = w.prepare_swap("in", _mappings(host_ids, new, pieces=2))
+                for l in range(lb, le):                          # layer by layer, as the protocol does
+                    w.swap_prepared_layers(prepared, l, l + 1)
+                w.htod_stream.synchronize()
+                assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np), tag
+                assert np.array_equal(w.host_kv_caches, host_np), tag
+            finally:
+                w.close()
+    finally:
+        _lib.reset_tuning()
+
+
 def test_auto_mode_takes_the_copy_engines_for_long_runs_and_the_kernel_for_scattered_blocks(gpu):
     """"auto" decides per call from the host ids: runs of consecutive host blocks
     whose PCIe extents reach the threshold go through the staging ring, scattered
