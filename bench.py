@@ -540,6 +540,7 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
         def forward():
             with torch.cuda.stream(model_stream):
                 for l in range(L):
+                    hooks.pre(l)
                     for _ in range(4):
                         torch.mm(a, b, out=c)
                     plan.append(key[l], value[l], pool[l])
@@ -591,6 +592,43 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
                         "both_done_after_ms": round(total, 2),
                         "one_after_the_other_ms": round(fwd_alone + swap_alone, 2),
                         "pcie_gbps_alone": round(nbytes / swap_alone / 1e6, 2),
+                        "bytes_per_call": int(nbytes)})
+            # the other half of the protocol (kv_worker.py:249-270, model_worker.py:254-263): the
+            # blocks of a request come back from the host layer by layer, and the model's layer l
+            # waits for "layer l landed" before it runs
+            in_maps = [kvc.BlockMapping.from_pairs(zip(range(n), rng_ids.tolist()))]
+            prepared_in = worker.prepare_swap("in", in_maps)
+            fetch_alone = None
+            for _ in range(4):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for l in range(L):
+                    worker.swap_prepared_layers(prepared_in, l, l + 1)
+                worker.htod_stream.synchronize()
+                t = (time.perf_counter() - t0) * 1e3
+                fetch_alone = t if fetch_alone is None else min(fetch_alone, t)
+
+            def kv_fetch_thread():
+                asyncio.run(worker.copy_kv(in_maps, kvc.Device.Host, kvc.Device.GPU))
+
+            hooks.enable_wait_before_execute = True
+            hooks.timeout = 60
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            th = threading.Thread(target=kv_fetch_thread)
+            th.start()
+            e0, e1 = timed_forward()
+            th.join(timeout=120)
+            torch.cuda.synchronize()
+            total = (time.perf_counter() - t0) * 1e3
+            hooks.enable_wait_before_execute = False
+            out.append({"name": f"fetch during a stand-in forward pass ({mode} swap; {L} layers; {n} blocks x {L} "
+                                f"layers x 64 KiB loaded layer by layer, each layer of the model waits for its own)",
+                        "forward_alone_ms": round(fwd_alone, 2), "fetch_alone_ms": round(fetch_alone, 2),
+                        "forward_behind_the_fetch_ms": round(e0.elapsed_time(e1), 2),
+                        "both_done_after_ms": round(total, 2),
+                        "one_after_the_other_ms": round(fwd_alone + fetch_alone, 2),
+                        "pcie_gbps_alone": round(nbytes / fetch_alone / 1e6, 2),
                         "bytes_per_call": int(nbytes)})
         finally:
             worker.close()
