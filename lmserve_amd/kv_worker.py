@@ -88,6 +88,15 @@ def flatten_block_mappings(block_mappings: Sequence[BlockMapping]) -> Tuple[np.n
     return np.asarray(src, dtype=np.int64), np.asarray(dst, dtype=np.int64)
 
 
+def check_distinct_destinations(dst_ids: np.ndarray, what: str) -> None:
+    """Raise `ValueError` if a block id occurs twice among the destinations of one call."""
+    if dst_ids.size > 1:
+        ids, counts = np.unique(dst_ids, return_counts=True)
+        if ids.size != dst_ids.size:
+            twice = ids[counts > 1][:8].tolist()
+            raise ValueError(f"{what}: destination block ids {twice} occur more than once in one call")
+
+
 def order_by_host_id(gpu_ids: np.ndarray, host_ids: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
     """The pairs of one swap call in ascending order of their host block id
     (stable), so that host blocks which lie next to each other in the pool are
@@ -179,6 +188,11 @@ class KVWorker:
       alignment and the file system allow, and spreads block extents over this
       many threads (the reference copies rows through a memory map on 4);
       `disk_preallocate` reserves a new file's blocks when it is made.
+    validate: check on the host that no block is the destination of two pairs of
+      one GPU<->Host call (`ValueError`). The reference copies the pairs one
+      after the other, so the later pair wins there (kv_worker.py:197-227);
+      here the pairs of a call move concurrently and such a call has no defined
+      result. Off by default: the scheduler hands out distinct blocks.
     """
 
     def __init__(
@@ -193,6 +207,7 @@ class KVWorker:
         disk_direct_io: bool = True,
         disk_threads: int = 8,
         disk_preallocate: bool = False,
+        validate: bool = False,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -216,6 +231,7 @@ class KVWorker:
         self.layer_stride = num_gpu_blocks * self.block_stride
         self.swap_mode = swap_mode
         self.staging_chunk_blocks = int(staging_chunk_blocks)
+        self.validate = bool(validate)
 
         self._host_pool = PinnedHostPool((self.num_host_blocks, num_layers, block_elems), np_dtype)
         self.host_kv_caches = self._host_pool.array
@@ -273,6 +289,8 @@ class KVWorker:
             return
         src = np.ascontiguousarray(src, dtype=np.int64)
         dst = np.ascontiguousarray(dst, dtype=np.int64)
+        if self.validate:
+            check_distinct_destinations(dst, "GPU->Host" if direction == "out" else "Host->GPU")
         if direction == "out":
             src, dst = order_by_host_id(src, dst)
         else:
@@ -325,6 +343,8 @@ class KVWorker:
         n = int(src.shape[0])
         if n == 0:
             return None
+        if self.validate:
+            check_distinct_destinations(dst, "GPU->Host" if direction == "out" else "Host->GPU")
         gpu_ids, host_ids = order_by_host_id(*((src, dst) if direction == "out" else (dst, src)))
         if stream is None:
             stream = self.dtoh_stream if direction == "out" else self.htod_stream

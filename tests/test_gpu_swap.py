@@ -305,6 +305,29 @@ def test_both_directions_at_once_on_disjoint_blocks(gpu, mode):
         w.close()
 
 
+def test_validating_worker_refuses_two_pairs_with_one_destination(gpu):
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb = 2, 16, 8
+    pool = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), 71)
+    dpool = to_bf16(pool, gpu)
+    w = kvc.KVWorker(dpool, nhb, validate=True)
+    try:
+        w.host_kv_caches[...] = sentinel_pool(w.host_kv_caches.shape, 72)
+        before_host = w.host_kv_caches.copy()
+        with pytest.raises(ValueError, match="GPU->Host: destination block ids \\[3\\]"):
+            w.copy_kv_sync(_mappings(np.asarray([1, 2, 5]), np.asarray([3, 0, 3]), pieces=1),
+                           kvc.Device.GPU, kvc.Device.Host)
+        with pytest.raises(ValueError, match="Host->GPU: destination block ids \\[7\\]"):
+            w.prepare_swap("in", _mappings(np.asarray([0, 1]), np.asarray([7, 7]), pieces=1))
+        torch.cuda.synchronize()
+        assert np.array_equal(w.host_kv_caches, before_host)                  # nothing ran
+        assert np.array_equal(bits_of(dpool), pool)
+        # one source fanned out to two destinations is fine
+        w.copy_kv_sync(_mappings(np.asarray([4, 4]), np.asarray([9, 10]), pieces=1), kvc.Device.Host, kvc.Device.GPU)
+    finally:
+        w.close()
+
+
 def test_seeded_random_swaps_match_the_oracle(gpu):
     """Forty seeded cases over what a call can vary: number of blocks, layer range,
     shape of the host id list (runs, singles, shuffled, reversed), ring size and

@@ -53,6 +53,14 @@ def test_pairs_of_a_swap_call_are_ordered_by_host_block_id():
     assert order_by_host_id(e, e)[1].size == 0
 
 
+def test_duplicate_destinations_of_a_swap_call_are_found():
+    from lmserve_amd.kv_worker import check_distinct_destinations
+    check_distinct_destinations(np.asarray([4, 1, 9], dtype=np.int64), "x")
+    check_distinct_destinations(np.zeros(0, dtype=np.int64), "x")
+    with pytest.raises(ValueError, match=r"Host->GPU: destination block ids \[1, 9\]"):
+        check_distinct_destinations(np.asarray([9, 1, 4, 1, 9], dtype=np.int64), "Host->GPU")
+
+
 def test_device_enum_matches_the_wire_values():
     assert (int(kvc.Device.GPU), int(kvc.Device.Host), int(kvc.Device.Disk)) == (0, 1, 2)
 
