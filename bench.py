@@ -67,6 +67,8 @@ def parse_args():
                         "translation (the config 3 launch with dense, block-run and random slots, for "
                         "address-translation counter runs; not in the default); "
                         "'none' for the headline only")
+    p.add_argument("--settle-seconds", type=float, default=8.0,
+                   help="quiet time before each section that uses the copy engines, after the bench has freed a pool")
     p.add_argument("--swap-blocks", type=int, default=8192,
                    help="blocks per swap direction; 8192 (40 GiB pinned) is config 5 at its stated size")
     p.add_argument("--pool-blocks", type=int, default=65536)
@@ -1087,7 +1089,7 @@ def main():
                            2 * nbytes, ms_w, ms_e, launch="eager"))
         del dense
         torch.cuda.empty_cache()
-        settle_copy_engines(torch, dev, "the swap rows")
+        settle_copy_engines(torch, dev, "the swap rows", args.settle_seconds)
         worker = kvc.KVWorker(pool5, n)
         try:
             def timed_sync(fn, reps):
@@ -1206,13 +1208,13 @@ def main():
         torch.cuda.empty_cache()
     if "overlap" in ops:
         try:
-            settle_copy_engines(torch, dev, "the write-through rows")
+            settle_copy_engines(torch, dev, "the write-through rows", args.settle_seconds)
             extra += bench_write_through_overlap(torch, kvc, wl, dev)
         except Exception as exc:
             log(f"write-through overlap skipped: {exc!r}")
     if "twoproc" in ops:
         try:
-            settle_copy_engines(torch, dev, "the two-process rows")
+            settle_copy_engines(torch, dev, "the two-process rows", args.settle_seconds)
             extra += bench_two_process_swap(torch, kvc, wl, dev)
         except Exception as exc:   # a second process is optional equipment of the bench
             log(f"two-process swap skipped: {exc!r}")
@@ -1234,7 +1236,7 @@ def main():
         n = min(4096, args.swap_blocks * 4, nbs // 2)
         old, host_ids, new = wl.swap_round_trip(nbs, n, seed=0)
         nbytes = n * Ls * sh.block_bytes
-        settle_copy_engines(torch, dev, "the shard's swap rows")
+        settle_copy_engines(torch, dev, "the shard's swap rows", args.settle_seconds)
         worker = kvc.KVWorker(pool_s, n)
         try:
             for mode in ("staged", "direct"):
