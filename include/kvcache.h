@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define KVC_ABI_VERSION 3
+#define KVC_ABI_VERSION 4
 
 typedef enum kvc_status {
   KVC_OK = 0,
@@ -313,8 +313,9 @@ int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pair
  * per slot, more when the call would otherwise take over 128 chunks).
  * KVC_SWAP_AUTO wants the staged size and falls back to the direct kernel when
  * the buffer holds the id lists only. The staged PCIe copies follow the runs of
- * consecutive host ids in the order given: a caller that sorts the pairs of a
- * call by host id gets the longest runs. Kernels run on kernel_stream, PCIe
+ * consecutive host ids; these two entry points order the pairs of the call by
+ * host id first (on a copy), so its host blocks form the longest runs they can.
+ * Kernels run on kernel_stream, PCIe
  * copies on copy_stream. Pass the same stream for both unless measured
  * otherwise: the gather or scatter of a chunk takes a hundredth of its PCIe
  * time, so two streams gain 1 % at best, and late in a busy process (graphs
@@ -343,6 +344,16 @@ int kvc_swap_in(void* pool, const void* host_pool,
                 void* staging, int64_t staging_bytes, int mode,
                 void* kernel_stream, void* copy_stream);
 
+/* Orders the (gpu id, host id) pairs of one swap call by ascending host block id,
+ * stably and in place (HOST arrays of n entries; no GPU work). The result of a
+ * swap does not depend on the order of its pairs (the reference copies them one
+ * after the other, runtime/worker/llm_worker/kv_worker.py:197-227, and they
+ * touch distinct blocks), but the staged PCIe leg moves one extent per run of
+ * consecutive host ids in the order given. kvc_swap_out / kvc_swap_in do this
+ * themselves on a copy of their lists (staged and auto mode); call it before
+ * kvc_swap_prepare, whose order the prepared calls keep. */
+int kvc_order_pairs_by_host_id(int64_t* gpu_ids, int64_t* host_ids, int64_t n);
+
 /* The id lists of a swap checked and uploaded ONCE, for callers that move the
  * same blocks in several calls -- the reference's layer loops issue one call per
  * layer with the same mappings (runtime/worker/llm_worker/kv_worker.py:249-295).
@@ -355,8 +366,9 @@ int kvc_swap_in(void* pool, const void* host_pool,
  *     destinations of a swap-in). Neither checks nor uploads anything; in
  *     KVC_SWAP_DIRECT mode the call is one kernel launch and host_ids may be
  *     NULL; KVC_SWAP_STAGED still needs the HOST array host_ids for its PCIe
- *     extents, and KVC_SWAP_AUTO reads it to choose (NULL: direct). The caller orders these calls after the prepare call (same
- *     stream, or an event) and keeps `staging` untouched in between.
+ *     extents, and KVC_SWAP_AUTO reads it to choose (NULL: direct). The caller
+ *     orders these calls after the prepare call (same stream, or an event) and
+ *     keeps `staging` untouched in between.
  * kvc_thread_release frees what the swap entry points keep per calling thread
  * (events, pinned id bounce buffers); it waits for that thread's pending id
  * uploads. Optional: a thread that never calls it keeps a few KiB of pinned

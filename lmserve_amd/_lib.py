@@ -47,7 +47,7 @@ KVC_LAUNCH_NON_TEMPORAL = 5
 KVC_LAUNCH_PIPE = 6
 KVC_LAUNCH_SWAP_MODE = 7
 
-KVC_ABI_VERSION = 3
+KVC_ABI_VERSION = 4
 KVC_NOALLOC_MAX_BLOCKS = 8192
 
 KVC_DTYPE_BF16 = 0
@@ -76,6 +76,7 @@ SIGNATURES = {
     "kvc_rotary_plan_run": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P, _I64, _I64, _P]),
     "kvc_rotary_plan_destroy": (c_int, [_P]),
     "kvc_rotary_plan_resolve_slots": (c_int, [_P, _P, _P]),
+    "kvc_order_pairs_by_host_id": (c_int, [_P, _P, _I64]),
     "kvc_swap_prepare": (c_int, [_P, _P, _I64, _I64, _I64, _P, _I64, _P]),
     "kvc_swap_out_prepared": (c_int, [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P,
                                       _I64, c_int, _P, _P]),

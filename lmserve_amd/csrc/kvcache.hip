@@ -37,6 +37,8 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <numeric>
+#include <vector>
 
 #include "common.h"
 #include "kvcache.h"
@@ -1231,6 +1233,32 @@ TileArgs direct_swap_tiles(bool out, char* pool, char* host_pool, const int64_t*
   return t;
 }
 
+// The pairs of one call in ascending order of their host block id (stable), in
+// place. Blocks that lie next to each other in the host pool are then next to
+// each other in the call and leave as one PCIe extent.
+int order_pairs_by_host_id(int64_t* gpu_ids, int64_t* host_ids, int64_t n) {
+  bool ascending = true;
+  for (int64_t i = 1; i < n && ascending; ++i) ascending = host_ids[i] >= host_ids[i - 1];
+  if (ascending) return KVC_OK;
+  try {
+    std::vector<int64_t> order((size_t)n);
+    std::iota(order.begin(), order.end(), int64_t(0));
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int64_t a, int64_t b) { return host_ids[a] < host_ids[b]; });
+    std::vector<int64_t> tmp((size_t)n);
+    for (int64_t i = 0; i < n; ++i) tmp[(size_t)i] = gpu_ids[order[(size_t)i]];
+    std::memcpy(gpu_ids, tmp.data(), (size_t)n * sizeof(int64_t));
+    for (int64_t i = 0; i < n; ++i) tmp[(size_t)i] = host_ids[order[(size_t)i]];
+    std::memcpy(host_ids, tmp.data(), (size_t)n * sizeof(int64_t));
+  } catch (const std::bad_alloc&) {
+    return fail(KVC_ERR_HIP, "out of host memory while ordering %lld pairs", (long long)n);
+  }
+  return KVC_OK;
+}
+
+// this thread's ordered copy of the id lists of an unprepared call: [gpu ids | host ids]
+thread_local std::vector<int64_t> g_ordered_ids;
+
 // KVC_SWAP_AUTO: the copy engines when the PCIe leg of this call is made of large
 // extents, the direct kernel when it would fall apart into small copies. The
 // engines leave the kernels of other streams alone, but every copy costs about
@@ -1253,6 +1281,25 @@ int resolve_auto_mode(const int64_t* host_ids, const SwapGeom& g, const void* st
 int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_t* gpu_ids,
              const int64_t* host_ids, const SwapGeom& g, void* staging, int64_t staging_bytes,
              int mode, bool prepared, void* kernel_stream, void* copy_stream) {
+  // An unprepared call that may go through the copy engines orders its pairs by
+  // host block id first (the result of a swap does not depend on their order):
+  // the staged PCIe leg follows the runs of consecutive host ids. A prepared
+  // call keeps the order in which kvc_swap_prepare uploaded the lists.
+  if (!prepared && mode != KVC_SWAP_DIRECT && gpu_ids && host_ids && g.n > 1) {
+    try {
+      g_ordered_ids.resize((size_t)(2 * g.n));
+    } catch (const std::bad_alloc&) {
+      return fail(KVC_ERR_HIP, "%s: out of host memory", fn);
+    }
+    int64_t* og = g_ordered_ids.data();
+    int64_t* oh = og + g.n;
+    std::memcpy(og, gpu_ids, (size_t)g.n * sizeof(int64_t));
+    std::memcpy(oh, host_ids, (size_t)g.n * sizeof(int64_t));
+    const int rc_order = order_pairs_by_host_id(og, oh, g.n);
+    if (rc_order != KVC_OK) return rc_order;
+    gpu_ids = og;
+    host_ids = oh;
+  }
   if (mode == KVC_SWAP_AUTO) mode = resolve_auto_mode(host_ids, g, staging, staging_bytes);
   g_last_swap_mode = mode;
   int64_t chunk_blocks = 0;
@@ -1803,6 +1850,13 @@ int kvc_swap_in(void* pool, const void* host_pool, const int64_t* src_ids, const
              layer_begin, layer_end};
   return run_swap("kvc_swap_in", false, (char*)pool, (char*)host_pool, dst_ids, src_ids, g, staging,
                   staging_bytes, mode, false, kernel_stream, copy_stream);
+}
+
+int kvc_order_pairs_by_host_id(int64_t* gpu_ids, int64_t* host_ids, int64_t n) {
+  if (n < 0) return fail(KVC_ERR_INVALID_ARG, "kvc_order_pairs_by_host_id: negative size");
+  if (n > 0 && (!gpu_ids || !host_ids))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_order_pairs_by_host_id: null id list");
+  return order_pairs_by_host_id(gpu_ids, host_ids, n);
 }
 
 int kvc_swap_prepare(const int64_t* gpu_ids, const int64_t* host_ids, int64_t n,

@@ -242,6 +242,25 @@ def test_plans_and_prepared_swap_validate_before_touching_the_gpu():
     assert L.kvc_thread_release() == _lib.KVC_OK       # nothing held by this thread: a no-op
 
 
+def test_pairs_are_ordered_by_host_block_id_like_a_stable_sort():
+    L = _lib.lib()
+    rng = np.random.default_rng(3)
+    for n in (0, 1, 2, 7, 1000):
+        gpu = rng.integers(0, 1 << 20, size=n).astype(np.int64)
+        host = rng.integers(0, max(1, n // 3), size=n).astype(np.int64)      # many ties
+        order = np.argsort(host, kind="stable")
+        g, h = gpu.copy(), host.copy()
+        assert L.kvc_order_pairs_by_host_id(g.ctypes.data, h.ctypes.data, n) == _lib.KVC_OK
+        assert np.array_equal(h, host[order]) and np.array_equal(g, gpu[order])
+    asc = np.asarray([0, 0, 3, 9], dtype=np.int64)
+    g = np.asarray([5, 4, 3, 2], dtype=np.int64)
+    assert L.kvc_order_pairs_by_host_id(g.ctypes.data, asc.ctypes.data, 4) == _lib.KVC_OK
+    assert g.tolist() == [5, 4, 3, 2] and asc.tolist() == [0, 0, 3, 9]       # already ascending: untouched
+    assert L.kvc_order_pairs_by_host_id(None, None, 0) == _lib.KVC_OK
+    assert L.kvc_order_pairs_by_host_id(None, asc.ctypes.data, 4) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_order_pairs_by_host_id(g.ctypes.data, asc.ctypes.data, -1) == _lib.KVC_ERR_INVALID_ARG
+
+
 def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
     """include/kvcache.h compiles as C99 with no extensions, and a C translation
     unit that only knows the header links against libkvcache.so and runs the

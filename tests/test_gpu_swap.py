@@ -305,6 +305,48 @@ def test_both_directions_at_once_on_disjoint_blocks(gpu, mode):
         w.close()
 
 
+def test_c_entry_points_order_the_pairs_of_an_unprepared_call_themselves(gpu):
+    """kvc_swap_out / kvc_swap_in called straight through the C ABI with a dense
+    range of host blocks in shuffled order: the library orders the pairs on its
+    own copy, so the call is one run, the per-call choice takes the staged path,
+    the caller's arrays stay as they were and the result is the oracle's."""
+    from lmserve_amd import _lib
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb, n = 4, 64, 32, 12
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, "auto", seed=81)
+    try:
+        _lib.set_tuning("auto_min_extent_bytes", 256 << 10)
+        rng = np.random.default_rng(82)
+        host_ids = rng.permutation(np.arange(10, 10 + n)).astype(np.int64)
+        old = rng.permutation(nb)[:n].astype(np.int64)
+        new = rng.permutation(nb)[:n].astype(np.int64)
+        keep_host, keep_old = host_ids.copy(), old.copy()
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        host_np = w.host_kv_caches.copy()
+        staging = torch.empty(int(_lib.lib().kvc_swap_staging_bytes(n, L, w.block_stride, _lib.KVC_SWAP_AUTO, 0)),
+                              dtype=torch.uint8, device=gpu)
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def call(fn, src, dst):
+            _lib.check(fn(dpool.data_ptr(), w._host_pool.ptr, src.ctypes.data, dst.ctypes.data, n, L,
+                          w.layer_stride, w.block_stride, nb, nhb, 0, L, staging.data_ptr(), staging.numel(),
+                          _lib.KVC_SWAP_AUTO, stream, stream))
+            assert _lib.last_swap_mode() == _lib.KVC_SWAP_STAGED
+            torch.cuda.synchronize()
+
+        orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids)
+        call(_lib.lib().kvc_swap_out, old, host_ids)
+        assert np.array_equal(w.host_kv_caches, host_np)
+        assert np.array_equal(host_ids, keep_host) and np.array_equal(old, keep_old)
+        orc.c_load_blocks_from_host(gpu_np, host_np, host_ids, new)
+        call(_lib.lib().kvc_swap_in, host_ids, new)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+    finally:
+        _lib.reset_tuning()
+        w.close()
+
+
 def test_validating_worker_refuses_two_pairs_with_one_destination(gpu):
     s = wl.LLAMA_3_2_1B
     L, nb, nhb = 2, 16, 8
