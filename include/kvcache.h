@@ -55,7 +55,7 @@ typedef enum kvc_swap_mode {
   KVC_SWAP_DIRECT = 1, /* one kernel that loads/stores the pinned host pool
                           through its device mapping (no staging traffic)       */
   KVC_SWAP_AUTO = 2    /* per call: staged when the host ids of the call form
-                          runs that make the PCIe copies 4 MiB or more in the
+                          runs that make the PCIe copies 1 MiB or more in the
                           mean (knob auto_min_extent_bytes), direct otherwise,
                           and direct when `staging` holds no ring               */
 } kvc_swap_mode;

@@ -88,10 +88,14 @@ struct Tuning {
                             // with 48-64 workgroups (more cost a 16 MiB one-layer launch 2-4 %),
                             // both directions at once want 96 or more each (91-92 against 87 GB/s
                             // in sum); the rest of the GPU stays free for the model
-  int auto_min_extent_bytes = 4 << 20;  // KVC_SWAP_AUTO: mean bytes per PCIe copy from which a call
-                                        // goes through the copy engines (a copy costs about 10 us
-                                        // beyond its transfer time: 88 % of the link rate at 4 MiB,
-                                        // 48 % at 512 KiB, 11 % at 64 KiB)
+  int auto_min_extent_bytes = 1 << 20;  // KVC_SWAP_AUTO: mean bytes per PCIe copy from which a call
+                                        // goes through the copy engines. A copy costs about 10 us
+                                        // beyond its transfer time (65 % of the link rate at 1 MiB,
+                                        // 88 % at 4 MiB, 11 % at 64 KiB), but what the choice is for
+                                        // is the forward pass beside it: one-layer calls of 1, 2, 4
+                                        // and 8 MiB behind a 13 ms forward pass lengthen it by 5, 10,
+                                        // 18 and 34 % through the direct kernel and by 1-6 % (8 MiB:
+                                        // 20 %) through the engines
 };
 Tuning g_tune;
 
@@ -119,7 +123,7 @@ Knob* knobs(int* count) {
       {"write_planes_threads", &g_tune.write_planes_threads, 0},
       {"write_pipe", &g_tune.write_pipe, -1},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 96},
-      {"auto_min_extent_bytes", &g_tune.auto_min_extent_bytes, 4 << 20},
+      {"auto_min_extent_bytes", &g_tune.auto_min_extent_bytes, 1 << 20},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
   };

@@ -174,7 +174,7 @@ class KVWorker:
       rate whatever the ids are; but while that kernel runs, kernels of other
       streams are held back (a stream of short GEMMs stands still beside a
       direct swap-out, measured on MI355X). "auto" (default): per call, staged
-      when the call's extents are 4 MiB or more in the mean, else direct. The
+      when the call's extents are 1 MiB or more in the mean, else direct. The
       mappings of a call are sorted by host block id first (their order does not
       matter to the result), so a call's host blocks form the longest runs they
       can.

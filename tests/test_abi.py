@@ -161,7 +161,7 @@ def test_tuning_knobs_read_back_and_reset():
     defaults = {"copy_unroll": 0, "gather_unroll": 0, "copy_nt": 1, "copy_max_wgs": 0, "copy_order": 0,
                 "write_vpt": 0, "write_nt": 1, "write_order": 0, "write_threads": 0, "write_planes": 1,
                 "write_planes_vpt": 0, "write_planes_min_bytes": 256 << 10, "write_planes_max_vpr": 256, "write_planes_threads": 0,
-                "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 4 << 20, "rope_threads": 0, "disk_bounce_mib": 4}
+                "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 1 << 20, "rope_threads": 0, "disk_bounce_mib": 4}
     for key, value in defaults.items():
         assert _lib.get_tuning(key) == value, key
     for i, key in enumerate(defaults):

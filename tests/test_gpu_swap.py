@@ -445,7 +445,8 @@ def test_auto_mode_takes_the_copy_engines_for_long_runs_and_the_kernel_for_scatt
         ("every second host block", np.arange(0, 2 * n, 2), (0, L), 256 << 10, _lib.KVC_SWAP_DIRECT),
         ("one run, one layer, under the threshold", np.arange(4, 4 + n), (1, 2), 1 << 20, _lib.KVC_SWAP_DIRECT),
         ("one run, one layer, over the threshold", np.arange(4, 4 + n), (1, 2), 256 << 10, _lib.KVC_SWAP_STAGED),
-        ("the default threshold on a small call", np.arange(4, 4 + n), (0, L), None, _lib.KVC_SWAP_DIRECT),
+        ("the default threshold, one run of 384 KiB", np.arange(4, 4 + n), (1, 2), None, _lib.KVC_SWAP_DIRECT),
+        ("the default threshold, one run of 1.5 MiB", np.arange(4, 4 + n), (0, L), None, _lib.KVC_SWAP_STAGED),
     ]
     try:
         gpu_np = pool.reshape(L, nb, -1).copy()
