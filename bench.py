@@ -640,6 +640,76 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
     return out
 
 
+def bench_small_write_through(torch, kvc, wl, dev):
+    """Where the per-call choice between the two swap modes sits: one-layer
+    write-throughs of 1, 2, 4 and 8 MiB (16 to 128 blocks of the Llama-3-8B shape,
+    consecutive host blocks) behind the same stand-in forward pass, by how much
+    they lengthen it in each mode."""
+    import asyncio
+    import threading
+
+    import numpy as np
+
+    s8 = wl.LLAMA_3_8B
+    L, nb = s8.num_layers, 4096
+    pool = torch.empty(L, nb, 2, s8.block_size, s8.num_kv_heads, s8.head_dim, dtype=torch.bfloat16, device=dev)
+    a = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    b = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    c = torch.empty(4096, 4096, dtype=torch.bfloat16, device=dev)
+    model_stream = torch.cuda.Stream()
+    out = []
+    for n in (16, 32, 64, 128):
+        ids = np.random.default_rng(5).permutation(nb)[:n]
+        maps = [kvc.BlockMapping.from_pairs(zip(ids.tolist(), range(n)))]
+        row = {"name": f"write-through of {n * 64 // 1024} MiB per layer ({n} blocks x {L} layers) during a stand-in "
+                       f"forward pass: what it adds to the forward pass",
+               "bytes_per_call": int(n * L * s8.block_bytes)}
+        for mode in ("staged", "direct"):
+            handle = kvc.KVWorkerHandle.create(L)
+            worker = kvc.KVWorker(pool, num_host_blocks=n, swap_mode=mode, kv_worker_handle=handle)
+            hooks = kvc.LayerSyncHooks(handle)
+            try:
+                def timed_forward():
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(model_stream)
+                    with torch.cuda.stream(model_stream):
+                        for l in range(L):
+                            for _ in range(4):
+                                torch.mm(a, b, out=c)
+                            hooks.post(l)
+                    e1.record(model_stream)
+                    return e0, e1
+
+                timed_forward()
+                torch.cuda.synchronize()
+                alone, beside = [], []
+                for _ in range(3):
+                    e0, e1 = timed_forward()
+                    torch.cuda.synchronize()
+                    alone.append(e0.elapsed_time(e1))
+                for _ in range(3):
+                    hooks.enable_record_after_execute = True
+                    th = threading.Thread(
+                        target=lambda: asyncio.run(worker.copy_kv(maps, kvc.Device.GPU, kvc.Device.Host)))
+                    torch.cuda.synchronize()
+                    th.start()
+                    e0, e1 = timed_forward()
+                    th.join(timeout=60)
+                    torch.cuda.synchronize()
+                    hooks.enable_record_after_execute = False
+                    beside.append(e0.elapsed_time(e1))
+                row[f"forward_alone_ms_{mode}"] = round(min(alone), 2)
+                row[f"forward_with_write_through_ms_{mode}"] = round(min(beside), 2)
+                row[f"forward_slowdown_pct_{mode}"] = round(100.0 * (min(beside) / min(alone) - 1.0), 1)
+            finally:
+                worker.close()
+                handle.close()
+        out.append(row)
+    del pool
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_two_process_swap(torch, kvc, wl, dev):
     """The reference's deployment: the KV worker is a process of its own that maps
     the pool from an IPC handle (kv_worker.py:97-160, cli.py:115-121). A pool in a
@@ -1210,6 +1280,7 @@ def main():
         try:
             settle_copy_engines(torch, dev, "the write-through rows", args.settle_seconds)
             extra += bench_write_through_overlap(torch, kvc, wl, dev)
+            extra += bench_small_write_through(torch, kvc, wl, dev)
         except Exception as exc:
             log(f"write-through overlap skipped: {exc!r}")
     if "twoproc" in ops:
