@@ -30,6 +30,7 @@ import asyncio
 import ctypes
 import enum
 import os
+import weakref
 from dataclasses import dataclass, field
 from typing import Iterable, List, Optional, Sequence, Tuple
 
@@ -254,7 +255,7 @@ class KVWorker:
         with torch.cuda.device(self.device):
             self.dtoh_stream = torch.cuda.Stream()
             self.htod_stream = torch.cuda.Stream()
-        self._staging = {"out": None, "in": None}
+        self._staging = {}   # (direction, stream handle) -> [workspace, weak reference to its PreparedSwap]
         self.kv_worker_handle = kv_worker_handle
 
         self.COPY_KV_OP_MAP = {
@@ -265,9 +266,19 @@ class KVWorker:
         }
 
     # ------------------------------------------------------------------ GPU legs
-    def _staging_for(self, direction: str, n: int, *layers_per_call: int) -> torch.Tensor:
-        """Device workspace of one direction, large enough for calls that cover
-        any of the given numbers of layers."""
+    def _staging_for(self, direction: str, stream: torch.cuda.Stream, n: int,
+                     *layers_per_call: int) -> Tuple[torch.Tensor, Optional[list]]:
+        """Device workspace for calls of one direction on one stream that cover any
+        of the given numbers of layers. Returns `(buffer, slot)`.
+
+        The head of a workspace holds the id lists of the call that uses it, so a
+        workspace serves one copy at a time. Each (direction, stream) keeps one
+        that calls reuse (work of one stream runs in order, so the next call's
+        upload comes after everything the previous call queued). While a
+        `PreparedSwap` that was given this workspace is still alive (its layers
+        may not all be queued yet), further calls get a buffer of their own:
+        `slot` is None then. Otherwise `slot` is the kept workspace's record,
+        whose owner a prepared swap sets to itself."""
         mode = SWAP_MODES[self.swap_mode]
         need = 0
         for nl in layers_per_call:
@@ -276,11 +287,18 @@ class KVWorker:
             if b < 0:
                 raise ValueError("bad swap geometry")
             need = max(need, b)
-        buf = self._staging[direction]
-        if buf is None or buf.numel() < need:
+        slot = self._staging.setdefault((direction, stream.cuda_stream), [None, None])
+        owner = slot[1]() if slot[1] is not None else None
+        if owner is not None:
             buf = torch.empty(int(need), dtype=torch.uint8, device=self.device)
-            self._staging[direction] = buf
-        return buf
+            buf.record_stream(stream)
+            return buf, None
+        slot[1] = None
+        if slot[0] is None or slot[0].numel() < need:
+            slot[0] = torch.empty(int(need), dtype=torch.uint8, device=self.device)
+        # the buffer may have been allocated with another stream current
+        slot[0].record_stream(stream)
+        return slot[0], slot
 
     def _swap(self, direction: str, src: np.ndarray, dst: np.ndarray, layer_begin: int,
               layer_end: int, stream: torch.cuda.Stream) -> None:
@@ -298,9 +316,7 @@ class KVWorker:
         with torch.cuda.device(self.device):
             # whatever the caller's current stream has queued on the pool comes first
             stream.wait_stream(torch.cuda.current_stream(self.device))
-            staging = self._staging_for(direction, n, layer_end - layer_begin)
-            # the staging buffer may have been allocated on another stream
-            staging.record_stream(stream)
+            staging, _ = self._staging_for(direction, stream, n, layer_end - layer_begin)
             fn = _lib.lib().kvc_swap_out if direction == "out" else _lib.lib().kvc_swap_in
             _lib.check(fn(self.gpu_kv_caches.data_ptr(), self._host_pool.ptr,
                           src.ctypes.data, dst.ctypes.data, n, self.num_layers, self.layer_stride,
@@ -351,12 +367,15 @@ class KVWorker:
         with torch.cuda.device(self.device):
             stream.wait_stream(torch.cuda.current_stream(self.device))
             # room for one layer per call and for the whole range in one call
-            staging = self._staging_for(direction, n, 1, self.num_layers)
-            staging.record_stream(stream)
+            staging, slot = self._staging_for(direction, stream, n, 1, self.num_layers)
             _lib.check(_lib.lib().kvc_swap_prepare(
                 gpu_ids.ctypes.data, host_ids.ctypes.data, n, self.num_gpu_blocks,
                 self.num_host_blocks, staging.data_ptr(), staging.numel(), stream.cuda_stream))
-        return PreparedSwap(direction, n, host_ids, staging, stream)
+        prepared = PreparedSwap(direction, n, host_ids, staging, stream)
+        if slot is not None:
+            # the kept workspace is this copy's until the object goes away
+            slot[1] = weakref.ref(prepared)
+        return prepared
 
     def swap_prepared_layers(self, prepared: Optional["PreparedSwap"], layer_begin: int,
                              layer_end: int) -> None:
@@ -482,7 +501,7 @@ class KVWorker:
             self.disk_tier.close()
             self.disk_tier = None
         self._host_pool.close()
-        self._staging = {"out": None, "in": None}
+        self._staging = {}
         # let go of the pool now: the direction table holds bound methods, so the
         # worker is part of a reference cycle and would otherwise keep tens of GiB
         # of HBM alive until the cycle collector runs

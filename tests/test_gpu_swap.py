@@ -305,6 +305,69 @@ def test_both_directions_at_once_on_disjoint_blocks(gpu, mode):
         w.close()
 
 
+@pytest.mark.parametrize("mode", MODES)
+def test_copies_prepared_side_by_side_keep_their_own_id_lists(gpu, mode):
+    """Two prepared swaps of one direction are alive at once (two CopyKV requests
+    whose layers interleave), an unprepared call runs between their layers, and a
+    prepared swap on a caller's own stream joins them: every copy moves its own
+    blocks, as the oracle does, whatever the order of the layer calls."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb = 6, 96, 40
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, mode, seed=91)
+    try:
+        rng = np.random.default_rng(92)
+        gperm = rng.permutation(nb).astype(np.int64)
+        hperm = rng.permutation(nhb).astype(np.int64)
+        parts = [(gperm[0:7], hperm[0:7]), (gperm[7:20], hperm[7:20]), (gperm[20:23], hperm[20:23]),
+                 (gperm[23:32], hperm[23:32])]
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        host_np = w.host_kv_caches.copy()
+        for g, h in parts:
+            orc.c_save_blocks_to_host(gpu_np, host_np, g, h)
+        side = torch.cuda.Stream()
+        a = w.prepare_swap("out", _mappings(*parts[0]))
+        b = w.prepare_swap("out", _mappings(*parts[1]))
+        c = w.prepare_swap("out", _mappings(*parts[3]), stream=side)
+        assert a.staging.data_ptr() != b.staging.data_ptr() != c.staging.data_ptr()
+        for layer in range(L):
+            w.swap_prepared_layers(b, layer, layer + 1)
+            if layer == 2:
+                w.save_kv_blocks_to_host_nowait(_mappings(*parts[2]))
+            w.swap_prepared_layers(c, layer, layer + 1)
+            w.swap_prepared_layers(a, layer, layer + 1)
+        torch.cuda.synchronize()
+        assert np.array_equal(w.host_kv_caches, host_np)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)   # pool untouched
+
+        # the same the other way, onto fresh pool blocks
+        fresh = gperm[40:72]
+        targets = [fresh[0:7], fresh[7:20], fresh[20:23], fresh[23:32]]
+        for (g, h), t in zip(parts, targets):
+            orc.c_load_blocks_from_host(gpu_np, host_np, h, t)
+        del a, b, c
+        a = w.prepare_swap("in", _mappings(parts[0][1], targets[0]))
+        b = w.prepare_swap("in", _mappings(parts[1][1], targets[1]))
+        c = w.prepare_swap("in", _mappings(parts[3][1], targets[3]), stream=side)
+        for layer in range(L):
+            w.swap_prepared_layers(a, layer, layer + 1)
+            w.swap_prepared_layers(c, layer, layer + 1)
+            if layer == 3:
+                w.load_kv_blocks_from_host_nowait(_mappings(parts[2][1], targets[2]))
+            w.swap_prepared_layers(b, layer, layer + 1)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+        assert np.array_equal(w.host_kv_caches, host_np)
+        # once the copies are gone, the kept workspace serves the next one again
+        kept = a.staging.data_ptr()
+        del a, b, c
+        d = w.prepare_swap("in", _mappings(parts[0][1], targets[0]))
+        assert d.staging.data_ptr() == kept
+        torch.cuda.synchronize()
+    finally:
+        w.close()
+
+
 def test_c_entry_points_order_the_pairs_of_an_unprepared_call_themselves(gpu):
     """kvc_swap_out / kvc_swap_in called straight through the C ABI with a dense
     range of host blocks in shuffled order: the library orders the pairs on its
