@@ -123,3 +123,87 @@ def test_random_geometry_write_copy_swap(gpu, seed):
             assert np.array_equal(_host(a, np_dtype), want), f"swap-in {mode}"
         finally:
             worker.close()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_one_and_eight_byte_elements_write_copy_gather_swap(gpu, seed):
+    """The storage widths the 16-bit cases do not reach: one byte per element (an
+    8-bit KV cache) and eight. Same operators, same oracle, bit-exact."""
+    rng = np.random.default_rng(3000 + seed)
+    width = 1 if seed % 2 == 0 else 8
+    np_dtype = np.uint8 if width == 1 else np.uint64
+    tdtype = torch.uint8 if width == 1 else torch.float64
+
+    def dev(a):
+        if width == 1:
+            return torch.from_numpy(a.copy()).to(gpu)
+        return torch.from_numpy(a.view(np.int64).copy()).view(torch.float64).to(gpu)
+
+    def host(t):
+        if width == 1:
+            return t.cpu().contiguous().numpy()
+        return t.cpu().contiguous().view(torch.int64).numpy().view(np.uint64)
+
+    L = int(rng.integers(1, 4))
+    bs = int(rng.choice([1, 3, 4, 16]))
+    H = int(rng.integers(1, 5))
+    D = int(rng.choice([1, 3, 8, 16, 48, 128, 256]))
+    nb = int(rng.integers(6, 30))
+    hi = np.iinfo(np_dtype).max
+    pool = rng.integers(0, hi, size=(L, nb, 2, bs, H, D), dtype=np_dtype)
+    n_req = int(rng.integers(1, 4))
+    filled = rng.integers(0, bs + 1, size=n_req).tolist()
+    new = rng.integers(1, bs + 2, size=n_req).tolist()
+    while sum((f + n + bs - 1) // bs for f, n in zip(filled, new)) > nb:
+        filled = [f // 2 for f in filled]
+        new = [max(1, n // 2) for n in new]
+    w = wl._write_workload(wl.KVShape("random", L, H, D, bs, width), nb, filled, new, rng)
+    idx, T = w.index, w.num_tokens
+    key = rng.integers(0, hi, size=(L, T, H, D), dtype=np_dtype)
+    value = rng.integers(0, hi, size=(L, T, H, D), dtype=np_dtype)
+    want = pool.copy()
+    for l in range(L):
+        orc.c_append_paged_kv_cache(key[l], value[l], idx.batch_indices, idx.positions, want[l],
+                                    idx.kv_block_indices, idx.kv_block_indptrs)
+    d = kvc.to_device_one_launch(w.inputs, bs, gpu)
+    dkey, dval = dev(key), dev(value)
+    assert dkey.dtype == tdtype
+    a, b, c = dev(pool), dev(pool), dev(pool)
+    for l in range(L):
+        kvc.append_paged_kv_cache(dkey[l], dval[l], d.batch_indices, d.positions, a[l],
+                                  d.kv_block_indices, d.kv_block_indptrs, d.kv_last_block_lens)
+        kvc.reshape_and_cache(dkey[l], dval[l], b[l], d.slot_mapping)
+    kvc.reshape_and_cache_layers(dkey, dval, c, d.slot_mapping.to(torch.int32))
+    torch.cuda.synchronize()
+    for name, got in (("paged per layer", a), ("slot per layer", b), ("slot one launch", c)):
+        assert np.array_equal(host(got), want), name
+
+    P = int(rng.integers(1, nb // 2 + 1))
+    flat, pairs = wl.copy_on_write_pairs(nb, P, seed=seed)
+    orc.c_copy_blocks(want, flat)
+    kvc.copy_blocks(a, pairs, validate=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(a), want), "copy_blocks"
+
+    # gather into the host layout, scatter back onto other blocks; the direct swap operators
+    n = int(rng.integers(1, nb // 2 + 1))
+    perm = rng.permutation(nb)
+    old, new_ids = perm[:n].astype(np.int64), perm[n:2 * n].astype(np.int64)
+    dense = kvc.gather_blocks(a, torch.from_numpy(old).to(gpu))
+    torch.cuda.synchronize()
+    assert np.array_equal(host(dense), want.reshape(L, nb, -1)[:, old].transpose(1, 0, 2))
+    nhb = n + 3
+    host_pool = torch.zeros(nhb, L, a[0][0].numel(), dtype=tdtype).pin_memory()
+    host_ids = rng.permutation(nhb)[:n].astype(np.int64)
+    want_host = host(host_pool).copy()
+    gpu_np = want.reshape(L, nb, -1)
+    orc.c_save_blocks_to_host(gpu_np, want_host, old, host_ids)
+    kvc.swap_out(a, host_pool, old, host_ids)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(host_pool), want_host), "swap_out"
+    orc.c_load_blocks_from_host(gpu_np, want_host, host_ids, new_ids)
+    kvc.swap_in(a, host_pool, host_ids, new_ids)
+    kvc.scatter_blocks(b, torch.from_numpy(new_ids).to(gpu), dense)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(a), want), "swap_in"
+    assert np.array_equal(host(b).reshape(L, nb, -1)[:, new_ids], want.reshape(L, nb, -1)[:, new_ids]), "scatter"
