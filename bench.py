@@ -179,6 +179,29 @@ def settle_copy_engines(torch, dev, what, quiet_s=8.0, limit_s=20.0):
     return waited
 
 
+class optional_section:
+    """A section of rows beyond the headline: if it fails, say so and go on, so
+    that the line with the headline is printed whatever happens here."""
+
+    def __init__(self, name, torch):
+        self.name, self.torch = name, torch
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is None or not issubclass(exc_type, Exception):
+            return False
+        log(f"{self.name} skipped: {exc!r}")
+        tb = None
+        try:
+            self.torch.cuda.synchronize()
+            self.torch.cuda.empty_cache()
+        except Exception as again:
+            log(f"after {self.name}: {again!r}")
+        return True
+
+
 def alloc_pool(torch, shape_cfg, num_blocks, dev):
     """[L, nb, 2, bs, H, D] bf16; drops layers if HBM cannot hold all of them."""
     L = shape_cfg.num_layers
@@ -907,375 +930,393 @@ def main():
 
     # ------------------------------------------------ rotation + write, per layer (config 2 shape)
     if "rope" in ops:
-        Hq, Hkv, D, T = 32, s8.num_kv_heads, s8.head_dim, 256
-        cs = kvc.make_cos_sin_cache(D, 8192, 500000.0, dtype=torch.bfloat16).to(dev)
-        R = ROTATE_DECODE
-        qs = [torch.randn(T, Hq * D, device=dev).to(torch.bfloat16) for _ in range(R)]
-        ks = [sets[r][1][0].reshape(T, Hkv * D) for r in range(R)]
-        vs = [sets[r][2][0].reshape(T, Hkv * D) for r in range(R)]
-        idxs = [sets[r][3] for r in range(R)]
-        pool_l = [pool[l] for l in range(L)]
-        E = 2
-        # q read+write, k read + cache write, v read + cache write, cos/sin row, indices
-        rope_bytes = T * (2 * Hq * D * E + 2 * Hkv * D * E + 2 * Hkv * D * E + 2 * D * E + 12)
+        with optional_section("rotation rows", torch):
+            Hq, Hkv, D, T = 32, s8.num_kv_heads, s8.head_dim, 256
+            cs = kvc.make_cos_sin_cache(D, 8192, 500000.0, dtype=torch.bfloat16).to(dev)
+            R = ROTATE_DECODE
+            qs = [torch.randn(T, Hq * D, device=dev).to(torch.bfloat16) for _ in range(R)]
+            ks = [sets[r][1][0].reshape(T, Hkv * D) for r in range(R)]
+            vs = [sets[r][2][0].reshape(T, Hkv * D) for r in range(R)]
+            idxs = [sets[r][3] for r in range(R)]
+            pool_l = [pool[l] for l in range(L)]
+            E = 2
+            # q read+write, k read + cache write, v read + cache write, cos/sin row, indices
+            rope_bytes = T * (2 * Hq * D * E + 2 * Hkv * D * E + 2 * Hkv * D * E + 2 * D * E + 12)
 
-        def two_launches(i):
-            r = i % R
-            idx = idxs[r]
-            for l in range(L):
-                q_o, k_o = kvc.rotary_pos_emb(qs[r], ks[r], idx.positions, cs, D)
-                kvc.append_paged_kv_cache(k_o, vs[r], idx.batch_indices, idx.positions, pool_l[l],
-                                          idx.kv_block_indices, idx.kv_block_indptrs,
-                                          idx.kv_last_block_lens)
+            def two_launches(i):
+                r = i % R
+                idx = idxs[r]
+                for l in range(L):
+                    q_o, k_o = kvc.rotary_pos_emb(qs[r], ks[r], idx.positions, cs, D)
+                    kvc.append_paged_kv_cache(k_o, vs[r], idx.batch_indices, idx.positions, pool_l[l],
+                                              idx.kv_block_indices, idx.kv_block_indptrs,
+                                              idx.kv_last_block_lens)
 
-        def fused(i):
-            r = i % R
-            idx = idxs[r]
-            for l in range(L):
-                kvc.rotary_pos_emb_and_append_paged(qs[r], ks[r], vs[r], idx.batch_indices,
-                                                    idx.positions, cs, D, pool_l[l],
-                                                    idx.kv_block_indices, idx.kv_block_indptrs,
-                                                    idx.kv_last_block_lens, return_key=False)
+            def fused(i):
+                r = i % R
+                idx = idxs[r]
+                for l in range(L):
+                    kvc.rotary_pos_emb_and_append_paged(qs[r], ks[r], vs[r], idx.batch_indices,
+                                                        idx.positions, cs, D, pool_l[l],
+                                                        idx.kv_block_indices, idx.kv_block_indptrs,
+                                                        idx.kv_last_block_lens, return_key=False)
 
-        plans = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
-                                          ix.kv_block_indptrs, ix.kv_last_block_lens, cs, Hq, Hkv, D,
-                                          s8.block_size) for ix in idxs]
-        q_buf = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=dev)
+            plans = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
+                                              ix.kv_block_indptrs, ix.kv_last_block_lens, cs, Hq, Hkv, D,
+                                              s8.block_size) for ix in idxs]
+            q_buf = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=dev)
 
-        def fused_plan(i):
-            r = i % R
-            for l in range(L):
-                plans[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
+            def fused_plan(i):
+                r = i % R
+                for l in range(L):
+                    plans[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
 
-        plans_r = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
-                                            ix.kv_block_indptrs, ix.kv_last_block_lens, cs, Hq, Hkv, D,
-                                            s8.block_size, resolve_slots=True) for ix in idxs]
+            plans_r = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
+                                                ix.kv_block_indptrs, ix.kv_last_block_lens, cs, Hq, Hkv, D,
+                                                s8.block_size, resolve_slots=True) for ix in idxs]
 
-        def fused_plan_resolved(i):
-            r = i % R
-            for l in range(L):
-                plans_r[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
+            def fused_plan_resolved(i):
+                r = i % R
+                for l in range(L):
+                    plans_r[r].run(qs[r], ks[r], vs[r], pool_l[l], query_out=q_buf)
 
-        n = max(R, args.steps // 8 // R * R)
-        for fn, label in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)"),
-                          (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)"),
-                          (fused_plan, "PagedRotaryWritePlan.run (1 launch per layer)")):
-            ms_w, ms_e = time_region(fn, n, 2, torch)
-            extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes, ms_w, ms_e,
-                               calls_per_step=L, launch="eager (one Python call per launch)"))
-        for fn, label, extra_b in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
-                                    2 * T * Hkv * D * E),   # rotated key written out and read back
-                                   (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0),
-                                   (fused_plan_resolved,
-                                    "PagedRotaryWritePlan(resolve_slots).run (1 launch per layer)", 0)):
-            try:
-                ms_w, ms_e = time_region(fn, n, 2, torch, graph_of=R)
-            except Exception as exc:
-                log(f"rope variant skipped: {exc!r}")
-                continue
-            extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes + extra_b, ms_w, ms_e,
-                               calls_per_step=L, launch="hipGraph replay"))
-        del qs, ks, vs, idxs
+            n = max(R, args.steps // 8 // R * R)
+            for fn, label in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)"),
+                              (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)"),
+                              (fused_plan, "PagedRotaryWritePlan.run (1 launch per layer)")):
+                ms_w, ms_e = time_region(fn, n, 2, torch)
+                extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes, ms_w, ms_e,
+                                   calls_per_step=L, launch="eager (one Python call per launch)"))
+            for fn, label, extra_b in ((two_launches, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
+                                        2 * T * Hkv * D * E),   # rotated key written out and read back
+                                       (fused, "rotary_pos_emb_and_append_paged (1 launch per layer)", 0),
+                                       (fused_plan_resolved,
+                                        "PagedRotaryWritePlan(resolve_slots).run (1 launch per layer)", 0)):
+                try:
+                    ms_w, ms_e = time_region(fn, n, 2, torch, graph_of=R)
+                except Exception as exc:
+                    log(f"rope variant skipped: {exc!r}")
+                    continue
+                extra.append(entry(f"cfg2 decode + rotation/{label}", rope_bytes + extra_b, ms_w, ms_e,
+                                   calls_per_step=L, launch="hipGraph replay"))
+            del qs, ks, vs, idxs
 
     # ------------------------------------------------ config 4: copy_blocks (same pool)
     if "copy" in ops:
-        maps = [torch.from_numpy(wl.copy_on_write_pairs(args.pool_blocks, 4096, seed=r)[0]).to(dev)
-                for r in range(2)]
-        nbytes = 2 * 4096 * L * s8.block_bytes + 16 * 4096
-        ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool, maps[i % 2]),
-                                 max(5, min(args.steps, 20)), 3, torch)
-        extra.append(entry(f"cfg4 copy_blocks (4096 pairs x {L} layers, 64 KiB blocks)", nbytes,
-                           ms_w, ms_e, launch="eager"))
+        with optional_section("config 4 copy_blocks row", torch):
+            maps = [torch.from_numpy(wl.copy_on_write_pairs(args.pool_blocks, 4096, seed=r)[0]).to(dev)
+                    for r in range(2)]
+            nbytes = 2 * 4096 * L * s8.block_bytes + 16 * 4096
+            ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool, maps[i % 2]),
+                                     max(5, min(args.steps, 20)), 3, torch)
+            extra.append(entry(f"cfg4 copy_blocks (4096 pairs x {L} layers, 64 KiB blocks)", nbytes,
+                               ms_w, ms_e, launch="eager"))
     # ------------------------------------------------ index preparation of a step
     if "index" in ops:
-        for tag, wk in (("cfg2 decode, 256 requests", sets[0][0]),
-                        ("cfg3 prefill chunk, 4 requests",
-                         wl.chunked_prefill(wl.QWEN_2_5_7B, num_blocks=16384, seed=0))):
-            reqs = wk.inputs
-            bs_ = wk.shape.block_size
-            n_ids = sum(len(r.block_ids) for r in reqs)
+        with optional_section("index preparation rows", torch):
+            for tag, wk in (("cfg2 decode, 256 requests", sets[0][0]),
+                            ("cfg3 prefill chunk, 4 requests",
+                             wl.chunked_prefill(wl.QWEN_2_5_7B, num_blocks=16384, seed=0))):
+                reqs = wk.inputs
+                bs_ = wk.shape.block_size
+                n_ids = sum(len(r.block_ids) for r in reqs)
 
-            def host_lists_and_uploads():
-                d = kvc.to_device(kvc.make_kv_index_inputs(reqs, bs_), bs_, dev, with_slot_mapping=False)
-                return d.positions
+                def host_lists_and_uploads():
+                    d = kvc.to_device(kvc.make_kv_index_inputs(reqs, bs_), bs_, dev, with_slot_mapping=False)
+                    return d.positions
 
-            def one_launch():
-                return kvc.to_device_one_launch(reqs, bs_, dev, with_slot_mapping=True).positions
+                def one_launch():
+                    return kvc.to_device_one_launch(reqs, bs_, dev, with_slot_mapping=True).positions
 
-            for fn, label in ((host_lists_and_uploads, "host list building + 6 uploads + 2 launches "
-                                                      "(the reference's construction)"),
-                              (one_launch, "4 packed uploads + 1 launch (slot_mapping included)")):
-                for _ in range(5):
-                    fn()
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-                reps = 30
-                for _ in range(reps):
-                    fn()
-                torch.cuda.synchronize()
-                us = (time.perf_counter() - t0) / reps * 1e6
-                extra.append({"name": f"index preparation/{tag} ({n_ids} block ids)/{label}",
-                              "wall_us_per_call": round(us, 1)})
+                for fn, label in ((host_lists_and_uploads, "host list building + 6 uploads + 2 launches "
+                                                          "(the reference's construction)"),
+                                  (one_launch, "4 packed uploads + 1 launch (slot_mapping included)")):
+                    for _ in range(5):
+                        fn()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    reps = 30
+                    for _ in range(reps):
+                        fn()
+                    torch.cuda.synchronize()
+                    us = (time.perf_counter() - t0) / reps * 1e6
+                    extra.append({"name": f"index preparation/{tag} ({n_ids} block ids)/{label}",
+                                  "wall_us_per_call": round(us, 1)})
 
     # ------------------------------------------------ launch-size sweep (8B shape, same pool)
     if "sweep" in ops:
-        extra += bench_size_sweep(torch, kvc, wl, pool, L, args.pool_blocks, dev)
+        with optional_section("launch size sweep", torch):
+            extra += bench_size_sweep(torch, kvc, wl, pool, L, args.pool_blocks, dev)
     del pool, sets
     torch.cuda.empty_cache()
 
     if "calib" in ops:
-        # a plain elementwise kernel of known size: reads 1 GiB, writes 1 GiB
-        a = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
-        b = torch.empty_like(a)
-        ms_w, ms_e = time_region(lambda i: torch.add(a, 1, out=b), 10, 2, torch)
-        extra.append(entry("calibration: plain elementwise kernel, 1 GiB read + 1 GiB written "
-                           "(torch.add(int32, 1))", 2 << 30, ms_w, ms_e, launch="eager"))
-        # write-only ceiling of the machine: a plain fill of 1 GiB
-        ms_w, ms_e = time_region(lambda i: b.fill_(3), 10, 2, torch)
-        extra.append(entry("calibration: plain fill, 1 GiB written (Tensor.fill_)", 1 << 30, ms_w, ms_e,
-                           launch="eager"))
-        del a, b
-        torch.cuda.empty_cache()
+        with optional_section("calibration rows", torch):
+            # a plain elementwise kernel of known size: reads 1 GiB, writes 1 GiB
+            a = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
+            b = torch.empty_like(a)
+            ms_w, ms_e = time_region(lambda i: torch.add(a, 1, out=b), 10, 2, torch)
+            extra.append(entry("calibration: plain elementwise kernel, 1 GiB read + 1 GiB written "
+                               "(torch.add(int32, 1))", 2 << 30, ms_w, ms_e, launch="eager"))
+            # write-only ceiling of the machine: a plain fill of 1 GiB
+            ms_w, ms_e = time_region(lambda i: b.fill_(3), 10, 2, torch)
+            extra.append(entry("calibration: plain fill, 1 GiB written (Tensor.fill_)", 1 << 30, ms_w, ms_e,
+                               launch="eager"))
+            del a, b
+            torch.cuda.empty_cache()
 
     # ------------------------------------------------ config 3: chunked-prefill write
     if "prefill" in ops:
-        sq = wl.QWEN_2_5_7B
-        pool3, L3 = alloc_pool(torch, sq, 16384, dev)
-        sets3 = write_inputs(torch, kvc, wl.chunked_prefill, sq, L3, 16384, dev, ROTATE_PREFILL)
-        e3, _ = bench_write_config(torch, kvc, "cfg3 chunked prefill", sets3, pool3, L3,
-                                   max(ROTATE_PREFILL, args.steps // 2), max(3, args.warmup // 2),
-                                   ["fused_slot:graph", "fused_paged:graph", "per_layer_paged:graph"])
-        extra += e3
-        if "rope" in ops:
-            # rotation + write per layer at the prefill chunk (28 query heads, 4 KV heads x 128)
-            Hq3, Hkv3, D3 = 28, sq.num_kv_heads, sq.head_dim
-            T3 = sets3[0][0].num_tokens
-            R3 = len(sets3)
-            cs3 = kvc.make_cos_sin_cache(D3, 65536, 1000000.0, dtype=torch.bfloat16).to(dev)
-            q3 = [torch.randn(T3, Hq3 * D3, device=dev).to(torch.bfloat16) for _ in range(R3)]
-            k3 = [sets3[r][1][0].reshape(T3, Hkv3 * D3) for r in range(R3)]
-            v3 = [sets3[r][2][0].reshape(T3, Hkv3 * D3) for r in range(R3)]
-            plans3 = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
-                                               ix.kv_block_indptrs, ix.kv_last_block_lens, cs3, Hq3,
-                                               Hkv3, D3, sq.block_size) for _, _, _, ix in sets3]
-            qo3 = torch.empty(T3, Hq3 * D3, dtype=torch.bfloat16, device=dev)
-            pool3_l = [pool3[l] for l in range(L3)]
-            bytes3 = T3 * (2 * Hq3 * D3 * 2 + 4 * Hkv3 * D3 * 2 + 2 * D3 * 2 + 12)
+        with optional_section("config 3 rows", torch):
+            sq = wl.QWEN_2_5_7B
+            pool3, L3 = alloc_pool(torch, sq, 16384, dev)
+            sets3 = write_inputs(torch, kvc, wl.chunked_prefill, sq, L3, 16384, dev, ROTATE_PREFILL)
+            e3, _ = bench_write_config(torch, kvc, "cfg3 chunked prefill", sets3, pool3, L3,
+                                       max(ROTATE_PREFILL, args.steps // 2), max(3, args.warmup // 2),
+                                       ["fused_slot:graph", "fused_paged:graph", "per_layer_paged:graph"])
+            extra += e3
+            if "rope" in ops:
+                # rotation + write per layer at the prefill chunk (28 query heads, 4 KV heads x 128)
+                Hq3, Hkv3, D3 = 28, sq.num_kv_heads, sq.head_dim
+                T3 = sets3[0][0].num_tokens
+                R3 = len(sets3)
+                cs3 = kvc.make_cos_sin_cache(D3, 65536, 1000000.0, dtype=torch.bfloat16).to(dev)
+                q3 = [torch.randn(T3, Hq3 * D3, device=dev).to(torch.bfloat16) for _ in range(R3)]
+                k3 = [sets3[r][1][0].reshape(T3, Hkv3 * D3) for r in range(R3)]
+                v3 = [sets3[r][2][0].reshape(T3, Hkv3 * D3) for r in range(R3)]
+                plans3 = [kvc.PagedRotaryWritePlan(ix.batch_indices, ix.positions, ix.kv_block_indices,
+                                                   ix.kv_block_indptrs, ix.kv_last_block_lens, cs3, Hq3,
+                                                   Hkv3, D3, sq.block_size) for _, _, _, ix in sets3]
+                qo3 = torch.empty(T3, Hq3 * D3, dtype=torch.bfloat16, device=dev)
+                pool3_l = [pool3[l] for l in range(L3)]
+                bytes3 = T3 * (2 * Hq3 * D3 * 2 + 4 * Hkv3 * D3 * 2 + 2 * D3 * 2 + 12)
 
-            def fused3(i):
-                r = i % R3
-                for l in range(L3):
-                    plans3[r].run(q3[r], k3[r], v3[r], pool3_l[l], query_out=qo3)
+                def fused3(i):
+                    r = i % R3
+                    for l in range(L3):
+                        plans3[r].run(q3[r], k3[r], v3[r], pool3_l[l], query_out=qo3)
 
-            def two3(i):
-                r = i % R3
-                ix = sets3[r][3]
-                for l in range(L3):
-                    q_o, k_o = kvc.rotary_pos_emb(q3[r], k3[r], ix.positions, cs3, D3)
-                    kvc.append_paged_kv_cache(k_o, v3[r], ix.batch_indices, ix.positions, pool3_l[l],
-                                              ix.kv_block_indices, ix.kv_block_indptrs,
-                                              ix.kv_last_block_lens)
+                def two3(i):
+                    r = i % R3
+                    ix = sets3[r][3]
+                    for l in range(L3):
+                        q_o, k_o = kvc.rotary_pos_emb(q3[r], k3[r], ix.positions, cs3, D3)
+                        kvc.append_paged_kv_cache(k_o, v3[r], ix.batch_indices, ix.positions, pool3_l[l],
+                                                  ix.kv_block_indices, ix.kv_block_indptrs,
+                                                  ix.kv_last_block_lens)
 
-            for fn, label, extra_b in ((two3, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
-                                        2 * T3 * Hkv3 * D3 * 2),
-                                       (fused3, "PagedRotaryWritePlan.run (1 launch per layer)", 0)):
-                try:
-                    ms_w, ms_e = time_region(fn, R3, 1, torch, graph_of=R3)
-                except Exception as exc:
-                    log(f"prefill rope variant skipped: {exc!r}")
-                    continue
-                extra.append(entry(f"cfg3 chunked prefill + rotation/{label}", bytes3 + extra_b, ms_w, ms_e,
-                                   calls_per_step=L3, launch="hipGraph replay"))
-            del q3, k3, v3, plans3, qo3
-        del sets3, pool3
-        torch.cuda.empty_cache()
+                for fn, label, extra_b in ((two3, "rotary_pos_emb + append_paged_kv_cache (2 launches per layer)",
+                                            2 * T3 * Hkv3 * D3 * 2),
+                                           (fused3, "PagedRotaryWritePlan.run (1 launch per layer)", 0)):
+                    try:
+                        ms_w, ms_e = time_region(fn, R3, 1, torch, graph_of=R3)
+                    except Exception as exc:
+                        log(f"prefill rope variant skipped: {exc!r}")
+                        continue
+                    extra.append(entry(f"cfg3 chunked prefill + rotation/{label}", bytes3 + extra_b, ms_w, ms_e,
+                                       calls_per_step=L3, launch="hipGraph replay"))
+                del q3, k3, v3, plans3, qo3
+            del sets3, pool3
+            torch.cuda.empty_cache()
 
     # ------------------------------------------------ config 3 launch, three slot patterns
     # (for counter runs: the same 2048-token x 28-layer launch writing one dense run per
     # layer, the workload's scattered 16-token block runs, and fully random rows; the
     # write_rows_kernel dispatches appear in that order, `reps` + 2 of each)
     if "translation" in ops:
-        sq = wl.QWEN_2_5_7B
-        nbq = 16384
-        poolq, Lq = alloc_pool(torch, sq, nbq, dev)
-        Tq, Rq, reps = 2048, ROTATE_PREFILL, max(2, min(args.steps, 64))
-        srcs = []
-        for r in range(Rq):
-            kq = torch.randn(Lq, Tq, sq.num_kv_heads, sq.head_dim, device=dev, dtype=torch.float32).to(torch.bfloat16)
-            srcs.append((kq, torch.randn_like(kq)))
-        patterns = (
-            ("one dense run per layer (slots 0..2047)",
-             [torch.arange(Tq, dtype=torch.int64, device=dev) for _ in range(Rq)]),
-            ("the workload's block runs (4 sequences x 32 scattered blocks of 16 tokens)",
-             [torch.from_numpy(wl.chunked_prefill(sq, num_blocks=nbq, seed=r).index.slot_mapping).to(dev)
-              for r in range(Rq)]),
-            ("random rows (2048 distinct random slots)",
-             [torch.from_numpy(wl.random_free_slots(sq, nbq, Tq, seed=r)).to(dev) for r in range(Rq)]),
-        )
-        nbytes = 2 * 2 * Tq * sq.row_bytes * Lq + 8 * Tq
-        rounds = 3                      # patterns interleaved, so drift hits all of them alike
-        per_pattern = {label: [] for label, _ in patterns}
-        for rnd in range(rounds):
-            for label, slot_sets in patterns:
-                for i in range(2):
-                    kvc.reshape_and_cache_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, slot_sets[i % Rq])
-                torch.cuda.synchronize()
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-                for i in range(reps):
-                    kvc.reshape_and_cache_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, slot_sets[i % Rq])
-                end.record()
-                torch.cuda.synchronize()
-                per_pattern[label].append(start.elapsed_time(end) / reps)
-                log(f"translation: round {rnd}: {reps + 2} write_rows_kernel dispatches, {label}, "
-                    f"{per_pattern[label][-1] * 1e3:.2f} us each")
-        for label, _ in patterns:
-            ms = sorted(per_pattern[label])[rounds // 2]
-            extra.append(entry(f"cfg3 launch, slot pattern: {label}", nbytes, ms, ms, launch="eager",
-                               launches_per_round=reps + 2, rounds=rounds,
-                               us_per_round=[round(x * 1e3, 2) for x in per_pattern[label]]))
-        del poolq, srcs
-        torch.cuda.empty_cache()
+        with optional_section("slot pattern rows", torch):
+            sq = wl.QWEN_2_5_7B
+            nbq = 16384
+            poolq, Lq = alloc_pool(torch, sq, nbq, dev)
+            Tq, Rq, reps = 2048, ROTATE_PREFILL, max(2, min(args.steps, 64))
+            srcs = []
+            for r in range(Rq):
+                kq = torch.randn(Lq, Tq, sq.num_kv_heads, sq.head_dim, device=dev, dtype=torch.float32).to(torch.bfloat16)
+                srcs.append((kq, torch.randn_like(kq)))
+            patterns = (
+                ("one dense run per layer (slots 0..2047)",
+                 [torch.arange(Tq, dtype=torch.int64, device=dev) for _ in range(Rq)]),
+                ("the workload's block runs (4 sequences x 32 scattered blocks of 16 tokens)",
+                 [torch.from_numpy(wl.chunked_prefill(sq, num_blocks=nbq, seed=r).index.slot_mapping).to(dev)
+                  for r in range(Rq)]),
+                ("random rows (2048 distinct random slots)",
+                 [torch.from_numpy(wl.random_free_slots(sq, nbq, Tq, seed=r)).to(dev) for r in range(Rq)]),
+            )
+            nbytes = 2 * 2 * Tq * sq.row_bytes * Lq + 8 * Tq
+            rounds = 3                      # patterns interleaved, so drift hits all of them alike
+            per_pattern = {label: [] for label, _ in patterns}
+            for rnd in range(rounds):
+                for label, slot_sets in patterns:
+                    for i in range(2):
+                        kvc.reshape_and_cache_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, slot_sets[i % Rq])
+                    torch.cuda.synchronize()
+                    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    for i in range(reps):
+                        kvc.reshape_and_cache_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, slot_sets[i % Rq])
+                    end.record()
+                    torch.cuda.synchronize()
+                    per_pattern[label].append(start.elapsed_time(end) / reps)
+                    log(f"translation: round {rnd}: {reps + 2} write_rows_kernel dispatches, {label}, "
+                        f"{per_pattern[label][-1] * 1e3:.2f} us each")
+            for label, _ in patterns:
+                ms = sorted(per_pattern[label])[rounds // 2]
+                extra.append(entry(f"cfg3 launch, slot pattern: {label}", nbytes, ms, ms, launch="eager",
+                                   launches_per_round=reps + 2, rounds=rounds,
+                                   us_per_round=[round(x * 1e3, 2) for x in per_pattern[label]]))
+            del poolq, srcs
+            torch.cuda.empty_cache()
 
     # ------------------------------------------------ config 5: swap round trip
     if "swap" in ops:
-        s70 = wl.LLAMA_3_1_70B
-        nb5 = 16384
-        n = min(args.swap_blocks, nb5 // 2)
-        pool5, L5 = alloc_pool(torch, s70, nb5, dev)
-        old, host_ids, new = wl.swap_round_trip(nb5, n, seed=0)
-        out_maps = [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))]
-        in_maps = [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))]
-        nbytes = n * L5 * s70.block_bytes
-        # the on-device half alone: gather to / scatter from a dense HBM buffer (HBM roofline)
-        ids_out = torch.from_numpy(old).to(dev)
-        ids_in = torch.from_numpy(new).to(dev)
-        dense = torch.empty(n, L5, s70.block_elems, dtype=torch.bfloat16, device=dev)
-        ms_w, ms_e = time_region(lambda i: kvc.gather_blocks(pool5, ids_out, out=dense), 10, 2, torch)
-        extra.append(entry(f"cfg5 gather stage, HBM only ({n} blocks x {L5} layers x 64 KiB -> dense buffer)",
-                           2 * nbytes, ms_w, ms_e, launch="eager"))
-        ms_w, ms_e = time_region(lambda i: kvc.scatter_blocks(pool5, ids_in, dense), 10, 2, torch)
-        extra.append(entry(f"cfg5 scatter stage, HBM only (dense buffer -> {n} blocks x {L5} layers x 64 KiB)",
-                           2 * nbytes, ms_w, ms_e, launch="eager"))
-        del dense
-        torch.cuda.empty_cache()
-        settle_copy_engines(torch, dev, "the swap rows", args.settle_seconds)
-        worker = kvc.KVWorker(pool5, n)
-        try:
-            def timed_sync(fn, reps):
-                fn()   # warm-up (first touch of the pinned pool, staging allocation)
-                times = []
-                for _ in range(reps):
-                    torch.cuda.synchronize()
+        with optional_section("config 5 swap rows", torch):
+            s70 = wl.LLAMA_3_1_70B
+            nb5 = 16384
+            n = min(args.swap_blocks, nb5 // 2)
+            pool5, L5 = alloc_pool(torch, s70, nb5, dev)
+            # the pinned host pool first (40 GiB at the stated size): a box that cannot pin
+            # that much runs the rows on fewer blocks, and their names say how many
+            worker = None
+            while worker is None:
+                try:
+                    worker = kvc.KVWorker(pool5, n)
+                except MemoryError as exc:
+                    if n <= 256:
+                        raise
+                    log(f"cannot pin a host pool of {n} blocks ({exc}); trying {n // 2}")
+                    n //= 2
+            try:
+                old, host_ids, new = wl.swap_round_trip(nb5, n, seed=0)
+                out_maps = [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))]
+                in_maps = [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))]
+                nbytes = n * L5 * s70.block_bytes
+                # the on-device half alone: gather to / scatter from a dense HBM buffer (HBM roofline)
+                ids_out = torch.from_numpy(old).to(dev)
+                ids_in = torch.from_numpy(new).to(dev)
+                dense = torch.empty(n, L5, s70.block_elems, dtype=torch.bfloat16, device=dev)
+                ms_w, ms_e = time_region(lambda i: kvc.gather_blocks(pool5, ids_out, out=dense), 10, 2, torch)
+                extra.append(entry(f"cfg5 gather stage, HBM only ({n} blocks x {L5} layers x 64 KiB -> dense buffer)",
+                                   2 * nbytes, ms_w, ms_e, launch="eager"))
+                ms_w, ms_e = time_region(lambda i: kvc.scatter_blocks(pool5, ids_in, dense), 10, 2, torch)
+                extra.append(entry(f"cfg5 scatter stage, HBM only (dense buffer -> {n} blocks x {L5} layers x 64 KiB)",
+                                   2 * nbytes, ms_w, ms_e, launch="eager"))
+                del dense
+                torch.cuda.empty_cache()
+                settle_copy_engines(torch, dev, "the swap rows", args.settle_seconds)
+                def timed_sync(fn, reps):
+                    fn()   # warm-up (first touch of the pinned pool, staging allocation)
+                    times = []
+                    for _ in range(reps):
+                        torch.cuda.synchronize()
+                        t0 = time.perf_counter()
+                        fn()
+                        times.append(time.perf_counter() - t0)
+                    return sorted(times)[len(times) // 2]
+
+                size = f"{n} blocks x {L5} layers x 64 KiB"
+                host_in = np.arange(n // 2, n, dtype=np.int64)
+                both_out = [kvc.BlockMapping.from_pairs(zip(old[:n // 2].tolist(), range(n // 2)))]
+                both_in = [kvc.BlockMapping.from_pairs(zip(host_in.tolist(), new[n // 2:].tolist()))]
+                # "staged" (default): gather/scatter kernel + DMA extents on a second stream;
+                # "direct": one kernel that addresses the mapped host pool
+                for mode in ("staged", "direct"):
+                    worker.swap_mode = mode
+                    for direction, maps, src, dst in (
+                            ("swap_out", out_maps, kvc.Device.GPU, kvc.Device.Host),
+                            ("swap_in", in_maps, kvc.Device.Host, kvc.Device.GPU)):
+                        t = timed_sync(lambda: worker.copy_kv_sync(maps, src, dst), 3)
+                        extra.append({"name": f"cfg5 {direction} ({mode}; {size})", "ms_per_call": round(t * 1e3, 2),
+                                      "pcie_gbps": round(nbytes / t / 1e9, 2), "bytes_per_call": int(nbytes)})
+
+                    # one call per layer, as the layer-pipelined protocol issues them: ids checked and
+                    # uploaded once (kvc_swap_prepare), then one call per layer
+                    enqueue = []
+
+                    def layer_by_layer_prepared():
+                        t0 = time.perf_counter()
+                        prep = worker.prepare_swap("out", out_maps)
+                        t1 = time.perf_counter()
+                        for l in range(L5):
+                            worker.swap_prepared_layers(prep, l, l + 1)
+                        enqueue.append((t1 - t0, time.perf_counter() - t1))
+                        worker.dtoh_stream.synchronize()
+
+                    t = timed_sync(layer_by_layer_prepared, 3)
+                    prep_s, calls_s = sorted(enqueue[1:])[len(enqueue[1:]) // 2]
+                    extra.append({"name": f"cfg5 swap_out layer by layer, ids uploaded once ({mode}; {L5} calls of {n} blocks x 1 layer)",
+                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                  "bytes_per_call": int(nbytes),
+                                  "host_ms_flatten_check_upload_once": round(prep_s * 1e3, 3),
+                                  "host_ms_to_enqueue_all_layer_calls": round(calls_s * 1e3, 3),
+                                  "host_us_per_layer_call": round(calls_s / L5 * 1e6, 2)})
+
+                    # both directions at once on the worker's two streams (PCIe is full duplex):
+                    # write-through of one set of blocks while another set is fetched
+                    def both():
+                        worker.save_kv_blocks_to_host_nowait(both_out)
+                        worker.load_kv_blocks_from_host_nowait(both_in)
+                        worker.dtoh_stream.synchronize()
+                        worker.htod_stream.synchronize()
+
+                    t = timed_sync(both, 3)
+                    extra.append({"name": f"cfg5 swap_out and swap_in at once ({mode}; {n // 2} blocks each way)",
+                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                  "pcie_gbps_note": "sum of both directions", "bytes_per_call": int(nbytes)})
+
+                # host blocks that do not neighbour each other (every second block of the host pool:
+                # what an allocator hands out after churn): the staged mode's PCIe leg falls apart into
+                # one copy per block, the direct kernel does not care, "auto" picks per call
+                ns = min(512, n // 2)
+                scat_maps = [kvc.BlockMapping.from_pairs(zip(old[:ns].tolist(), range(0, 2 * ns, 2)))]
+                sbytes = ns * L5 * s70.block_bytes
+                for mode in ("staged", "direct", "auto"):
+                    worker.swap_mode = mode
+                    picked = {}
+
+                    def scattered_layer_by_layer():
+                        prep = worker.prepare_swap("out", scat_maps)
+                        for l in range(L5):
+                            worker.swap_prepared_layers(prep, l, l + 1)
+                        picked["layer"] = _lib.last_swap_mode()
+                        worker.dtoh_stream.synchronize()
+
+                    def scattered_one_call():
+                        worker.save_kv_blocks_to_host_nowait(scat_maps)
+                        picked["all"] = _lib.last_swap_mode()
+                        worker.dtoh_stream.synchronize()
+
+                    names = {_lib.KVC_SWAP_STAGED: "staged", _lib.KVC_SWAP_DIRECT: "direct"}
+                    t = timed_sync(scattered_layer_by_layer, 3)
+                    extra.append({"name": f"cfg5 swap_out to scattered host blocks, layer by layer ({mode}"
+                                          f"{' -> ' + names[picked['layer']] if mode == 'auto' else ''}; "
+                                          f"{L5} calls of {ns} blocks x 1 layer, 64 KiB extents)",
+                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
+                                  "bytes_per_call": int(sbytes)})
+                    t = timed_sync(scattered_one_call, 3)
+                    extra.append({"name": f"cfg5 swap_out to scattered host blocks, one call ({mode}"
+                                          f"{' -> ' + names[picked['all']] if mode == 'auto' else ''}; "
+                                          f"{ns} blocks x {L5} layers, 5 MiB extents)",
+                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
+                                  "bytes_per_call": int(sbytes)})
+                worker.swap_mode = "direct"
+                enqueue2 = []
+
+                def layer_by_layer_unprepared():
                     t0 = time.perf_counter()
-                    fn()
-                    times.append(time.perf_counter() - t0)
-                return sorted(times)[len(times) // 2]
-
-            size = f"{n} blocks x {L5} layers x 64 KiB"
-            host_in = np.arange(n // 2, n, dtype=np.int64)
-            both_out = [kvc.BlockMapping.from_pairs(zip(old[:n // 2].tolist(), range(n // 2)))]
-            both_in = [kvc.BlockMapping.from_pairs(zip(host_in.tolist(), new[n // 2:].tolist()))]
-            # "staged" (default): gather/scatter kernel + DMA extents on a second stream;
-            # "direct": one kernel that addresses the mapped host pool
-            for mode in ("staged", "direct"):
-                worker.swap_mode = mode
-                for direction, maps, src, dst in (
-                        ("swap_out", out_maps, kvc.Device.GPU, kvc.Device.Host),
-                        ("swap_in", in_maps, kvc.Device.Host, kvc.Device.GPU)):
-                    t = timed_sync(lambda: worker.copy_kv_sync(maps, src, dst), 3)
-                    extra.append({"name": f"cfg5 {direction} ({mode}; {size})", "ms_per_call": round(t * 1e3, 2),
-                                  "pcie_gbps": round(nbytes / t / 1e9, 2), "bytes_per_call": int(nbytes)})
-
-                # one call per layer, as the layer-pipelined protocol issues them: ids checked and
-                # uploaded once (kvc_swap_prepare), then one call per layer
-                enqueue = []
-
-                def layer_by_layer_prepared():
-                    t0 = time.perf_counter()
-                    prep = worker.prepare_swap("out", out_maps)
-                    t1 = time.perf_counter()
                     for l in range(L5):
-                        worker.swap_prepared_layers(prep, l, l + 1)
-                    enqueue.append((t1 - t0, time.perf_counter() - t1))
+                        worker.save_kv_blocks_to_host_nowait(out_maps, layer_begin=l, layer_end=l + 1)
+                    enqueue2.append(time.perf_counter() - t0)
                     worker.dtoh_stream.synchronize()
 
-                t = timed_sync(layer_by_layer_prepared, 3)
-                prep_s, calls_s = sorted(enqueue[1:])[len(enqueue[1:]) // 2]
-                extra.append({"name": f"cfg5 swap_out layer by layer, ids uploaded once ({mode}; {L5} calls of {n} blocks x 1 layer)",
+                t = timed_sync(layer_by_layer_unprepared, 1)
+                extra.append({"name": f"cfg5 swap_out layer by layer, ids flattened, checked and uploaded per call (direct; {L5} calls)",
                               "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
                               "bytes_per_call": int(nbytes),
-                              "host_ms_flatten_check_upload_once": round(prep_s * 1e3, 3),
-                              "host_ms_to_enqueue_all_layer_calls": round(calls_s * 1e3, 3),
-                              "host_us_per_layer_call": round(calls_s / L5 * 1e6, 2)})
-
-                # both directions at once on the worker's two streams (PCIe is full duplex):
-                # write-through of one set of blocks while another set is fetched
-                def both():
-                    worker.save_kv_blocks_to_host_nowait(both_out)
-                    worker.load_kv_blocks_from_host_nowait(both_in)
-                    worker.dtoh_stream.synchronize()
-                    worker.htod_stream.synchronize()
-
-                t = timed_sync(both, 3)
-                extra.append({"name": f"cfg5 swap_out and swap_in at once ({mode}; {n // 2} blocks each way)",
-                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
-                              "pcie_gbps_note": "sum of both directions", "bytes_per_call": int(nbytes)})
-
-            # host blocks that do not neighbour each other (every second block of the host pool:
-            # what an allocator hands out after churn): the staged mode's PCIe leg falls apart into
-            # one copy per block, the direct kernel does not care, "auto" picks per call
-            ns = min(512, n // 2)
-            scat_maps = [kvc.BlockMapping.from_pairs(zip(old[:ns].tolist(), range(0, 2 * ns, 2)))]
-            sbytes = ns * L5 * s70.block_bytes
-            for mode in ("staged", "direct", "auto"):
-                worker.swap_mode = mode
-                picked = {}
-
-                def scattered_layer_by_layer():
-                    prep = worker.prepare_swap("out", scat_maps)
-                    for l in range(L5):
-                        worker.swap_prepared_layers(prep, l, l + 1)
-                    picked["layer"] = _lib.last_swap_mode()
-                    worker.dtoh_stream.synchronize()
-
-                def scattered_one_call():
-                    worker.save_kv_blocks_to_host_nowait(scat_maps)
-                    picked["all"] = _lib.last_swap_mode()
-                    worker.dtoh_stream.synchronize()
-
-                names = {_lib.KVC_SWAP_STAGED: "staged", _lib.KVC_SWAP_DIRECT: "direct"}
-                t = timed_sync(scattered_layer_by_layer, 3)
-                extra.append({"name": f"cfg5 swap_out to scattered host blocks, layer by layer ({mode}"
-                                      f"{' -> ' + names[picked['layer']] if mode == 'auto' else ''}; "
-                                      f"{L5} calls of {ns} blocks x 1 layer, 64 KiB extents)",
-                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
-                              "bytes_per_call": int(sbytes)})
-                t = timed_sync(scattered_one_call, 3)
-                extra.append({"name": f"cfg5 swap_out to scattered host blocks, one call ({mode}"
-                                      f"{' -> ' + names[picked['all']] if mode == 'auto' else ''}; "
-                                      f"{ns} blocks x {L5} layers, 5 MiB extents)",
-                              "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(sbytes / t / 1e9, 2),
-                              "bytes_per_call": int(sbytes)})
-            worker.swap_mode = "direct"
-            enqueue2 = []
-
-            def layer_by_layer_unprepared():
-                t0 = time.perf_counter()
-                for l in range(L5):
-                    worker.save_kv_blocks_to_host_nowait(out_maps, layer_begin=l, layer_end=l + 1)
-                enqueue2.append(time.perf_counter() - t0)
-                worker.dtoh_stream.synchronize()
-
-            t = timed_sync(layer_by_layer_unprepared, 1)
-            extra.append({"name": f"cfg5 swap_out layer by layer, ids flattened, checked and uploaded per call (direct; {L5} calls)",
-                          "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
-                          "bytes_per_call": int(nbytes),
-                          "host_ms_to_enqueue_all_layer_calls": round(enqueue2[-1] * 1e3, 3)})
-        finally:
-            worker.close()
-        del pool5
-        torch.cuda.empty_cache()
+                              "host_ms_to_enqueue_all_layer_calls": round(enqueue2[-1] * 1e3, 3)})
+            finally:
+                worker.close()
+            del pool5
+            torch.cuda.empty_cache()
     if "overlap" in ops:
         try:
             settle_copy_engines(torch, dev, "the write-through rows", args.settle_seconds)
@@ -1292,46 +1333,47 @@ def main():
 
     # ------------------------------------------------ one rank's slice of Llama-3.1-70B at tp=8
     if "shard" in ops:
-        sh = wl.LLAMA_3_1_70B.shard(8)          # 1 KV head: 256-byte rows, 8 KiB blocks, 80 layers
-        nbs = 65536
-        pool_s, Ls = alloc_pool(torch, sh, nbs, dev)
-        sets_s = write_inputs(torch, kvc, wl.decode_step, sh, Ls, nbs, dev, ROTATE_DECODE, batch=256)
-        es, _ = bench_write_config(torch, kvc, "70B/tp8 shard decode", sets_s, pool_s, Ls, args.steps,
-                                   args.warmup, ["fused_slot:graph", "per_layer_paged:graph"])
-        extra += es
-        maps = [torch.from_numpy(wl.copy_on_write_pairs(nbs, 4096, seed=r)[0]).to(dev) for r in range(2)]
-        nbytes = 2 * 4096 * Ls * sh.block_bytes + 16 * 4096
-        ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool_s, maps[i % 2]), 20, 3, torch)
-        extra.append(entry(f"70B/tp8 shard copy_blocks (4096 pairs x {Ls} layers, 8 KiB blocks)", nbytes,
-                           ms_w, ms_e, launch="eager"))
-        n = min(4096, args.swap_blocks * 4, nbs // 2)
-        old, host_ids, new = wl.swap_round_trip(nbs, n, seed=0)
-        nbytes = n * Ls * sh.block_bytes
-        settle_copy_engines(torch, dev, "the shard's swap rows", args.settle_seconds)
-        worker = kvc.KVWorker(pool_s, n)
-        try:
-            for mode in ("staged", "direct"):
-                worker.swap_mode = mode
-                for direction, maps_, src, dst in (
-                        ("swap_out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))],
-                         kvc.Device.GPU, kvc.Device.Host),
-                        ("swap_in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))],
-                         kvc.Device.Host, kvc.Device.GPU)):
-                    worker.copy_kv_sync(maps_, src, dst)
-                    times = []
-                    for _ in range(3):
-                        torch.cuda.synchronize()
-                        t0 = time.perf_counter()
+        with optional_section("tensor-parallel shard rows", torch):
+            sh = wl.LLAMA_3_1_70B.shard(8)          # 1 KV head: 256-byte rows, 8 KiB blocks, 80 layers
+            nbs = 65536
+            pool_s, Ls = alloc_pool(torch, sh, nbs, dev)
+            sets_s = write_inputs(torch, kvc, wl.decode_step, sh, Ls, nbs, dev, ROTATE_DECODE, batch=256)
+            es, _ = bench_write_config(torch, kvc, "70B/tp8 shard decode", sets_s, pool_s, Ls, args.steps,
+                                       args.warmup, ["fused_slot:graph", "per_layer_paged:graph"])
+            extra += es
+            maps = [torch.from_numpy(wl.copy_on_write_pairs(nbs, 4096, seed=r)[0]).to(dev) for r in range(2)]
+            nbytes = 2 * 4096 * Ls * sh.block_bytes + 16 * 4096
+            ms_w, ms_e = time_region(lambda i: kvc.copy_blocks(pool_s, maps[i % 2]), 20, 3, torch)
+            extra.append(entry(f"70B/tp8 shard copy_blocks (4096 pairs x {Ls} layers, 8 KiB blocks)", nbytes,
+                               ms_w, ms_e, launch="eager"))
+            n = min(4096, args.swap_blocks * 4, nbs // 2)
+            old, host_ids, new = wl.swap_round_trip(nbs, n, seed=0)
+            nbytes = n * Ls * sh.block_bytes
+            settle_copy_engines(torch, dev, "the shard's swap rows", args.settle_seconds)
+            worker = kvc.KVWorker(pool_s, n)
+            try:
+                for mode in ("staged", "direct"):
+                    worker.swap_mode = mode
+                    for direction, maps_, src, dst in (
+                            ("swap_out", [kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))],
+                             kvc.Device.GPU, kvc.Device.Host),
+                            ("swap_in", [kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))],
+                             kvc.Device.Host, kvc.Device.GPU)):
                         worker.copy_kv_sync(maps_, src, dst)
-                        times.append(time.perf_counter() - t0)
-                    t = sorted(times)[1]
-                    extra.append({"name": f"70B/tp8 shard {direction} ({mode}; {n} blocks x {Ls} layers x 8 KiB)",
-                                  "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
-                                  "bytes_per_call": int(nbytes)})
-        finally:
-            worker.close()
-        del pool_s, sets_s
-        torch.cuda.empty_cache()
+                        times = []
+                        for _ in range(3):
+                            torch.cuda.synchronize()
+                            t0 = time.perf_counter()
+                            worker.copy_kv_sync(maps_, src, dst)
+                            times.append(time.perf_counter() - t0)
+                        t = sorted(times)[1]
+                        extra.append({"name": f"70B/tp8 shard {direction} ({mode}; {n} blocks x {Ls} layers x 8 KiB)",
+                                      "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
+                                      "bytes_per_call": int(nbytes)})
+            finally:
+                worker.close()
+            del pool_s, sets_s
+            torch.cuda.empty_cache()
 
     # ------------------------------------------------ host <-> disk tier (config 5 block rows)
     if "disk" in ops:
