@@ -524,7 +524,7 @@ def cpu_baseline_others(torch, wl, seconds_each):
     return out
 
 
-def bench_write_through_overlap(torch, kvc, wl, dev):
+def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
     """What the layer-pipelined protocol is for (kv_worker.py:272-295,
     model_worker.py:254-276): the KV worker saves layer l of the step's blocks to
     the host pool while the model is already computing layer l+1. A stand-in
@@ -533,7 +533,14 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
     layer-by-layer swap-out runs alone, and then both run together with the
     worker (a thread of this process, as the tests run it) following the hooks:
     once in the default staged mode (DMA engines carry the PCIe leg) and once in
-    the direct mode (a kernel writes to the mapped host pool)."""
+    the direct mode (a kernel writes to the mapped host pool).
+
+    scattered=True: the host blocks are every second block of the host pool (what
+    an allocator hands out after churn), so a layer's rows are 64 KiB pieces that
+    do not neighbour each other. The worker's default then carries each layer as
+    one copy into a dense pinned buffer and lets host threads place the rows;
+    beside it, the same worker without that buffer (the direct kernel) and the
+    copy engines on the rows as they lie (one copy per block)."""
     import asyncio
     import threading
 
@@ -553,14 +560,47 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
                                 idx.kv_last_block_lens, s8.num_kv_heads, s8.head_dim, s8.block_size,
                                 torch.bfloat16, resolve_slots=True)
     rng_ids = np.random.default_rng(5).permutation(nb)[:n]
-    maps = [kvc.BlockMapping.from_pairs(zip(rng_ids.tolist(), range(n)))]
+    host_ids = list(range(0, 2 * n, 2)) if scattered else list(range(n))
+    nhb = 2 * n if scattered else n
+    maps = [kvc.BlockMapping.from_pairs(zip(rng_ids.tolist(), host_ids))]
     model_stream = torch.cuda.Stream()
     nbytes = n * L * s8.block_bytes
     out = []
-    for mode in ("staged", "direct"):
+    variants = [("staged", 0, "staged swap"), ("direct", 0, "direct swap")]
+    if scattered:
+        variants = [("auto", 1 << 30, "scattered host blocks; auto: one copy per layer into a dense pinned "
+                                      "buffer, rows placed by host threads"),
+                    ("auto", 0, "scattered host blocks; auto without the pinned buffer: the direct kernel"),
+                    ("staged", 0, "scattered host blocks; staged: the copy engines, one copy per block")]
+    for mode, bounce_bytes, label in variants:
         handle = kvc.KVWorkerHandle.create(L)
-        worker = kvc.KVWorker(pool, num_host_blocks=n, swap_mode=mode, kv_worker_handle=handle)
+        worker = kvc.KVWorker(pool, num_host_blocks=nhb, swap_mode=mode, kv_worker_handle=handle,
+                              host_bounce_bytes=bounce_bytes)
         hooks = kvc.LayerSyncHooks(handle)
+
+        def protocol_alone(copy_maps, src, dst, saving):
+            """The layer-by-layer copy through `copy_kv` with nothing else on the GPU: the
+            model side only rings the doorbells (save) or takes them (fetch)."""
+            best = None
+            for _ in range(4):
+                torch.cuda.synchronize()
+                th = threading.Thread(target=lambda: asyncio.run(worker.copy_kv(copy_maps, src, dst)))
+                hooks.enable_record_after_execute = saving
+                hooks.enable_wait_before_execute = not saving
+                hooks.timeout = 60
+                t0 = time.perf_counter()
+                th.start()
+                with torch.cuda.stream(model_stream):
+                    for l in range(L):
+                        hooks.pre(l)
+                        hooks.post(l)
+                th.join(timeout=120)
+                torch.cuda.synchronize()
+                t = (time.perf_counter() - t0) * 1e3
+                best = t if best is None else min(best, t)
+            hooks.enable_record_after_execute = False
+            hooks.enable_wait_before_execute = False
+            return best
 
         def forward():
             with torch.cuda.stream(model_stream):
@@ -584,9 +624,9 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
             e0, e1 = timed_forward()
             torch.cuda.synchronize()
             fwd_alone = e0.elapsed_time(e1)
-            prepared = worker.prepare_swap("out", maps)
-            swap_alone = None
-            for _ in range(4):                                   # the first pass touches the pinned pool
+            prepared = None if scattered else worker.prepare_swap("out", maps)
+            swap_alone = protocol_alone(maps, kvc.Device.GPU, kvc.Device.Host, True) if scattered else None
+            for _ in range(0 if scattered else 4):               # the first pass touches the pinned pool
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for l in range(L):
@@ -609,7 +649,8 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
             total = (time.perf_counter() - t0) * 1e3
             hooks.enable_record_after_execute = False
             fwd_with = e0.elapsed_time(e1)
-            out.append({"name": f"write-through during a stand-in forward pass ({mode} swap; {L} layers; {n} blocks x "
+            del prepared
+            out.append({"name": f"write-through during a stand-in forward pass ({label}; {L} layers; {n} blocks x "
                                 f"{L} layers x 64 KiB saved layer by layer behind the model's post hooks)",
                         "forward_alone_ms": round(fwd_alone, 2), "swap_alone_ms": round(swap_alone, 2),
                         "forward_with_write_through_ms": round(fwd_with, 2),
@@ -621,10 +662,10 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
             # the other half of the protocol (kv_worker.py:249-270, model_worker.py:254-263): the
             # blocks of a request come back from the host layer by layer, and the model's layer l
             # waits for "layer l landed" before it runs
-            in_maps = [kvc.BlockMapping.from_pairs(zip(range(n), rng_ids.tolist()))]
-            prepared_in = worker.prepare_swap("in", in_maps)
-            fetch_alone = None
-            for _ in range(4):
+            in_maps = [kvc.BlockMapping.from_pairs(zip(host_ids, rng_ids.tolist()))]
+            prepared_in = None if scattered else worker.prepare_swap("in", in_maps)
+            fetch_alone = protocol_alone(in_maps, kvc.Device.Host, kvc.Device.GPU, False) if scattered else None
+            for _ in range(0 if scattered else 4):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for l in range(L):
@@ -632,6 +673,8 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
                 worker.htod_stream.synchronize()
                 t = (time.perf_counter() - t0) * 1e3
                 fetch_alone = t if fetch_alone is None else min(fetch_alone, t)
+
+            del prepared_in
 
             def kv_fetch_thread():
                 asyncio.run(worker.copy_kv(in_maps, kvc.Device.Host, kvc.Device.GPU))
@@ -647,7 +690,7 @@ def bench_write_through_overlap(torch, kvc, wl, dev):
             torch.cuda.synchronize()
             total = (time.perf_counter() - t0) * 1e3
             hooks.enable_wait_before_execute = False
-            out.append({"name": f"fetch during a stand-in forward pass ({mode} swap; {L} layers; {n} blocks x {L} "
+            out.append({"name": f"fetch during a stand-in forward pass ({label}; {L} layers; {n} blocks x {L} "
                                 f"layers x 64 KiB loaded layer by layer, each layer of the model waits for its own)",
                         "forward_alone_ms": round(fwd_alone, 2), "fetch_alone_ms": round(fetch_alone, 2),
                         "forward_behind_the_fetch_ms": round(e0.elapsed_time(e1), 2),
@@ -1321,6 +1364,7 @@ def main():
         try:
             settle_copy_engines(torch, dev, "the write-through rows", args.settle_seconds)
             extra += bench_write_through_overlap(torch, kvc, wl, dev)
+            extra += bench_write_through_overlap(torch, kvc, wl, dev, scattered=True)
             extra += bench_small_write_through(torch, kvc, wl, dev)
         except Exception as exc:
             log(f"write-through overlap skipped: {exc!r}")

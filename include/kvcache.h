@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define KVC_ABI_VERSION 4
+#define KVC_ABI_VERSION 5
 
 typedef enum kvc_status {
   KVC_OK = 0,
@@ -578,6 +578,56 @@ int kvc_disk_save_blocks(kvc_disk* disk, const void* host_pool, int64_t num_host
 int kvc_disk_load_blocks(kvc_disk* disk, void* host_pool, int64_t num_host_blocks,
                          const int64_t* src_disk_ids, const int64_t* dst_host_ids, int64_t n,
                          int threads);
+
+/*
+ * Host side of a one-layer swap to or from scattered host blocks, on host threads.
+ * Serves
+ *   _save_layer_kv_blocks_to_host     (runtime/worker/llm_worker/kv_worker.py:213-227)
+ *   _load_layer_kv_blocks_from_host   (kv_worker.py:197-211)
+ * when the layer's rows do not neighbour each other in the host pool
+ * [num_host_blocks, L, block] (kv_worker.py:123-127): the PCIe leg of the layer
+ * is then one copy between the GPU and a dense pinned buffer
+ * (kvc_swap_out_prepared / kvc_swap_in_prepared with that buffer as a one-layer
+ * host pool and host ids 0..n-1), and this call moves the rows between the
+ * buffer and their places in the pool:
+ *   to_pool != 0: pool[host_ids[i]] [pool_offset .. pool_offset + row_bytes) = dense[i]
+ *   to_pool == 0: dense[i] = pool[host_ids[i]] [pool_offset .. pool_offset + row_bytes)
+ * with pool_block_bytes the bytes of one host block over all layers,
+ * pool_offset = layer * block bytes and dense rows row_bytes apart. Ids are
+ * range-checked first. Synchronous, `threads` host threads (<= 0: 4; fewer for
+ * small calls); no GPU work, callable from any thread. Rows of one call must be
+ * distinct when to_pool != 0.
+ */
+int kvc_host_copy_rows(void* host_pool, int64_t num_host_blocks, int64_t pool_block_bytes,
+                       int64_t pool_offset, void* dense, const int64_t* host_ids, int64_t n,
+                       int64_t row_bytes, int to_pool, int threads);
+
+/*
+ * The same row copies as a queue with a thread of its own, so that the caller's
+ * loop over the layers (kv_worker.py:249-295) never waits for the host side:
+ * kvc_row_mover_submit checks the ids, copies them and returns a ticket
+ * (0, 1, 2, ... in the order of the calls; a negative kvc_status on error);
+ * the mover's thread takes the jobs in that order, waits for `after_event` first
+ * when one is given (a hipEvent_t of the device that is current at the submit:
+ * "the layer has landed in the dense buffer" for a save, "the GPU has read the
+ * region" for a load), and moves the rows on `threads` host threads.
+ * kvc_row_mover_done tells without blocking whether a ticket's job has finished
+ * (1) or not (0); kvc_row_mover_wait blocks until it has, together with every
+ * job submitted before it, and returns the status of the first job that failed
+ * since the last wait. The event, the pool and the dense buffer must stay valid
+ * until the job is done. kvc_row_mover_destroy finishes the queued jobs first.
+ * One thread submits to a mover at a time; done and wait may be called from
+ * any thread.
+ */
+typedef struct kvc_row_mover kvc_row_mover;
+int kvc_row_mover_create(int threads, kvc_row_mover** out);
+int64_t kvc_row_mover_submit(kvc_row_mover* mover, void* after_event, void* host_pool,
+                             int64_t num_host_blocks, int64_t pool_block_bytes, int64_t pool_offset,
+                             void* dense, const int64_t* host_ids, int64_t n, int64_t row_bytes,
+                             int to_pool);
+int kvc_row_mover_done(kvc_row_mover* mover, int64_t ticket);
+int kvc_row_mover_wait(kvc_row_mover* mover, int64_t ticket);
+int kvc_row_mover_destroy(kvc_row_mover* mover);
 
 /* Pinned, device-addressable host memory for the host pool; replaces
  * pycuda.driver.pagelocked_empty (runtime/worker/llm_worker/kv_worker.py:123-127).

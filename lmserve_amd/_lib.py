@@ -47,7 +47,7 @@ KVC_LAUNCH_NON_TEMPORAL = 5
 KVC_LAUNCH_PIPE = 6
 KVC_LAUNCH_SWAP_MODE = 7
 
-KVC_ABI_VERSION = 4
+KVC_ABI_VERSION = 5
 KVC_NOALLOC_MAX_BLOCKS = 8192
 
 KVC_DTYPE_BF16 = 0
@@ -122,6 +122,12 @@ SIGNATURES = {
     "kvc_disk_info": (_I64, [_P, c_int]),
     "kvc_disk_save_blocks": (c_int, [_P, _P, _I64, _P, _P, _I64, c_int]),
     "kvc_disk_load_blocks": (c_int, [_P, _P, _I64, _P, _P, _I64, c_int]),
+    "kvc_host_copy_rows": (c_int, [_P, _I64, _I64, _I64, _P, _P, _I64, _I64, c_int, c_int]),
+    "kvc_row_mover_create": (c_int, [c_int, ctypes.POINTER(_P)]),
+    "kvc_row_mover_submit": (_I64, [_P, _P, _P, _I64, _I64, _I64, _P, _P, _I64, _I64, c_int]),
+    "kvc_row_mover_done": (c_int, [_P, _I64]),
+    "kvc_row_mover_wait": (c_int, [_P, _I64]),
+    "kvc_row_mover_destroy": (c_int, [_P]),
     "kvc_host_alloc_pinned": (_P, [c_size_t]),
     "kvc_host_free_pinned": (c_int, [_P]),
 }

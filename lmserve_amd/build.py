@@ -14,7 +14,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
 SOURCES = [os.path.join(PKG_DIR, "csrc", "kvcache.hip"),
            os.path.join(PKG_DIR, "csrc", "rope_cache.hip"),
-           os.path.join(PKG_DIR, "csrc", "disk_tier.cpp")]
+           os.path.join(PKG_DIR, "csrc", "disk_tier.cpp"),
+           os.path.join(PKG_DIR, "csrc", "host_rows.cpp")]
 INCLUDE = os.path.join(REPO_ROOT, "include")
 LIB_PATH = os.path.join(PKG_DIR, "libkvcache.so")
 FAST_SRC = os.path.join(PKG_DIR, "csrc", "fastcall.cpp")

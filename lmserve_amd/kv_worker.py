@@ -20,6 +20,13 @@ forward pass) flattens, checks and uploads its id lists once
 (`kvc_swap_prepare`); each layer is then a single launch
 (`kvc_swap_out_prepared` / `kvc_swap_in_prepared`).
 
+When the layers of a copy travel one per call and the host blocks do not
+neighbour each other (a layer's rows are then 64 KiB pieces a whole host block
+apart: too small for the copy engines, and a kernel that stores them over PCIe
+holds back the model's kernels), the PCIe leg of a layer is one copy between
+the GPU and a dense pinned buffer and host threads move the rows between that
+buffer and their places in the host pool (`kvc_host_copy_rows`).
+
 The Host<->Disk legs (kv_worker.py:229-247) go through the native disk tier of
 the same library (`disk_tier.DiskTier`: whole-block positional I/O on the
 reference's `.npy` file); they involve no GPU work.
@@ -156,6 +163,44 @@ class PreparedSwap:
     host_ids: np.ndarray           # kept alive: the staged mode reads it per call
     staging: torch.Tensor          # head: [gpu_ids | host_ids] on the device
     stream: torch.cuda.Stream
+    dense_ids: Optional[np.ndarray] = None   # 0..n-1, for calls that land in a dense bounce region
+
+
+class HostBounce:
+    """Dense pinned buffer of `slots` regions, each one layer of `n` blocks: what a
+    one-layer PCIe copy lands in (or leaves from) when its rows are scattered over
+    the host pool."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        self.ptr = _lib.lib().kvc_host_alloc_pinned(max(self.nbytes, 1))
+        if not self.ptr:
+            raise MemoryError(f"cannot pin {self.nbytes} bytes of host memory: {_lib.last_error()}")
+        self.busy = False
+        self.slots = 0
+        self.slot_bytes = 0
+        self.mover = None     # kvc_row_mover: its thread moves the rows of the regions
+
+    def row_mover(self, threads: int):
+        if self.mover is None:
+            mover = ctypes.c_void_p()
+            _lib.check(_lib.lib().kvc_row_mover_create(int(threads), ctypes.byref(mover)))
+            self.mover = mover
+        return self.mover
+
+    def shape(self, slots: int, slot_bytes: int) -> None:
+        self.slots, self.slot_bytes = int(slots), int(slot_bytes)
+
+    def slot_ptr(self, layer_idx: int) -> int:
+        return self.ptr + (layer_idx % self.slots) * self.slot_bytes
+
+    def close(self) -> None:
+        if self.mover is not None:
+            _lib.check(_lib.lib().kvc_row_mover_destroy(self.mover))   # after its queued jobs
+            self.mover = None
+        if self.ptr:
+            _lib.check(_lib.lib().kvc_host_free_pinned(self.ptr))
+            self.ptr = None
 
 
 class KVWorker:
@@ -189,6 +234,16 @@ class KVWorker:
       alignment and the file system allow, and spreads block extents over this
       many threads (the reference copies rows through a memory map on 4);
       `disk_preallocate` reserves a new file's blocks when it is made.
+    host_bounce_bytes / host_copy_threads: layer-by-layer copies (the protocol
+      with a handle) whose host blocks are scattered so that a layer's PCIe
+      extents would be under 1 MiB in the mean go through a dense pinned buffer
+      of up to this many bytes (2 to 4 regions of one layer of the copy's
+      blocks; allocated on first use and kept) and this many host threads, in
+      the "auto" and "staged" modes: the copy engines carry each layer as one
+      copy and the model's kernels keep running. 0 turns it off ("auto" then
+      takes the direct kernel for such copies). A copy too large for the buffer,
+      or a second one of the same direction while the buffer is in use, goes
+      the usual way.
     validate: check on the host that no block is the destination of two pairs of
       one GPU<->Host call (`ValueError`). The reference copies the pairs one
       after the other, so the later pair wins there (kv_worker.py:197-227);
@@ -209,6 +264,8 @@ class KVWorker:
         disk_threads: int = 8,
         disk_preallocate: bool = False,
         validate: bool = False,
+        host_bounce_bytes: int = 1 << 30,
+        host_copy_threads: int = 6,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -233,6 +290,10 @@ class KVWorker:
         self.swap_mode = swap_mode
         self.staging_chunk_blocks = int(staging_chunk_blocks)
         self.validate = bool(validate)
+        self.host_bounce_bytes = int(host_bounce_bytes)
+        self.host_copy_threads = int(host_copy_threads)
+        self._bounce = {"out": None, "in": None}
+        self.last_copy_went_through_host_bounce = False
 
         self._host_pool = PinnedHostPool((self.num_host_blocks, num_layers, block_elems), np_dtype)
         self.host_kv_caches = self._host_pool.array
@@ -393,6 +454,70 @@ class KVWorker:
                           prepared.staging.numel(), SWAP_MODES[self.swap_mode],
                           prepared.stream.cuda_stream, prepared.stream.cuda_stream))
 
+    # ------------------------------- one layer per call, scattered host blocks
+    def _bounce_for(self, prepared: Optional["PreparedSwap"]) -> Optional[HostBounce]:
+        """The dense pinned buffer for the one-layer calls of `prepared`, marked
+        busy, or None when they should go the usual way."""
+        if prepared is None or self.swap_mode == "direct" or self.host_bounce_bytes <= 0:
+            return None
+        n, ids = prepared.n, prepared.host_ids
+        runs = 1 + int(np.count_nonzero(ids[1:] != ids[:-1] + 1))
+        if n * self.block_stride >= runs * _lib.get_tuning("auto_min_extent_bytes"):
+            return None            # long extents: the copy engines take the rows as they lie
+        slot_bytes = n * self.block_stride
+        slots = min(4, self.host_bounce_bytes // slot_bytes, self.num_layers)
+        if slots < min(2, self.num_layers):
+            return None
+        bounce = self._bounce[prepared.direction]
+        if bounce is not None and bounce.busy:
+            return None
+        if bounce is None or bounce.nbytes < slots * slot_bytes:
+            if bounce is not None:
+                with torch.cuda.device(self.device):
+                    prepared.stream.synchronize()   # nothing of an earlier copy still lands in it
+                bounce.close()
+            bounce = self._bounce[prepared.direction] = HostBounce(slots * slot_bytes)
+        bounce.shape(slots, slot_bytes)
+        bounce.busy = True
+        return bounce
+
+    def _swap_layer_through_bounce(self, prepared: "PreparedSwap", layer_idx: int, slot_ptr: int) -> None:
+        """Enqueue one layer of a prepared swap between the pool and a dense region
+        of the bounce buffer: that region is the call's host pool (one layer, host
+        ids 0..n-1), so the PCIe leg is one copy per staging chunk."""
+        lib = _lib.lib()
+        fn = lib.kvc_swap_out_prepared if prepared.direction == "out" else lib.kvc_swap_in_prepared
+        if prepared.dense_ids is None:
+            prepared.dense_ids = np.arange(prepared.n, dtype=np.int64)
+        with torch.cuda.device(self.device):
+            _lib.check(fn(self.gpu_kv_caches.data_ptr() + layer_idx * self.layer_stride, slot_ptr,
+                          prepared.dense_ids.ctypes.data, prepared.n, 1, self.layer_stride,
+                          self.block_stride, self.num_gpu_blocks, prepared.n, 0, 1,
+                          prepared.staging.data_ptr(), prepared.staging.numel(), _lib.KVC_SWAP_STAGED,
+                          prepared.stream.cuda_stream, prepared.stream.cuda_stream))
+
+    def _submit_host_rows(self, bounce: HostBounce, prepared: "PreparedSwap", layer_idx: int,
+                          to_pool: bool, after: Optional[torch.cuda.Event]) -> int:
+        """Queue the rows of one layer between its bounce region and their host
+        blocks (the mover's thread waits for `after` first); returns the ticket."""
+        with torch.cuda.device(self.device):
+            ticket = _lib.lib().kvc_row_mover_submit(
+                bounce.row_mover(self.host_copy_threads), after.cuda_event if after is not None else None,
+                self._host_pool.ptr, self.num_host_blocks, self.num_layers * self.block_stride,
+                layer_idx * self.block_stride, bounce.slot_ptr(layer_idx), prepared.host_ids.ctypes.data,
+                prepared.n, self.block_stride, 1 if to_pool else 0)
+        if ticket < 0:
+            _lib.check(int(ticket))
+        return int(ticket)
+
+    async def _host_rows_done(self, bounce: HostBounce, ticket: int) -> None:
+        """Return once the mover has finished `ticket` (and every job before it)."""
+        lib = _lib.lib()
+        if lib.kvc_row_mover_done(bounce.mover, ticket) == 1:
+            _lib.check(lib.kvc_row_mover_wait(bounce.mover, ticket))       # returns at once: picks up errors
+        else:
+            _lib.check(await asyncio.to_thread(lib.kvc_row_mover_wait, bounce.mover, ticket))
+
     async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
                                      stream: torch.cuda.Stream) -> None:
         """GPU->Host (kv_worker.py:272-295). With a handle: per layer, wait for the
@@ -404,15 +529,35 @@ class KVWorker:
             self.save_kv_blocks_to_host_nowait(block_mappings, stream)
         elif len(block_mappings) > 0:
             prepared = self.prepare_swap("out", block_mappings, stream)
-            for layer_idx in range(self.num_layers):
-                while handle.kv_queue.empty():
-                    await asyncio.sleep(1e-5)
-                handle.kv_queue.get()
-                if handle.sync == "events":
-                    stream.wait_event(handle.post_events[layer_idx])
-                # sync == "host": the token was sent after the layer's write had completed
-                self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
-                await asyncio.sleep(0)  # let other tasks of the loop run
+            bounce = self._bounce_for(prepared)
+            self.last_copy_went_through_host_bounce = bounce is not None
+            tickets: List[int] = []                 # per layer: its rows' job in the mover
+            landed: List[torch.cuda.Event] = []     # per layer: the layer sits in its bounce region
+            try:
+                for layer_idx in range(self.num_layers):
+                    while handle.kv_queue.empty():
+                        await asyncio.sleep(1e-5)
+                    handle.kv_queue.get()
+                    if handle.sync == "events":
+                        stream.wait_event(handle.post_events[layer_idx])
+                    # sync == "host": the token was sent after the layer's write had completed
+                    if bounce is None:
+                        self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
+                    else:
+                        if layer_idx >= bounce.slots:       # the region's earlier rows must have left it
+                            await self._host_rows_done(bounce, tickets[layer_idx - bounce.slots])
+                        self._swap_layer_through_bounce(prepared, layer_idx, bounce.slot_ptr(layer_idx))
+                        landed.append(torch.cuda.Event())
+                        landed[-1].record(stream)
+                        tickets.append(self._submit_host_rows(bounce, prepared, layer_idx, True, landed[-1]))
+                    await asyncio.sleep(0)  # let other tasks of the loop run
+            finally:
+                if bounce is not None:
+                    try:
+                        if tickets:
+                            await self._host_rows_done(bounce, tickets[-1])
+                    finally:
+                        bounce.busy = False
         await asyncio.to_thread(stream.synchronize)
 
     async def load_kv_blocks_from_host(self, block_mappings: Sequence[BlockMapping],
@@ -425,14 +570,42 @@ class KVWorker:
             self.load_kv_blocks_from_host_nowait(block_mappings, stream)
         elif len(block_mappings) > 0:
             prepared = self.prepare_swap("in", block_mappings, stream)
-            for layer_idx in range(self.num_layers):
-                self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
-                await asyncio.sleep(0)
-                handle.pre_events[layer_idx].record(stream)
-                if handle.sync == "events":
-                    handle.model_queue.put(b"")
-                else:
-                    handle.ring_when_done(handle.pre_events[layer_idx], handle.model_queue)
+            bounce = self._bounce_for(prepared)
+            self.last_copy_went_through_host_bounce = bounce is not None
+            tickets: List[int] = []                    # per layer: the job that fills its bounce region
+            region_read: List[torch.cuda.Event] = []   # per layer: the GPU has taken the region's rows
+            try:
+                if bounce is not None:
+                    # host threads fill the regions ahead of the GPU: the first ones now, region
+                    # l % slots again for layer l + slots once the GPU has read layer l from it
+                    for ahead in range(min(bounce.slots, self.num_layers)):
+                        tickets.append(self._submit_host_rows(bounce, prepared, ahead, False, None))
+                for layer_idx in range(self.num_layers):
+                    if bounce is None:
+                        self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
+                    else:
+                        await self._host_rows_done(bounce, tickets[layer_idx])
+                        self._swap_layer_through_bounce(prepared, layer_idx, bounce.slot_ptr(layer_idx))
+                        region_read.append(torch.cuda.Event())
+                        region_read[-1].record(stream)
+                        if layer_idx + bounce.slots < self.num_layers:
+                            tickets.append(self._submit_host_rows(bounce, prepared, layer_idx + bounce.slots,
+                                                                  False, region_read[-1]))
+                    await asyncio.sleep(0)
+                    handle.pre_events[layer_idx].record(stream)
+                    if handle.sync == "events":
+                        handle.model_queue.put(b"")
+                    else:
+                        handle.ring_when_done(handle.pre_events[layer_idx], handle.model_queue)
+            finally:
+                if bounce is not None:
+                    try:
+                        if tickets:                      # after an error: let the queued jobs come to rest
+                            await self._host_rows_done(bounce, tickets[-1])
+                        if region_read:
+                            await asyncio.to_thread(region_read[-1].synchronize)
+                    finally:
+                        bounce.busy = False
         await asyncio.to_thread(stream.synchronize)
 
     # ----------------------------------------------------------------- disk legs
@@ -501,6 +674,10 @@ class KVWorker:
             self.disk_tier.close()
             self.disk_tier = None
         self._host_pool.close()
+        for direction, bounce in self._bounce.items():
+            if bounce is not None:
+                bounce.close()
+                self._bounce[direction] = None
         self._staging = {}
         # let go of the pool now: the direction table holds bound methods, so the
         # worker is part of a reference cycle and would otherwise keep tens of GiB

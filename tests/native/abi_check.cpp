@@ -486,6 +486,25 @@ int main() {
     KVC_OK_OR_DIE(kvc_host_free_pinned(host));
   }
 
+  // 9. one layer of scattered host blocks through a dense buffer (host threads only)
+  {
+    const int64_t n = 5, layer = 1;
+    std::vector<uint16_t> host_pool((size_t)(nhb * L * blk_elems)), dense((size_t)(n * blk_elems));
+    for (auto& x : host_pool) x = (uint16_t)rng();
+    for (auto& x : dense) x = (uint16_t)rng();
+    std::vector<int64_t> ids = {9, 0, 4, 2, 7};
+    std::vector<uint16_t> want_p(host_pool);
+    for (int64_t i = 0; i < n; ++i)
+      std::memcpy(&want_p[(size_t)((ids[i] * L + layer) * blk_elems)], &dense[(size_t)(i * blk_elems)], blk_bytes);
+    KVC_OK_OR_DIE(kvc_host_copy_rows(host_pool.data(), nhb, L * blk_bytes, layer * blk_bytes, dense.data(),
+                                     ids.data(), n, blk_bytes, 1, 3));
+    expect_equal("kvc_host_copy_rows into the pool", host_pool.data(), want_p.data(), host_pool.size() * 2);
+    std::vector<uint16_t> back(dense.size());
+    KVC_OK_OR_DIE(kvc_host_copy_rows(host_pool.data(), nhb, L * blk_bytes, layer * blk_bytes, back.data(),
+                                     ids.data(), n, blk_bytes, 0, 3));
+    expect_equal("kvc_host_copy_rows out of the pool", back.data(), dense.data(), dense.size() * 2);
+  }
+
   KVC_OK_OR_DIE(kvc_thread_release());
   HIP_OK(hipDeviceSynchronize());
   if (fails) {

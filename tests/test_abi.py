@@ -261,6 +261,90 @@ def test_pairs_are_ordered_by_host_block_id_like_a_stable_sort():
     assert L.kvc_order_pairs_by_host_id(g.ctypes.data, asc.ctypes.data, -1) == _lib.KVC_ERR_INVALID_ARG
 
 
+@pytest.mark.parametrize("threads", [1, 3, 8])
+def test_host_rows_between_a_dense_buffer_and_scattered_host_blocks(threads):
+    """kvc_host_copy_rows runs on the host alone: rows of one layer to and from
+    scattered blocks of a [num_host_blocks, L, block] pool, against NumPy indexing,
+    the rest of the pool untouched; then the argument checks."""
+    L_fn = _lib.lib().kvc_host_copy_rows
+    rng = np.random.default_rng(7 + threads)
+    nhb, layers, row = 97, 3, 40 << 10          # 120 KiB host blocks, 40 KiB rows
+    pool = rng.integers(0, 255, size=(nhb, layers, row), dtype=np.uint8)
+    for n in (1, 8, 61):                        # below one MiB (inline) and above (threads)
+        ids = rng.permutation(nhb)[:n].astype(np.int64)
+        for layer in (0, layers - 1):
+            dense = rng.integers(0, 255, size=(n, row), dtype=np.uint8)
+            want = pool.copy()
+            want[ids, layer] = dense
+            assert L_fn(pool.ctypes.data, nhb, layers * row, layer * row, dense.ctypes.data,
+                        ids.ctypes.data, n, row, 1, threads) == 0
+            assert np.array_equal(pool, want)
+            back = np.zeros_like(dense)
+            assert L_fn(pool.ctypes.data, nhb, layers * row, layer * row, back.ctypes.data,
+                        ids.ctypes.data, n, row, 0, threads) == 0
+            assert np.array_equal(back, dense) and np.array_equal(pool, want)
+    ids = np.asarray([0, nhb], dtype=np.int64)
+    dense = np.zeros((2, row), dtype=np.uint8)
+    before = pool.copy()
+    assert L_fn(pool.ctypes.data, nhb, layers * row, 0, dense.ctypes.data, ids.ctypes.data, 2, row, 1,
+                threads) == _lib.KVC_ERR_OUT_OF_RANGE
+    assert "host block id" in _lib.last_error()
+    assert L_fn(pool.ctypes.data, nhb, layers * row, 2 * row + 1, dense.ctypes.data, ids.ctypes.data, 1, row,
+                1, threads) == _lib.KVC_ERR_INVALID_ARG
+    assert L_fn(None, nhb, layers * row, 0, dense.ctypes.data, ids.ctypes.data, 1, row, 1, threads) \
+        == _lib.KVC_ERR_INVALID_ARG
+    assert L_fn(pool.ctypes.data, nhb, layers * row, 0, dense.ctypes.data, ids.ctypes.data, 0, row, 1,
+                threads) == 0
+    assert np.array_equal(pool, before)
+
+
+def test_row_mover_runs_its_jobs_in_order_and_reports_errors():
+    """The queue form of the host row copies, without events (so on the CPU): jobs
+    finish in the order of their tickets, a wait covers everything before it, the
+    id list may go away after the submit, bad arguments fail at the submit."""
+    L = _lib.lib()
+    mover = ctypes.c_void_p()
+    assert L.kvc_row_mover_create(3, ctypes.byref(mover)) == 0
+    try:
+        rng = np.random.default_rng(11)
+        nhb, layers, row, n = 64, 4, 48 << 10, 40
+        pool = rng.integers(0, 255, size=(nhb, layers, row), dtype=np.uint8)
+        want = pool.copy()
+        dense = [rng.integers(0, 255, size=(n, row), dtype=np.uint8) for _ in range(layers)]
+        tickets = []
+        for layer in range(layers):
+            ids = rng.permutation(nhb)[:n].astype(np.int64)
+            want[ids, layer] = dense[layer]
+            tickets.append(L.kvc_row_mover_submit(mover, None, pool.ctypes.data, nhb, layers * row, layer * row,
+                                                  dense[layer].ctypes.data, ids.ctypes.data, n, row, 1))
+            ids[:] = -1                     # the mover keeps its own copy of the list
+        assert tickets == [0, 1, 2, 3]
+        assert L.kvc_row_mover_wait(mover, tickets[-1]) == 0
+        assert all(L.kvc_row_mover_done(mover, t) == 1 for t in tickets)
+        assert np.array_equal(pool, want)
+        # out of the pool again, one job reading what the job before it wrote
+        ids = rng.permutation(nhb)[:n].astype(np.int64)
+        back = np.zeros((n, row), dtype=np.uint8)
+        t1 = L.kvc_row_mover_submit(mover, None, pool.ctypes.data, nhb, layers * row, 2 * row,
+                                    dense[0].ctypes.data, ids.ctypes.data, n, row, 1)
+        t2 = L.kvc_row_mover_submit(mover, None, pool.ctypes.data, nhb, layers * row, 2 * row,
+                                    back.ctypes.data, ids.ctypes.data, n, row, 0)
+        assert (t1, t2) == (4, 5)
+        assert L.kvc_row_mover_wait(mover, t2) == 0
+        assert np.array_equal(back, dense[0])
+        bad = np.asarray([nhb], dtype=np.int64)
+        assert L.kvc_row_mover_submit(mover, None, pool.ctypes.data, nhb, layers * row, 0, back.ctypes.data,
+                                      bad.ctypes.data, 1, row, 1) == _lib.KVC_ERR_OUT_OF_RANGE
+        assert L.kvc_row_mover_wait(mover, 99) == _lib.KVC_ERR_INVALID_ARG
+        assert L.kvc_row_mover_submit(mover, None, pool.ctypes.data, nhb, layers * row, 0, back.ctypes.data,
+                                      bad.ctypes.data, 0, row, 1) == 6          # an empty job is a job
+        assert L.kvc_row_mover_wait(mover, 6) == 0
+    finally:
+        assert L.kvc_row_mover_destroy(mover) == 0
+    assert L.kvc_row_mover_destroy(None) == 0
+    assert L.kvc_row_mover_submit(None, None, None, 0, 0, 0, None, None, 0, 0, 0) == _lib.KVC_ERR_INVALID_ARG
+
+
 def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
     """include/kvcache.h compiles as C99 with no extensions, and a C translation
     unit that only knows the header links against libkvcache.so and runs the

@@ -23,9 +23,10 @@ def _busy(dev, n=3):
     return a
 
 
+@pytest.mark.parametrize("bounce", [True, False])
 @pytest.mark.parametrize("mode", ["direct", "staged", "auto"])
 @pytest.mark.parametrize("sync", ["events", "host"])
-def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync):
+def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync, bounce):
     """GPU->Host runs concurrently with the forward pass; layer l may be saved
     only after the model recorded post_events[l] (sync="events": the worker's
     stream waits for the event; sync="host": the doorbell itself is rung only
@@ -36,7 +37,8 @@ def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync):
     pool_np = random_pool((L, nb, 2, bs, H, D), 1)
     dpool = to_bf16(pool_np, gpu)
     handle = kvc.KVWorkerHandle.create(L, sync=sync)
-    worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle)
+    worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle,
+                          host_bounce_bytes=(1 << 30) if bounce else 0)
     hooks = kvc.LayerSyncHooks(handle)
     hooks.enable_record_after_execute = True
     try:
@@ -77,14 +79,92 @@ def test_write_through_waits_for_each_layers_kv_write(gpu, mode, sync):
         assert np.array_equal(bits_of(dpool), want_pool)
         assert np.array_equal(worker.host_kv_caches, want_host)
         assert handle.kv_queue.empty()
+        # four scattered host blocks, one layer per call: rows of 32 KiB, so the copy goes
+        # through the dense pinned buffer wherever the copy engines would carry it
+        assert worker.last_copy_went_through_host_bounce == (bounce and mode != "direct")
     finally:
         worker.close()
         handle.close()
 
 
+@pytest.mark.parametrize("budget_regions", [4, 2, 1])
+def test_scattered_host_blocks_layer_by_layer_through_the_dense_pinned_buffer(gpu, budget_regions):
+    """Forty blocks to scattered host blocks and back onto other pool blocks, one
+    layer per call over nine layers: more layers than the buffer has regions, so
+    regions are reused while host threads still empty (or the GPU still reads)
+    the earlier ones. With room for a single region the copy goes the usual way.
+    Host pool and GPU pool must be the oracle's after each direction."""
+    s = wl.LLAMA_3_2_1B
+    L, nb, nhb, n = 9, 128, 100, 40
+    pool_np = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), 31)
+    dpool = to_bf16(pool_np, gpu)
+    handle = kvc.KVWorkerHandle.create(L)
+    block_bytes = 2 * s.block_size * s.num_kv_heads * s.head_dim * 2
+    worker = kvc.KVWorker(dpool, nhb, kv_worker_handle=handle, host_copy_threads=3,
+                          host_bounce_bytes=budget_regions * n * block_bytes)
+    hooks = kvc.LayerSyncHooks(handle)
+    try:
+        worker.host_kv_caches[...] = sentinel_pool(worker.host_kv_caches.shape, 32)
+        rng = np.random.default_rng(33)
+        perm = rng.permutation(nb).astype(np.int64)
+        old, new = perm[:n], perm[n:2 * n]
+        host_ids = (rng.permutation(nhb // 2)[:n] * 2).astype(np.int64)      # never neighbours
+        gpu_np = pool_np.reshape(L, nb, -1).copy()
+        host_np = worker.host_kv_caches.copy()
+        orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids)
+
+        def run(maps, src, dst):
+            errors = []
+
+            def body():
+                try:
+                    asyncio.run(worker.copy_kv(maps, src, dst))
+                except Exception as exc:
+                    errors.append(exc)
+            th = threading.Thread(target=body, daemon=True)
+            th.start()
+            return th, errors
+
+        hooks.enable_record_after_execute = True
+        th, errors = run(_split(old, host_ids), kvc.Device.GPU, kvc.Device.Host)
+        for l in range(L):
+            _busy(gpu, 1)
+            hooks.post(l)
+        th.join(timeout=60)
+        assert not th.is_alive() and not errors, errors
+        assert worker.last_copy_went_through_host_bounce == (budget_regions >= 2)
+        assert np.array_equal(worker.host_kv_caches, host_np)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+
+        hooks.enable_record_after_execute = False
+        hooks.enable_wait_before_execute = True
+        hooks.timeout = 30
+        orc.c_load_blocks_from_host(gpu_np, host_np, host_ids, new)
+        th, errors = run(_split(host_ids, new), kvc.Device.Host, kvc.Device.GPU)
+        for l in range(L):
+            hooks.pre(l)
+        th.join(timeout=60)
+        assert not th.is_alive() and not errors, errors
+        torch.cuda.synchronize()
+        assert worker.last_copy_went_through_host_bounce == (budget_regions >= 2)
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+        assert np.array_equal(worker.host_kv_caches, host_np)
+        assert handle.model_queue.empty() and handle.kv_queue.empty()
+    finally:
+        worker.close()
+        handle.close()
+
+
+def _split(src, dst, pieces=3):
+    cuts = np.linspace(0, len(src), pieces + 1).astype(int)
+    return [kvc.BlockMapping.from_pairs(zip(src[a:b].tolist(), dst[a:b].tolist()))
+            for a, b in zip(cuts[:-1], cuts[1:])]
+
+
+@pytest.mark.parametrize("bounce", [True, False])
 @pytest.mark.parametrize("mode", ["direct", "staged", "auto"])
 @pytest.mark.parametrize("sync", ["events", "host"])
-def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode, sync):
+def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode, sync, bounce):
     """Host->GPU: the model waits per layer on pre_events[l] (after the doorbell;
     with sync="host" the doorbell alone, rung after the layer's load completed)
     and must then see that layer's fetched blocks."""
@@ -93,7 +173,8 @@ def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode, sync):
     pool_np = random_pool((L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim), 5)
     dpool = to_bf16(pool_np, gpu)
     handle = kvc.KVWorkerHandle.create(L, sync=sync)
-    worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle)
+    worker = kvc.KVWorker(dpool, nhb, swap_mode=mode, kv_worker_handle=handle,
+                          host_bounce_bytes=(1 << 30) if bounce else 0)
     hooks = kvc.LayerSyncHooks(handle)
     hooks.enable_wait_before_execute = True
     hooks.timeout = 30
@@ -120,6 +201,8 @@ def test_fetch_releases_each_layer_to_the_model_in_order(gpu, mode, sync):
             got = bits_of(seen[l]).reshape(len(dst), -1)
             assert np.array_equal(got, host[src, l]), f"layer {l} was read before its fetch landed"
         assert handle.model_queue.empty()
+        assert worker.last_copy_went_through_host_bounce == (bounce and mode != "direct")
+        assert np.array_equal(worker.host_kv_caches, host)      # the host pool is only read
     finally:
         worker.close()
         handle.close()
