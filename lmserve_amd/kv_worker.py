@@ -237,8 +237,8 @@ class KVWorker:
     host_bounce_bytes / host_copy_threads: layer-by-layer copies (the protocol
       with a handle) whose host blocks are scattered so that a layer's PCIe
       extents would be under 1 MiB in the mean go through a dense pinned buffer
-      of up to this many bytes (2 to 4 regions of one layer of the copy's
-      blocks; allocated on first use and kept) and this many host threads, in
+      of up to this many bytes (2 to `host_bounce_regions` regions of one layer
+      of the copy's blocks; allocated on first use and kept) and this many host threads, in
       the "auto" and "staged" modes: the copy engines carry each layer as one
       copy and the model's kernels keep running. 0 turns it off ("auto" then
       takes the direct kernel for such copies). A copy too large for the buffer,
@@ -265,7 +265,8 @@ class KVWorker:
         disk_preallocate: bool = False,
         validate: bool = False,
         host_bounce_bytes: int = 1 << 30,
-        host_copy_threads: int = 6,
+        host_copy_threads: int = 4,
+        host_bounce_regions: int = 4,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -292,6 +293,7 @@ class KVWorker:
         self.validate = bool(validate)
         self.host_bounce_bytes = int(host_bounce_bytes)
         self.host_copy_threads = int(host_copy_threads)
+        self.host_bounce_regions = max(2, int(host_bounce_regions))
         self._bounce = {"out": None, "in": None}
         self.last_copy_went_through_host_bounce = False
 
@@ -465,7 +467,7 @@ class KVWorker:
         if n * self.block_stride >= runs * _lib.get_tuning("auto_min_extent_bytes"):
             return None            # long extents: the copy engines take the rows as they lie
         slot_bytes = n * self.block_stride
-        slots = min(4, self.host_bounce_bytes // slot_bytes, self.num_layers)
+        slots = min(self.host_bounce_regions, self.host_bounce_bytes // slot_bytes, self.num_layers)
         if slots < min(2, self.num_layers):
             return None
         bounce = self._bounce[prepared.direction]
