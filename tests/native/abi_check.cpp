@@ -503,6 +503,32 @@ int main() {
     KVC_OK_OR_DIE(kvc_host_copy_rows(host_pool.data(), nhb, L * blk_bytes, layer * blk_bytes, back.data(),
                                      ids.data(), n, blk_bytes, 0, 3));
     expect_equal("kvc_host_copy_rows out of the pool", back.data(), dense.data(), dense.size() * 2);
+
+    // the queue form: a job that waits for "the rows have landed in the pinned buffer"
+    uint16_t* landing = (uint16_t*)kvc_host_alloc_pinned(dense.size() * 2);
+    if (!landing) { std::fprintf(stderr, "pinned alloc failed: %s\n", kvc_last_error_string()); return 4; }
+    void* d_rows;
+    HIP_OK(hipMalloc(&d_rows, dense.size() * 2));
+    std::vector<uint16_t> fresh(dense.size());
+    for (auto& x : fresh) x = (uint16_t)rng();
+    HIP_OK(hipMemcpy(d_rows, fresh.data(), fresh.size() * 2, hipMemcpyHostToDevice));
+    hipEvent_t landed;
+    HIP_OK(hipEventCreateWithFlags(&landed, hipEventDisableTiming));
+    kvc_row_mover* mover = nullptr;
+    KVC_OK_OR_DIE(kvc_row_mover_create(2, &mover));
+    HIP_OK(hipMemcpyAsync(landing, d_rows, fresh.size() * 2, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipEventRecord(landed, stream));
+    const int64_t ticket = kvc_row_mover_submit(mover, landed, host_pool.data(), nhb, L * blk_bytes, 2 * blk_bytes,
+                                                landing, ids.data(), n, blk_bytes, 1);
+    if (ticket != 0) { std::fprintf(stderr, "kvc_row_mover_submit: %s\n", kvc_last_error_string()); return 5; }
+    KVC_OK_OR_DIE(kvc_row_mover_wait(mover, ticket));
+    for (int64_t i = 0; i < n; ++i)
+      std::memcpy(&want_p[(size_t)((ids[i] * L + 2) * blk_elems)], &fresh[(size_t)(i * blk_elems)], blk_bytes);
+    expect_equal("kvc_row_mover job after an event", host_pool.data(), want_p.data(), host_pool.size() * 2);
+    KVC_OK_OR_DIE(kvc_row_mover_destroy(mover));
+    HIP_OK(hipEventDestroy(landed));
+    HIP_OK(hipFree(d_rows));
+    KVC_OK_OR_DIE(kvc_host_free_pinned(landing));
   }
 
   KVC_OK_OR_DIE(kvc_thread_release());

@@ -20,4 +20,4 @@ def test_c_abi_from_a_plain_hip_program(gpu):
     print(proc.stderr)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "ABI CHECK PASSED" in proc.stdout
-    assert proc.stdout.count("ok: ") == 38
+    assert proc.stdout.count("ok: ") == 39
