@@ -675,11 +675,11 @@ class KVWorker:
         if self.disk_tier is not None:
             self.disk_tier.close()
             self.disk_tier = None
-        self._host_pool.close()
-        for direction, bounce in self._bounce.items():
+        for direction, bounce in self._bounce.items():   # first: its mover still writes into the pool
             if bounce is not None:
                 bounce.close()
                 self._bounce[direction] = None
+        self._host_pool.close()
         self._staging = {}
         # let go of the pool now: the direction table holds bound methods, so the
         # worker is part of a reference cycle and would otherwise keep tens of GiB
