@@ -75,6 +75,12 @@ def parse_args():
     p.add_argument("--disk-blocks", type=int, default=256,
                    help="blocks moved by the disk-tier measurement (5 MiB each)")
     p.add_argument("--disk-dir", default=None, help="directory of the disk-tier file (default: tmp)")
+    p.add_argument("--hw-queues", type=int, default=8,
+                   help="GPU_MAX_HW_QUEUES for this process (0 = leave the environment alone). The write-through "
+                        "rows run the model's stream and the KV worker's streams in ONE process; with the "
+                        "runtime's default of 4 hardware queues two of those streams can land on one queue "
+                        "and wait for each other, which the reference's two processes (a set of queues "
+                        "each) never do")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
     return p.parse_args()
@@ -566,16 +572,19 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
     model_stream = torch.cuda.Stream()
     nbytes = n * L * s8.block_bytes
     out = []
-    variants = [("staged", 0, "staged swap"), ("direct", 0, "direct swap")]
+    variants = [("staged", 0, False, "staged swap"), ("direct", 0, False, "direct swap"),
+                ("staged", 1 << 30, True, "consecutive host blocks all the same through the dense pinned buffer: "
+                                          "1-D copies + host threads")]
     if scattered:
-        variants = [("auto", 1 << 30, "scattered host blocks; auto: one copy per layer into a dense pinned "
-                                      "buffer, rows placed by host threads"),
-                    ("auto", 0, "scattered host blocks; auto without the pinned buffer: the direct kernel"),
-                    ("staged", 0, "scattered host blocks; staged: the copy engines, one copy per block")]
-    for mode, bounce_bytes, label in variants:
+        variants = [("auto", 1 << 30, False, "scattered host blocks; auto: one copy per layer into a dense pinned "
+                                             "buffer, rows placed by host threads"),
+                    ("auto", 0, False, "scattered host blocks; auto without the pinned buffer: the direct kernel"),
+                    ("staged", 0, False, "scattered host blocks; staged: the copy engines, one copy per block")]
+    for mode, bounce_bytes, always, label in variants:
         handle = kvc.KVWorkerHandle.create(L)
         worker = kvc.KVWorker(pool, num_host_blocks=nhb, swap_mode=mode, kv_worker_handle=handle,
-                              host_bounce_bytes=bounce_bytes)
+                              host_bounce_bytes=bounce_bytes, host_bounce_always=always)
+        scattered_timing = scattered or always      # measured through the protocol, not through prepared calls
         hooks = kvc.LayerSyncHooks(handle)
 
         def protocol_alone(copy_maps, src, dst, saving):
@@ -624,9 +633,9 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
             e0, e1 = timed_forward()
             torch.cuda.synchronize()
             fwd_alone = e0.elapsed_time(e1)
-            prepared = None if scattered else worker.prepare_swap("out", maps)
-            swap_alone = protocol_alone(maps, kvc.Device.GPU, kvc.Device.Host, True) if scattered else None
-            for _ in range(0 if scattered else 4):               # the first pass touches the pinned pool
+            prepared = None if scattered_timing else worker.prepare_swap("out", maps)
+            swap_alone = protocol_alone(maps, kvc.Device.GPU, kvc.Device.Host, True) if scattered_timing else None
+            for _ in range(0 if scattered_timing else 4):               # the first pass touches the pinned pool
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for l in range(L):
@@ -638,17 +647,23 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
             def kv_thread():
                 asyncio.run(worker.copy_kv(maps, kvc.Device.GPU, kvc.Device.Host))
 
+            # three passes, the median by completion time reported (with all of them listed): the
+            # first pass of a new worker beside a busy GPU can hold one of its enqueues for the
+            # length of the forward pass, a one-time cost a server does not meet again
             hooks.enable_record_after_execute = True
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            th = threading.Thread(target=kv_thread)
-            th.start()
-            e0, e1 = timed_forward()
-            th.join(timeout=120)
-            torch.cuda.synchronize()
-            total = (time.perf_counter() - t0) * 1e3
+            passes = []
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                th = threading.Thread(target=kv_thread)
+                th.start()
+                e0, e1 = timed_forward()
+                th.join(timeout=120)
+                torch.cuda.synchronize()
+                passes.append(((time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)))
             hooks.enable_record_after_execute = False
-            fwd_with = e0.elapsed_time(e1)
+            total, fwd_with = sorted(passes)[1]
+            save_passes = [(round(f, 2), round(t, 2)) for t, f in passes]
             del prepared
             out.append({"name": f"write-through during a stand-in forward pass ({label}; {L} layers; {n} blocks x "
                                 f"{L} layers x 64 KiB saved layer by layer behind the model's post hooks)",
@@ -656,6 +671,7 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
                         "forward_with_write_through_ms": round(fwd_with, 2),
                         "forward_slowdown_pct": round(100.0 * (fwd_with / fwd_alone - 1.0), 1),
                         "both_done_after_ms": round(total, 2),
+                        "passes_forward_ms_and_done_after_ms": save_passes,
                         "one_after_the_other_ms": round(fwd_alone + swap_alone, 2),
                         "pcie_gbps_alone": round(nbytes / swap_alone / 1e6, 2),
                         "bytes_per_call": int(nbytes)})
@@ -663,9 +679,9 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
             # blocks of a request come back from the host layer by layer, and the model's layer l
             # waits for "layer l landed" before it runs
             in_maps = [kvc.BlockMapping.from_pairs(zip(host_ids, rng_ids.tolist()))]
-            prepared_in = None if scattered else worker.prepare_swap("in", in_maps)
-            fetch_alone = protocol_alone(in_maps, kvc.Device.Host, kvc.Device.GPU, False) if scattered else None
-            for _ in range(0 if scattered else 4):
+            prepared_in = None if scattered_timing else worker.prepare_swap("in", in_maps)
+            fetch_alone = protocol_alone(in_maps, kvc.Device.Host, kvc.Device.GPU, False) if scattered_timing else None
+            for _ in range(0 if scattered_timing else 4):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for l in range(L):
@@ -681,20 +697,24 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
 
             hooks.enable_wait_before_execute = True
             hooks.timeout = 60
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            th = threading.Thread(target=kv_fetch_thread)
-            th.start()
-            e0, e1 = timed_forward()
-            th.join(timeout=120)
-            torch.cuda.synchronize()
-            total = (time.perf_counter() - t0) * 1e3
+            passes = []
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                th = threading.Thread(target=kv_fetch_thread)
+                th.start()
+                e0, e1 = timed_forward()
+                th.join(timeout=120)
+                torch.cuda.synchronize()
+                passes.append(((time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)))
             hooks.enable_wait_before_execute = False
+            total, fwd_behind = sorted(passes)[1]
             out.append({"name": f"fetch during a stand-in forward pass ({label}; {L} layers; {n} blocks x {L} "
                                 f"layers x 64 KiB loaded layer by layer, each layer of the model waits for its own)",
                         "forward_alone_ms": round(fwd_alone, 2), "fetch_alone_ms": round(fetch_alone, 2),
-                        "forward_behind_the_fetch_ms": round(e0.elapsed_time(e1), 2),
+                        "forward_behind_the_fetch_ms": round(fwd_behind, 2),
                         "both_done_after_ms": round(total, 2),
+                        "passes_forward_ms_and_done_after_ms": [(round(f, 2), round(t, 2)) for t, f in passes],
                         "one_after_the_other_ms": round(fwd_alone + fetch_alone, 2),
                         "pcie_gbps_alone": round(nbytes / fetch_alone / 1e6, 2),
                         "bytes_per_call": int(nbytes)})
@@ -892,6 +912,8 @@ def main():
         print("bench.py measures one GPU only: this path has no cross-GPU step "
               f"(--gpus {args.gpus} is not supported)", file=sys.stderr)
         sys.exit(2)
+    if args.hw_queues > 0:
+        os.environ["GPU_MAX_HW_QUEUES"] = str(min(args.hw_queues, 32))   # read when the runtime starts
     import torch
 
     import lmserve_amd as kvc
@@ -1458,7 +1480,8 @@ def main():
                    "entry": "kvc_reshape_and_cache_layers (all layers in one launch)",
                    "launch": "one eager launch per step on torch's current stream",
                    "rotation": f"{ROTATE_DECODE} K/V source sets and slot sets cycled",
-                   "clock_prewarm_s": PREWARM_S},
+                   "clock_prewarm_s": PREWARM_S,
+                   "hardware_queues_of_the_process": os.environ.get("GPU_MAX_HW_QUEUES", "runtime default")},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_CFG2_ONE_LAUNCH

@@ -16,6 +16,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <cstdint>
 #include <cstdio>
@@ -138,7 +139,13 @@ struct kvc_row_mover {
       char text[256] = "";
       if (job.after) {
         hipError_t e = hipSetDevice(job.device);
-        if (e == hipSuccess) e = hipEventSynchronize(job.after);
+        // polled, not hipEventSynchronize: a thread that sleeps inside the runtime's wait
+        // was seen to hold up another thread's enqueue on the event's stream for as long
+        // as other streams kept the GPU busy
+        while (e == hipSuccess && (e = hipEventQuery(job.after)) == hipErrorNotReady) {
+          e = hipSuccess;
+          std::this_thread::sleep_for(std::chrono::microseconds(20));
+        }
         if (e != hipSuccess) {
           rc = KVC_ERR_HIP;
           std::snprintf(text, sizeof text, "kvc_row_mover: waiting for the event failed: %s", hipGetErrorString(e));

@@ -243,7 +243,12 @@ class KVWorker:
       copy and the model's kernels keep running. 0 turns it off ("auto" then
       takes the direct kernel for such copies). A copy too large for the buffer,
       or a second one of the same direction while the buffer is in use, goes
-      the usual way.
+      the usual way. `host_bounce_always=True` sends every layer-by-layer copy
+      that way, consecutive host blocks included: 5 % slower than the copy
+      engines on the rows as they lie (their one-layer transfers are 2-D copies)
+      while those are in their good state, and unaffected by the state they
+      fall into for some seconds after the process has freed device memory
+      (48 against 38 GB/s there).
     validate: check on the host that no block is the destination of two pairs of
       one GPU<->Host call (`ValueError`). The reference copies the pairs one
       after the other, so the later pair wins there (kv_worker.py:197-227);
@@ -267,6 +272,7 @@ class KVWorker:
         host_bounce_bytes: int = 1 << 30,
         host_copy_threads: int = 4,
         host_bounce_regions: int = 4,
+        host_bounce_always: bool = False,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -294,6 +300,7 @@ class KVWorker:
         self.host_bounce_bytes = int(host_bounce_bytes)
         self.host_copy_threads = int(host_copy_threads)
         self.host_bounce_regions = max(2, int(host_bounce_regions))
+        self.host_bounce_always = bool(host_bounce_always)
         self._bounce = {"out": None, "in": None}
         self.last_copy_went_through_host_bounce = False
 
@@ -464,7 +471,8 @@ class KVWorker:
             return None
         n, ids = prepared.n, prepared.host_ids
         runs = 1 + int(np.count_nonzero(ids[1:] != ids[:-1] + 1))
-        if n * self.block_stride >= runs * _lib.get_tuning("auto_min_extent_bytes"):
+        if not self.host_bounce_always and \
+                n * self.block_stride >= runs * _lib.get_tuning("auto_min_extent_bytes"):
             return None            # long extents: the copy engines take the rows as they lie
         slot_bytes = n * self.block_stride
         slots = min(self.host_bounce_regions, self.host_bounce_bytes // slot_bytes, self.num_layers)
