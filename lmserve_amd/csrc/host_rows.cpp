@@ -139,9 +139,8 @@ struct kvc_row_mover {
       char text[256] = "";
       if (job.after) {
         hipError_t e = hipSetDevice(job.device);
-        // polled, not hipEventSynchronize: a thread that sleeps inside the runtime's wait
-        // was seen to hold up another thread's enqueue on the event's stream for as long
-        // as other streams kept the GPU busy
+        // polled with short sleeps rather than hipEventSynchronize, which spins on a core
+        // for an event made without the blocking-sync flag (the caller's events are torch's)
         while (e == hipSuccess && (e = hipEventQuery(job.after)) == hipErrorNotReady) {
           e = hipSuccess;
           std::this_thread::sleep_for(std::chrono::microseconds(20));
