@@ -64,6 +64,8 @@ def parse_args():
                         "index (index preparation of a step: host construction vs one launch), "
                         "sweep (write / copy_blocks / plain kernel over launch sizes; not in the default), "
                         "calib (a plain elementwise kernel of known size, for counter calibration); "
+                        "queues (KV workers made one after the other beside a forward pass, to be run with "
+                        "--hw-queues 4 and 8; not in the default); "
                         "translation (the config 3 launch with dense, block-run and random slots, for "
                         "address-translation counter runs; not in the default); "
                         "'none' for the headline only")
@@ -796,6 +798,82 @@ def bench_small_write_through(torch, kvc, wl, dev):
     return out
 
 
+def bench_worker_states(torch, kvc, wl, dev, workers=9):
+    """Not in the default run (`--ops queues`, to be run with `--hw-queues 4` and
+    `--hw-queues 8`): KV workers made one after the other in this process, each
+    writing 1 GiB through to the host layer by layer beside the stand-in forward
+    pass, four passes each. With the runtime's four hardware queues some workers
+    spend their whole life in a slow state (their stream shares a queue with the
+    model's); the row lists every worker's passes and a plain copy on its stream."""
+    import asyncio
+    import threading
+
+    import numpy as np
+
+    s8 = wl.LLAMA_3_8B
+    L, nb, n = s8.num_layers, 4096, 512
+    pool = torch.empty(L, nb, 2, s8.block_size, s8.num_kv_heads, s8.head_dim, dtype=torch.bfloat16, device=dev)
+    a = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    b = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    c = torch.empty(4096, 4096, dtype=torch.bfloat16, device=dev)
+    ids = np.random.default_rng(5).permutation(nb)[:n]
+    model_stream = torch.cuda.Stream()
+    probe_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    probe_dst = torch.empty(64 << 20, dtype=torch.uint8).pin_memory()
+    rows = []
+    for w in range(workers):
+        dense = w % 3 != 2          # two workers on the dense-buffer path, then one on 2-D copies
+        host_ids = list(range(0, 2 * n, 2)) if (w % 2 and dense) else list(range(n))
+        maps = [kvc.BlockMapping.from_pairs(zip(ids.tolist(), host_ids))]
+        handle = kvc.KVWorkerHandle.create(L)
+        worker = kvc.KVWorker(pool, num_host_blocks=2 * n, swap_mode="staged", kv_worker_handle=handle,
+                              host_bounce_always=dense, host_bounce_bytes=(1 << 30) if dense else 0)
+        hooks = kvc.LayerSyncHooks(handle)
+        try:
+            def both(gemms):
+                hooks.enable_record_after_execute = True
+                th = threading.Thread(target=lambda: asyncio.run(worker.copy_kv(maps, kvc.Device.GPU, kvc.Device.Host)))
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                th.start()
+                e0.record(model_stream)
+                with torch.cuda.stream(model_stream):
+                    for l in range(L):
+                        for _ in range(gemms):
+                            torch.mm(a, b, out=c)
+                        hooks.post(l)
+                e1.record(model_stream)
+                th.join(timeout=120)
+                torch.cuda.synchronize()
+                hooks.enable_record_after_execute = False
+                return round(e0.elapsed_time(e1), 1), round((time.perf_counter() - t0) * 1e3, 1)
+
+            both(0)
+            both(4)                       # the one-time cost of a new worker's first pass beside a busy GPU
+            passes = [both(4) for _ in range(4)]
+            rates = []
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                with torch.cuda.stream(worker.dtoh_stream):
+                    probe_dst.copy_(probe_src, non_blocking=True)
+                worker.dtoh_stream.synchronize()
+                rates.append((64 << 20) / (time.perf_counter() - t0) / 1e9)
+            rows.append({"worker": w, "path": "dense pinned buffer + host threads" if dense else "2-D copies of the rows as they lie",
+                         "host_blocks": "every second" if (w % 2 and dense) else "consecutive",
+                         "passes_forward_ms_and_done_after_ms": passes,
+                         "plain_64MiB_copy_on_its_stream_gbps": round(max(rates), 1)})
+        finally:
+            worker.close()
+            handle.close()
+    del pool
+    torch.cuda.empty_cache()
+    return [{"name": f"{workers} KV workers one after the other in this process, 1 GiB write-through each beside the "
+                     f"stand-in forward pass (GPU_MAX_HW_QUEUES={os.environ.get('GPU_MAX_HW_QUEUES', 'default')})",
+             "workers": rows}]
+
+
 def bench_two_process_swap(torch, kvc, wl, dev):
     """The reference's deployment: the KV worker is a process of its own that maps
     the pool from an IPC handle (kv_worker.py:97-160, cli.py:115-121). A pool in a
@@ -1390,6 +1468,9 @@ def main():
             extra += bench_small_write_through(torch, kvc, wl, dev)
         except Exception as exc:
             log(f"write-through overlap skipped: {exc!r}")
+    if "queues" in ops:
+        with optional_section("worker states", torch):
+            extra += bench_worker_states(torch, kvc, wl, dev)
     if "twoproc" in ops:
         try:
             settle_copy_engines(torch, dev, "the two-process rows", args.settle_seconds)
