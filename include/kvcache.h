@@ -20,6 +20,12 @@
  *     (the reference leaves them undefined), host-resident id lists are
  *     rejected with KVC_ERR_OUT_OF_RANGE before anything is launched.
  *
+ * STABLE SURFACE. Everything declared in this file keeps its name, arguments and
+ * meaning until KVC_ABI_VERSION changes; kvc_abi_version() lets a binding check
+ * at load time. Launch-shape knobs, launch introspection, the host-side row
+ * mover and the run-descriptor write are declared in kvcache_experimental.h and
+ * may change without a version bump.
+ *
  * Pool layout (runtime/worker/llm_worker/model_worker.py:221-228):
  *   kv_caches[L, num_blocks, 2, block_size, H, D], contiguous; kv_caches[l] is
  *   the per-layer "NHD" paged cache handed to attention.
@@ -36,7 +42,7 @@
 extern "C" {
 #endif
 
-#define KVC_ABI_VERSION 5
+#define KVC_ABI_VERSION 6
 
 typedef enum kvc_status {
   KVC_OK = 0,
@@ -45,7 +51,9 @@ typedef enum kvc_status {
   KVC_ERR_OUT_OF_RANGE = -3,  /* a host-resident block id is outside its pool  */
   KVC_ERR_STAGING = -4,       /* staging buffer too small for the request      */
   KVC_ERR_HIP = -5,           /* a HIP runtime call failed (see error string)  */
-  KVC_ERR_IO = -6             /* a file operation of the disk tier failed      */
+  KVC_ERR_IO = -6,            /* a file operation of the disk tier failed      */
+  KVC_ERR_TIMEOUT = -7,       /* a host-side wait gave up at its deadline      */
+  KVC_ERR_CANCELLED = -8      /* a host-side wait was cancelled by the caller  */
 } kvc_status;
 
 /* how kvc_swap_out / kvc_swap_in move the bytes over PCIe */
@@ -62,57 +70,6 @@ typedef enum kvc_swap_mode {
 
 int kvc_abi_version(void);
 const char* kvc_last_error_string(void);
-
-/* Launch-shape knobs for measurement sweeps; process-wide, not thread-safe
- * against concurrent launches. No counterpart in the reference. Keys:
- *   "copy_unroll", "gather_unroll"   16-byte vectors per lane in the tile kernel (1, 2, 4, 8, 16;
- *                                     0 = by launch size)
- *   "copy_nt"                         non-temporal loads and stores in the tile kernel (0/1)
- *   "copy_order"                      1 = walk all blocks of a layer before the next layer
- *   "copy_max_wgs"                    grid cap of the tile kernel (0 = one workgroup per chunk)
- *   "direct_max_wgs"                  grid cap of the direct swap kernel
- *   "write_vpt"                       vectors per lane in the write kernel (0 = by size, 1, 2, 4, 8)
- *   "write_threads"                   lanes per workgroup in the write kernel (0 = by size, 64, 128, 256)
- *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads
- *   "write_order"                     1 = a token's workgroups are neighbours in the grid
- *   "write_planes"                    the plane kernel (lanes of a workgroup run over consecutive
- *                                     tokens of one (layer, K|V) plane): 0 = never, 1 = by row
- *                                     width and launch size, 2 = whenever the row shape allows
- *   "write_planes_vpt"                planes per lane in that kernel (0 = by size, 1, 2, 4, 8)
- *   "write_planes_threads"            lanes per workgroup in that kernel (0 = by rule, 256, 512, 1024)
- *   "write_planes_min_bytes"          rows under 1 KiB: source bytes per launch from which it runs
- *   "write_planes_max_vpr"            widest row it takes, in 16-byte vectors (at most 256)
- *   "write_pipe"                      1 = a lane waits for each of its loads before issuing the
- *                                     next, 0 = loads back to back, -1 = by rule
- *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
- *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier
- * Unknown key: KVC_ERR_INVALID_ARG. kvc_reset_tuning puts every knob back to its
- * default; kvc_tuning_modified counts the knobs that are not at their default. */
-int kvc_set_tuning(const char* key, int value);
-int kvc_get_tuning(const char* key, int* value);
-int kvc_reset_tuning(void);
-int kvc_tuning_modified(void);
-
-/* Shape of the most recent kernel launch made by the calling thread (for tests
- * and sweeps that must know which instantiation ran). No counterpart in the
- * reference. Unknown `what`: KVC_ERR_INVALID_ARG. */
-enum {
-  KVC_KERNEL_NONE = 0,
-  KVC_KERNEL_WRITE_ROWS = 1,        /* token per workgroup                          */
-  KVC_KERNEL_COPY_TILES = 2,        /* block copy, gather, scatter, direct swap     */
-  KVC_KERNEL_WRITE_PLANES = 3       /* lanes over consecutive tokens of one plane   */
-};
-enum {
-  KVC_LAUNCH_KERNEL = 0,       /* one of KVC_KERNEL_*                               */
-  KVC_LAUNCH_VEC_BYTES = 1,    /* bytes per load/store instruction per lane         */
-  KVC_LAUNCH_PER_LANE = 2,     /* vectors (or planes) in flight per lane            */
-  KVC_LAUNCH_THREADS = 3,      /* lanes per workgroup                               */
-  KVC_LAUNCH_GRID = 4,         /* workgroups                                        */
-  KVC_LAUNCH_NON_TEMPORAL = 5, /* bit 0 stores, bit 1 loads (tile kernel: both = 1) */
-  KVC_LAUNCH_PIPE = 6,         /* write kernels: 1 = a lane waits for each of its loads */
-  KVC_LAUNCH_SWAP_MODE = 7     /* the kvc_swap_mode this thread's last swap call ran in  */
-};
-int64_t kvc_last_launch_info(int what);
 
 /* ---------------------------------------------------------------------------
  * K/V write, slot-mapped.
@@ -234,6 +191,14 @@ int kvc_write_plan_destroy(kvc_write_plan* plan);
  * be ordered after this call (same stream, or an event). */
 int kvc_write_plan_resolve_slots(kvc_write_plan* plan, int64_t* slots, void* stream);
 
+/* The same with slots the caller already has on the device (the slot_mapping
+ * output of kvc_build_write_index): no launch, the plan only remembers the
+ * pointer. A plan made once over fixed-capacity index buffers and given their
+ * slot_mapping this way can be recorded into a hipGraph together with the index
+ * build: every replay then writes the step whose scalars the buffers hold.
+ * NULL returns the plan to page-table addressing. */
+int kvc_write_plan_set_slots(kvc_write_plan* plan, const int64_t* slots);
+
 /* ---------------------------------------------------------------------------
  * Index preparation for the paged write.
  * Replace the flashinfer.get_seq_lens / flashinfer.get_batch_indices_positions
@@ -269,13 +234,32 @@ int kvc_get_batch_indices_positions(const int32_t* append_indptr, const int32_t*
  * kv_indices is the concatenation of the requests' block tables. slot_mapping
  * may be NULL; a position outside its request's table yields slot -1.
  * Outputs: cu_seqlens_q, kv_indptr [batch_size+1], kv_last_page_len [batch_size],
- * batch_indices, positions (int32) and slot_mapping (int64) [nnz]. */
+ * batch_indices, positions (int32) and slot_mapping (int64) [nnz].
+ *
+ * Every size argument is a CAPACITY, so one recorded launch (a hipGraph node)
+ * serves every later step that fits: the step's own sizes are read from device
+ * memory. Requests with input_lens[b] = 0 (and num_blocks[b] = 0) pad the batch;
+ * per-token outputs from the step's token count up to nnz are set to -1, which
+ * every write entry point skips; num_kv_indices bounds the block-table array.
+ *
+ * Optional block runs (runs != NULL): a run is a maximal range of one request's
+ * new tokens that falls into one block -- consecutive tokens on the source side,
+ * consecutive entries of one block on the cache side, which is how a prefill
+ * chunk fills whole blocks (runtime/src/llm_engine/scheduler.rs:466-512).
+ *   run_indptr[b+1] = runs of requests 0..b                 (run_indptr[0] = 0)
+ *   runs[r] = {first token, block id (-1: outside the table), first entry, token count}
+ *   *num_runs = run_indptr[batch_size]
+ * runs is int32 [max_runs][4], 16-byte aligned; max_runs must be at least
+ * min(nnz, nnz / page_size + 2 * batch_size) (checked). Descriptors from
+ * *num_runs up to max_runs are set empty. */
 int kvc_build_write_index(const int32_t* input_lens, const int32_t* context_lens,
                           const int32_t* num_blocks, const int32_t* kv_indices,
                           int64_t batch_size, int64_t num_kv_indices, int64_t page_size,
                           int64_t nnz, int32_t* cu_seqlens_q, int32_t* kv_indptr,
                           int32_t* kv_last_page_len, int32_t* batch_indices,
-                          int32_t* positions, int64_t* slot_mapping, void* stream);
+                          int32_t* positions, int64_t* slot_mapping,
+                          int32_t* run_indptr, int32_t* runs, int32_t* num_runs,
+                          int64_t max_runs, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Block copy inside the pool (prefix-sharing copy-on-write).
@@ -344,6 +328,22 @@ int kvc_swap_in(void* pool, const void* host_pool,
                 void* staging, int64_t staging_bytes, int mode,
                 void* kernel_stream, void* copy_stream);
 
+/* Which way a KVC_SWAP_AUTO call goes, without making it: KVC_SWAP_STAGED or
+ * KVC_SWAP_DIRECT for n pairs with these HOST host ids (in the order the call
+ * would use: ascending for kvc_swap_out / kvc_swap_in, as given for the prepared
+ * calls), a layer range of num_layers_in_range layers and a staging buffer of
+ * staging_bytes. The direct kernel holds the PCIe rate whatever the ids are, but
+ * holds back the kernels of other streams while it runs (a forward pass beside a
+ * direct write-through of 1 GiB took 2.3 times as long on MI355X); a caller that
+ * runs a model on the same GPU should give AUTO a staging buffer of
+ * kvc_swap_staging_bytes(..., KVC_SWAP_STAGED, ...) and host blocks that form
+ * runs, or move the rows through a dense pinned buffer (kvcache_experimental.h).
+ * kvc_swap_last_mode: the mode the calling thread's most recent swap call ran in
+ * (-1 before the first). */
+int kvc_swap_resolve_mode(const int64_t* host_ids, int64_t n, int64_t num_layers_in_range,
+                          int64_t block_bytes, int64_t staging_bytes);
+int kvc_swap_last_mode(void);
+
 /* Orders the (gpu id, host id) pairs of one swap call by ascending host block id,
  * stably and in place (HOST arrays of n entries; no GPU work). The result of a
  * swap does not depend on the order of its pairs (the reference copies them one
@@ -394,8 +394,9 @@ int kvc_swap_in_prepared(void* pool, const void* host_pool, const int64_t* host_
 int kvc_thread_release(void);
 
 /* A direct swap that allocates nothing and needs no workspace. It has no
- * counterpart in the reference; it is for callers that cannot allocate: code
- * under HIP graph capture, serving loops and harnesses that forbid hipMalloc.
+ * counterpart in the reference; it is for callers that cannot allocate: tight
+ * serving loops and harnesses that forbid hipMalloc, and code that records its
+ * stream into a hipGraph (after one call outside the capture, see below).
  * kvc_swap_out / kvc_swap_in in KVC_SWAP_DIRECT mode with `staging` replaced by
  * a static device array inside the library (KVC_NOALLOC_MAX_BLOCKS id pairs,
  * 128 KiB per device, held until the process ends):
@@ -406,7 +407,12 @@ int kvc_thread_release(void);
  * kernel arguments, so the call consists of kernel launches on `stream` only:
  * no hipMalloc, no hipFree, no pinned bounce buffer, no memcpy, no events.
  * n > KVC_NOALLOC_MAX_BLOCKS: KVC_ERR_UNSUPPORTED, nothing launched. The first
- * call on a device looks up the array's address there.
+ * call on a device looks up the array's address there (hipGetSymbolAddress, which
+ * may load the code object and is not a stream operation): make one call, n = 1
+ * is enough, at start-up and outside any stream capture. A call moves its ids in
+ * packets of 448 pairs, one small launch each ahead of the copy kernel: up to
+ * 19 + 1 launches at the maximum size. A recorded call replays the ids it was
+ * recorded with.
  * Every call on one device shares that device's array: calls on one stream are
  * ordered by the stream; calls that overlap on different streams of one device
  * race on the id lists and must be ordered by the caller. */
@@ -505,6 +511,8 @@ int kvc_rotary_plan_destroy(kvc_rotary_plan* plan);
  * kvc_rotary_plan_run addresses the cache through `slots` (nnz int64 entries of
  * caller-owned device memory), as kvc_rotary_pos_emb_and_cache would. */
 int kvc_rotary_plan_resolve_slots(kvc_rotary_plan* plan, int64_t* slots, void* stream);
+/* As kvc_write_plan_set_slots. */
+int kvc_rotary_plan_set_slots(kvc_rotary_plan* plan, const int64_t* slots);
 
 /* The on-device half of a swap on its own: gather scattered pool blocks into a
  * dense device buffer laid out like the host pool, [n, layer_end-layer_begin,
@@ -578,56 +586,6 @@ int kvc_disk_save_blocks(kvc_disk* disk, const void* host_pool, int64_t num_host
 int kvc_disk_load_blocks(kvc_disk* disk, void* host_pool, int64_t num_host_blocks,
                          const int64_t* src_disk_ids, const int64_t* dst_host_ids, int64_t n,
                          int threads);
-
-/*
- * Host side of a one-layer swap to or from scattered host blocks, on host threads.
- * Serves
- *   _save_layer_kv_blocks_to_host     (runtime/worker/llm_worker/kv_worker.py:213-227)
- *   _load_layer_kv_blocks_from_host   (kv_worker.py:197-211)
- * when the layer's rows do not neighbour each other in the host pool
- * [num_host_blocks, L, block] (kv_worker.py:123-127): the PCIe leg of the layer
- * is then one copy between the GPU and a dense pinned buffer
- * (kvc_swap_out_prepared / kvc_swap_in_prepared with that buffer as a one-layer
- * host pool and host ids 0..n-1), and this call moves the rows between the
- * buffer and their places in the pool:
- *   to_pool != 0: pool[host_ids[i]] [pool_offset .. pool_offset + row_bytes) = dense[i]
- *   to_pool == 0: dense[i] = pool[host_ids[i]] [pool_offset .. pool_offset + row_bytes)
- * with pool_block_bytes the bytes of one host block over all layers,
- * pool_offset = layer * block bytes and dense rows row_bytes apart. Ids are
- * range-checked first. Synchronous, `threads` host threads (<= 0: 4; fewer for
- * small calls); no GPU work, callable from any thread. Rows of one call must be
- * distinct when to_pool != 0.
- */
-int kvc_host_copy_rows(void* host_pool, int64_t num_host_blocks, int64_t pool_block_bytes,
-                       int64_t pool_offset, void* dense, const int64_t* host_ids, int64_t n,
-                       int64_t row_bytes, int to_pool, int threads);
-
-/*
- * The same row copies as a queue with a thread of its own, so that the caller's
- * loop over the layers (kv_worker.py:249-295) never waits for the host side:
- * kvc_row_mover_submit checks the ids, copies them and returns a ticket
- * (0, 1, 2, ... in the order of the calls; a negative kvc_status on error);
- * the mover's thread takes the jobs in that order, waits for `after_event` first
- * when one is given (a hipEvent_t of the device that is current at the submit:
- * "the layer has landed in the dense buffer" for a save, "the GPU has read the
- * region" for a load), and moves the rows on `threads` host threads.
- * kvc_row_mover_done tells without blocking whether a ticket's job has finished
- * (1) or not (0); kvc_row_mover_wait blocks until it has, together with every
- * job submitted before it, and returns the status of the first job that failed
- * since the last wait. The event, the pool and the dense buffer must stay valid
- * until the job is done. kvc_row_mover_destroy finishes the queued jobs first.
- * One thread submits to a mover at a time; done and wait may be called from
- * any thread.
- */
-typedef struct kvc_row_mover kvc_row_mover;
-int kvc_row_mover_create(int threads, kvc_row_mover** out);
-int64_t kvc_row_mover_submit(kvc_row_mover* mover, void* after_event, void* host_pool,
-                             int64_t num_host_blocks, int64_t pool_block_bytes, int64_t pool_offset,
-                             void* dense, const int64_t* host_ids, int64_t n, int64_t row_bytes,
-                             int to_pool);
-int kvc_row_mover_done(kvc_row_mover* mover, int64_t ticket);
-int kvc_row_mover_wait(kvc_row_mover* mover, int64_t ticket);
-int kvc_row_mover_destroy(kvc_row_mover* mover);
 
 /* Pinned, device-addressable host memory for the host pool; replaces
  * pycuda.driver.pagelocked_empty (runtime/worker/llm_worker/kv_worker.py:123-127).

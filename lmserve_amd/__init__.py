@@ -9,6 +9,8 @@
     disk_tier   DiskTier (host <-> block file, native positional I/O)
     kv_pool     pool sizing, layer-sync handle and model-side hooks, hand-over to a second process
     kv_service  the KV worker as a process of its own (pool mapped from an IPC handle)
+    step_graph  KVWriteStep: fixed-capacity index buffers and plans, so that a step's index build
+                and per-layer writes can be recorded once into a hipGraph and replayed for later steps
 
 Every operator runs a hand-written HIP kernel from libkvcache.so through the
 C ABI of include/kvcache.h; the disk tier is host-side file I/O in the same
@@ -28,8 +30,10 @@ from .kv_worker import (BlockMapping, BlockMappingEntry, Device, KVWorker, Pinne
                         flatten_block_mappings)
 from .rotary import (PagedRotaryWritePlan, RotaryEmbedding, make_cos_sin_cache, rotary_pos_emb,
                      rotary_pos_emb_and_append_paged, rotary_pos_emb_and_cache)
-from .paged import (PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cache_layers,
-                    build_write_index, get_batch_indices_positions, get_seq_lens)
+from .paged import (BlockRuns, PagedKVWritePlan, append_paged_kv_cache, append_paged_kv_cache_layers,
+                    build_write_index, get_batch_indices_positions, get_seq_lens, max_block_runs,
+                    slot_block_runs, write_block_runs_layers)
+from .step_graph import KVWriteStep
 
 __all__ = [
     "copy_blocks", "fill_key_cache", "reshape_and_cache", "reshape_and_cache_layers",
@@ -45,5 +49,6 @@ __all__ = [
     "make_kv_worker_params", "open_kv_worker_params", "serve_kv_worker",
     "plan_cache",
     "InferInput", "KVIndexInputs", "make_kv_index_inputs", "to_device", "to_device_one_launch",
-    "build_write_index",
+    "build_write_index", "BlockRuns", "max_block_runs", "slot_block_runs", "write_block_runs_layers",
+    "KVWriteStep",
 ]

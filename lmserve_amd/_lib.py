@@ -1,4 +1,5 @@
-"""ctypes binding of libkvcache.so (the C ABI in include/kvcache.h).
+"""ctypes binding of libkvcache.so (the C ABI in include/kvcache.h and
+include/kvcache_experimental.h).
 
 There is no fallback: if the library is missing, `lib()` raises. Every
 operator in this package goes through the handles defined here.
@@ -20,6 +21,8 @@ KVC_ERR_OUT_OF_RANGE = -3
 KVC_ERR_STAGING = -4
 KVC_ERR_HIP = -5
 KVC_ERR_IO = -6
+KVC_ERR_TIMEOUT = -7
+KVC_ERR_CANCELLED = -8
 
 KVC_DISK_DIRECT = 1
 KVC_DISK_PREALLOCATE = 2
@@ -38,6 +41,7 @@ KVC_KERNEL_NONE = 0
 KVC_KERNEL_WRITE_ROWS = 1
 KVC_KERNEL_COPY_TILES = 2
 KVC_KERNEL_WRITE_PLANES = 3
+KVC_KERNEL_WRITE_RUNS = 4
 KVC_LAUNCH_KERNEL = 0
 KVC_LAUNCH_VEC_BYTES = 1
 KVC_LAUNCH_PER_LANE = 2
@@ -47,7 +51,7 @@ KVC_LAUNCH_NON_TEMPORAL = 5
 KVC_LAUNCH_PIPE = 6
 KVC_LAUNCH_SWAP_MODE = 7
 
-KVC_ABI_VERSION = 5
+KVC_ABI_VERSION = 6
 KVC_NOALLOC_MAX_BLOCKS = 8192
 
 KVC_DTYPE_BF16 = 0
@@ -98,7 +102,17 @@ SIGNATURES = {
     "kvc_get_seq_lens": (c_int, [_P, _P, _I64, _I64, _P, _P]),
     "kvc_get_batch_indices_positions": (c_int, [_P, _P, _I64, _I64, _P, _P, _P]),
     "kvc_build_write_index": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P,
-                                      _P]),
+                                      _P, _P, _P, _I64, _P]),
+    "kvc_slot_runs": (c_int, [_P, c_int, _I64, _I64, _P, _P, _I64, _P]),
+    "kvc_write_runs_layers": (c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                      _I64, _I64, _I64, _I64, _I64, _I64, c_int, _P]),
+    "kvc_write_plan_set_slots": (c_int, [_P, _P]),
+    "kvc_rotary_plan_set_slots": (c_int, [_P, _P]),
+    "kvc_swap_resolve_mode": (c_int, [_P, _I64, _I64, _I64, _I64]),
+    "kvc_swap_last_mode": (c_int, []),
+    "kvc_row_mover_submit_after_flag": (_I64, [_P, _P, _P, _I64, _I64, _I64, _P, _P, _I64, _I64, c_int]),
+    "kvc_row_mover_set_timeout_ms": (c_int, [_P, _I64]),
+    "kvc_row_mover_cancel": (c_int, [_P]),
     "kvc_rotary_pos_emb": (c_int, [_P, _P, _P, c_int, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                    _I64, _P, _P, _I64, _I64, c_int, _P]),
     "kvc_rotary_pos_emb_and_cache": (c_int, [_P, _P, _P, _P, c_int, _P, _I64, _I64, _I64, _I64, _I64,
@@ -214,6 +228,8 @@ def check(rc: int) -> None:
         raise IndexError(msg)
     if rc == KVC_ERR_IO:
         raise OSError(msg)
+    if rc == KVC_ERR_TIMEOUT:
+        raise TimeoutError(msg)
     raise KVCacheLibraryError(msg)
 
 
@@ -234,7 +250,7 @@ def reset_tuning() -> None:
 def last_swap_mode() -> int:
     """The KVC_SWAP_* mode the calling thread's most recent swap call ran in
     (what KVC_SWAP_AUTO chose); -1 before the first."""
-    return int(lib().kvc_last_launch_info(KVC_LAUNCH_SWAP_MODE))
+    return int(lib().kvc_swap_last_mode())
 
 
 def last_launch() -> dict:

@@ -28,6 +28,7 @@
 #include <vector>
 
 #include "kvcache.h"
+#include "kvcache_experimental.h"
 
 namespace kvc {
 int fail(int code, const char* fmt, ...);
@@ -111,9 +112,10 @@ struct kvc_row_mover {
   struct Job {
     RowCopy copy;
     std::vector<int64_t> ids;
-    hipEvent_t after;
-    int device;
-    int64_t ticket;
+    hipEvent_t after = nullptr;               // wait for this event of `device` first, or
+    const volatile int32_t* flag = nullptr;   // for this host word to become non-zero
+    int device = 0;
+    int64_t ticket = 0;
   };
   std::mutex mu;
   std::condition_variable has_jobs, progressed;
@@ -123,7 +125,55 @@ struct kvc_row_mover {
   char error[256] = "";
   bool stopping = false;
   int threads = 4;
+  // A job's wait gives up after this long (KVC_ERR_TIMEOUT) or when kvc_row_mover_cancel
+  // is called (KVC_ERR_CANCELLED). Either way the rows of that job stay where they are,
+  // and so do those of every job that was already queued behind it (they wait for work
+  // of the same stream): tickets below `skip_below` complete at once, without copying.
+  // Jobs submitted after that run as usual.
+  std::atomic<int64_t> timeout_ms{30000};
+  std::atomic<bool> cancel{false};
+  int64_t skip_below = 0;
   std::thread dispatcher;
+
+  // KVC_OK once the job's condition holds; the caller's thread sleeps in 20 us steps
+  // (hipEventSynchronize would spin on a core for an event made without the
+  // blocking-sync flag, and the caller's events are torch's)
+  int wait_for(const Job& job, char* text, size_t text_len) {
+    if (!job.after && !job.flag) return KVC_OK;
+    if (job.after) {
+      const hipError_t e = hipSetDevice(job.device);
+      if (e != hipSuccess) {
+        std::snprintf(text, text_len, "kvc_row_mover: hipSetDevice failed: %s", hipGetErrorString(e));
+        return KVC_ERR_HIP;
+      }
+    }
+    const auto begin = std::chrono::steady_clock::now();
+    for (;;) {
+      if (job.after) {
+        const hipError_t e = hipEventQuery(job.after);
+        if (e == hipSuccess) return KVC_OK;
+        if (e != hipErrorNotReady) {
+          std::snprintf(text, text_len, "kvc_row_mover: waiting for the event failed: %s", hipGetErrorString(e));
+          return KVC_ERR_HIP;
+        }
+      } else if (__atomic_load_n(job.flag, __ATOMIC_ACQUIRE) != 0) {
+        return KVC_OK;
+      }
+      if (cancel.load(std::memory_order_acquire)) {
+        std::snprintf(text, text_len, "kvc_row_mover: cancelled while job %lld waited", (long long)job.ticket);
+        return KVC_ERR_CANCELLED;
+      }
+      const int64_t limit = timeout_ms.load(std::memory_order_relaxed);
+      const auto waited = std::chrono::duration_cast<std::chrono::milliseconds>(
+                              std::chrono::steady_clock::now() - begin).count();
+      if (limit >= 0 && waited >= limit) {
+        std::snprintf(text, text_len, "kvc_row_mover: job %lld: %s not reached after %lld ms", (long long)job.ticket,
+                      job.after ? "event" : "host flag", (long long)waited);
+        return KVC_ERR_TIMEOUT;
+      }
+      std::this_thread::sleep_for(std::chrono::microseconds(20));
+    }
+  }
 
   void run() {
     for (;;) {
@@ -137,18 +187,18 @@ struct kvc_row_mover {
       }
       int rc = KVC_OK;
       char text[256] = "";
-      if (job.after) {
-        hipError_t e = hipSetDevice(job.device);
-        // polled with short sleeps rather than hipEventSynchronize, which spins on a core
-        // for an event made without the blocking-sync flag (the caller's events are torch's)
-        while (e == hipSuccess && (e = hipEventQuery(job.after)) == hipErrorNotReady) {
-          e = hipSuccess;
-          std::this_thread::sleep_for(std::chrono::microseconds(20));
-        }
-        if (e != hipSuccess) {
-          rc = KVC_ERR_HIP;
-          std::snprintf(text, sizeof text, "kvc_row_mover: waiting for the event failed: %s", hipGetErrorString(e));
-        }
+      bool skip;
+      {
+        std::lock_guard<std::mutex> lock(mu);
+        skip = job.ticket < skip_below;
+        if (!skip) cancel.store(false, std::memory_order_release);   // a job newer than the last cancel
+      }
+      if (skip) {
+        rc = KVC_ERR_CANCELLED;
+        std::snprintf(text, sizeof text, "kvc_row_mover: job %lld skipped after an earlier job gave up",
+                      (long long)job.ticket);
+      } else {
+        rc = wait_for(job, text, sizeof text);
       }
       if (rc == KVC_OK) {
         job.copy.host_ids = job.ids.data();
@@ -163,6 +213,7 @@ struct kvc_row_mover {
           status = rc;
           std::memcpy(error, text, sizeof error);
         }
+        if (rc == KVC_ERR_TIMEOUT) skip_below = next_ticket;   // everything queued so far stays where it is
         done_ticket = job.ticket;
       }
       progressed.notify_all();
@@ -188,17 +239,17 @@ int kvc_row_mover_create(int threads, kvc_row_mover** out) {
   return KVC_OK;
 }
 
-int64_t kvc_row_mover_submit(kvc_row_mover* mover, void* after_event, void* host_pool,
-                             int64_t num_host_blocks, int64_t pool_block_bytes, int64_t pool_offset,
-                             void* dense, const int64_t* host_ids, int64_t n, int64_t row_bytes,
-                             int to_pool) {
-  const char* fn = "kvc_row_mover_submit";
+static int64_t submit_job(const char* fn, kvc_row_mover* mover, void* after_event, const int32_t* flag,
+                          void* host_pool, int64_t num_host_blocks, int64_t pool_block_bytes,
+                          int64_t pool_offset, void* dense, const int64_t* host_ids, int64_t n,
+                          int64_t row_bytes, int to_pool) {
   if (!mover) return fail(KVC_ERR_INVALID_ARG, "%s: null mover", fn);
   const int rc = check_rows(fn, host_pool, num_host_blocks, pool_block_bytes, pool_offset, dense, host_ids,
                             n, row_bytes);
   if (rc != KVC_OK) return rc;
   kvc_row_mover::Job job;
   job.after = (hipEvent_t)after_event;
+  job.flag = flag;
   job.device = 0;
   if (after_event && hipGetDevice(&job.device) != hipSuccess)
     return fail(KVC_ERR_HIP, "%s: hipGetDevice failed", fn);
@@ -224,6 +275,36 @@ int64_t kvc_row_mover_submit(kvc_row_mover* mover, void* after_event, void* host
   }
   mover->has_jobs.notify_one();
   return ticket;
+}
+
+int64_t kvc_row_mover_submit(kvc_row_mover* mover, void* after_event, void* host_pool,
+                             int64_t num_host_blocks, int64_t pool_block_bytes, int64_t pool_offset,
+                             void* dense, const int64_t* host_ids, int64_t n, int64_t row_bytes,
+                             int to_pool) {
+  return submit_job("kvc_row_mover_submit", mover, after_event, nullptr, host_pool, num_host_blocks,
+                    pool_block_bytes, pool_offset, dense, host_ids, n, row_bytes, to_pool);
+}
+
+int64_t kvc_row_mover_submit_after_flag(kvc_row_mover* mover, const int32_t* flag, void* host_pool,
+                                        int64_t num_host_blocks, int64_t pool_block_bytes,
+                                        int64_t pool_offset, void* dense, const int64_t* host_ids,
+                                        int64_t n, int64_t row_bytes, int to_pool) {
+  return submit_job("kvc_row_mover_submit_after_flag", mover, nullptr, flag, host_pool, num_host_blocks,
+                    pool_block_bytes, pool_offset, dense, host_ids, n, row_bytes, to_pool);
+}
+
+int kvc_row_mover_set_timeout_ms(kvc_row_mover* mover, int64_t timeout_ms) {
+  if (!mover) return fail(KVC_ERR_INVALID_ARG, "kvc_row_mover_set_timeout_ms: null mover");
+  mover->timeout_ms.store(timeout_ms, std::memory_order_relaxed);
+  return KVC_OK;
+}
+
+int kvc_row_mover_cancel(kvc_row_mover* mover) {
+  if (!mover) return fail(KVC_ERR_INVALID_ARG, "kvc_row_mover_cancel: null mover");
+  std::lock_guard<std::mutex> lock(mover->mu);
+  mover->skip_below = mover->next_ticket;                  // every job submitted so far
+  mover->cancel.store(true, std::memory_order_release);    // the one that is waiting right now
+  return KVC_OK;
 }
 
 int kvc_row_mover_done(kvc_row_mover* mover, int64_t ticket) {

@@ -42,6 +42,7 @@
 
 #include "common.h"
 #include "kvcache.h"
+#include "kvcache_experimental.h"
 
 // ---------------------------------------------------------------------------
 // error plumbing (shared with the other translation units through common.h)
@@ -88,6 +89,9 @@ struct Tuning {
                             // with 48-64 workgroups (more cost a 16 MiB one-layer launch 2-4 %),
                             // both directions at once want 96 or more each (91-92 against 87 GB/s
                             // in sum); the rest of the GPU stays free for the model
+  int runs_unroll = 0;       // write_runs: 16-byte vectors per lane (1, 2, 4), 0 = by size
+  int runs_order = 0;        // write_runs: 1 = all runs of a plane are neighbours in the grid
+  int runs_nt = 1;           // write_runs: non-temporal loads and stores
   int auto_min_extent_bytes = 1 << 20;  // KVC_SWAP_AUTO: mean bytes per PCIe copy from which a call
                                         // goes through the copy engines. A copy costs about 10 us
                                         // beyond its transfer time (65 % of the link rate at 1 MiB,
@@ -124,6 +128,9 @@ Knob* knobs(int* count) {
       {"write_pipe", &g_tune.write_pipe, -1},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 96},
       {"auto_min_extent_bytes", &g_tune.auto_min_extent_bytes, 1 << 20},
+      {"runs_unroll", &g_tune.runs_unroll, 0},
+      {"runs_order", &g_tune.runs_order, 0},
+      {"runs_nt", &g_tune.runs_nt, 1},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
   };
@@ -461,6 +468,90 @@ __global__ __launch_bounds__(kThreads) void copy_tiles_kernel(TileArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// write_runs_kernel
+// ---------------------------------------------------------------------------
+// The K/V write as a tile copy. A block run (see build_write_index_kernel) of
+// one (layer, K|V) plane is contiguous on both sides when rows are dense: up to
+// block_size rows of the source plane go to consecutive entries of one cache
+// block. A workgroup owns a chunk of 256 lanes x UNROLL x VEC bytes of one
+// (run, plane), reads the run's descriptor on the scalar unit, issues all its
+// loads before its first store. The grid is sized for `max_runs` runs; the
+// number of runs of this step is read from device memory, so a recorded launch
+// serves steps of any size up to that capacity.
+struct RunArgs {
+  const char* key;
+  const char* value;
+  char* key_cache;
+  char* value_cache;
+  const int32_t* runs;      // [max_runs][4]: first token, block id, first entry, token count
+  const int32_t* num_runs;  // device scalar
+  uint32_t max_runs, num_planes, chunks_per_run;
+  uint32_t vecs_per_row;
+  int vpr_shift;            // log2(vecs_per_row) or -1
+  int plane_major;          // 1: blockIdx = (plane, run, chunk); 0: (run, plane, chunk)
+  int64_t key_token_stride, value_token_stride;  // bytes
+  int64_t key_layer_stride, value_layer_stride;
+  int64_t cache_block_stride, cache_slot_stride, cache_layer_stride;
+  int64_t num_cache_blocks, block_size, num_tokens;
+};
+
+template <int VEC, int UNROLL, bool NT>
+__global__ __launch_bounds__(kThreads) void write_runs_kernel(RunArgs a) {
+  using V = typename VecOf<VEC>::type;
+  const uint32_t chunk = blockIdx.x % a.chunks_per_run;
+  const uint32_t rest = blockIdx.x / a.chunks_per_run;
+  uint32_t run, plane;
+  if (a.plane_major) {
+    plane = rest / a.max_runs;
+    run = rest - plane * a.max_runs;
+  } else {
+    run = rest / a.num_planes;
+    plane = rest - run * a.num_planes;
+  }
+  if (run >= (uint32_t)*a.num_runs) return;
+  const int4 d = reinterpret_cast<const int4*>(a.runs)[run];
+  const int64_t first_token = d.x, block = d.y, entry = d.z, count = d.w;
+  if (block < 0 || block >= a.num_cache_blocks || count <= 0 || entry < 0 ||
+      entry + count > a.block_size || first_token < 0 || first_token + count > a.num_tokens)
+    return;
+  const uint32_t nvec = (uint32_t)count * a.vecs_per_row;
+  const uint32_t v_first = chunk * (kThreads * UNROLL);
+  if (v_first >= nvec) return;  // a short run needs fewer chunks than a full one
+  const int64_t layer = plane >> 1;
+  const bool is_v = plane & 1u;
+  const char* src = (is_v ? a.value + layer * a.value_layer_stride : a.key + layer * a.key_layer_stride);
+  const int64_t src_token_stride = is_v ? a.value_token_stride : a.key_token_stride;
+  src += first_token * src_token_stride;
+  char* dst = (is_v ? a.value_cache : a.key_cache) + layer * a.cache_layer_stride +
+              block * a.cache_block_stride + entry * a.cache_slot_stride;
+  const auto split = [&](uint32_t v, uint32_t& tok, uint32_t& vec) {
+    if (a.vpr_shift >= 0) {
+      tok = v >> a.vpr_shift;
+      vec = v & (a.vecs_per_row - 1u);
+    } else {
+      tok = v / a.vecs_per_row;
+      vec = v - tok * a.vecs_per_row;
+    }
+  };
+  V data[UNROLL];
+#pragma unroll
+  for (int j = 0; j < UNROLL; ++j) {
+    uint32_t tok, vec;
+    split(min(v_first + j * kThreads + threadIdx.x, nvec - 1u), tok, vec);
+    data[j] = ld<NT>(reinterpret_cast<const V*>(src + (int64_t)tok * src_token_stride + (int64_t)vec * VEC));
+  }
+#pragma unroll
+  for (int j = 0; j < UNROLL; ++j) {
+    const uint32_t v = v_first + j * kThreads + threadIdx.x;
+    if (v < nvec) {
+      uint32_t tok, vec;
+      split(v, tok, vec);
+      st<NT>(reinterpret_cast<V*>(dst + (int64_t)tok * a.cache_slot_stride + (int64_t)vec * VEC), data[j]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // index kernels
 // ---------------------------------------------------------------------------
 __global__ void seq_lens_kernel(const int32_t* kv_indptr, const int32_t* last_page_len,
@@ -509,61 +600,89 @@ __global__ void batch_indices_positions_kernel(const int32_t* append_indptr,
 }
 
 // Whole index preparation of a step in one launch (one workgroup): prefix sums
-// of the per-request new-token counts and block counts, the last-page fill, and
-// for every new token its request, absolute position and slot.
+// of the per-request new-token counts, block counts and block-run counts, the
+// last-page fill, and for every new token its request, absolute position and
+// slot. The per-token outputs are CAPACITY-bound: entries from the step's token
+// count up to `nnz` are filled with -1 (a request index, position and slot every
+// write kernel skips), so a launch recorded once for `nnz` tokens serves steps
+// of any smaller size.
+// A block run is a maximal range of a request's new tokens that falls into one
+// block: consecutive tokens on the source side, consecutive cache entries on
+// the other. Its descriptor is four int32: first token, block id, first entry,
+// token count. The first token of every run writes it.
 constexpr int kPrepThreads = 1024;
 
 __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
     const int32_t* input_lens, const int32_t* context_lens, const int32_t* num_blocks,
     const int32_t* kv_indices, int32_t batch_size, int64_t num_kv_indices, int32_t page_size,
     int64_t nnz, int32_t* cu_seqlens_q, int32_t* kv_indptr, int32_t* kv_last_page_len,
-    int32_t* batch_indices, int32_t* positions, int64_t* slot_mapping) {
-  __shared__ int32_t carry[2];
+    int32_t* batch_indices, int32_t* positions, int64_t* slot_mapping, int32_t* run_indptr,
+    int32_t* runs, int32_t* num_runs, int64_t max_runs) {
+  __shared__ int32_t carry[3];
   __shared__ int32_t part_q[kPrepThreads];
   __shared__ int32_t part_b[kPrepThreads];
+  __shared__ int32_t part_r[kPrepThreads];
   const int tid = threadIdx.x;
   if (tid == 0) {
-    carry[0] = 0;
-    carry[1] = 0;
+    carry[0] = carry[1] = carry[2] = 0;
     cu_seqlens_q[0] = 0;
     kv_indptr[0] = 0;
+    if (run_indptr) run_indptr[0] = 0;
   }
+  // every descriptor starts out empty: a run whose first token lies beyond `nnz` is never written
+  if (runs)
+    for (int64_t r = tid; r < max_runs; r += kPrepThreads)
+      reinterpret_cast<int4*>(runs)[r] = make_int4(0, -1, 0, 0);
   __syncthreads();
   // chunked inclusive scan (Hillis-Steele inside a chunk of kPrepThreads requests)
   for (int32_t base = 0; base < batch_size; base += kPrepThreads) {
     const int32_t b = base + tid;
     const int32_t q = b < batch_size ? input_lens[b] : 0;
     const int32_t n = b < batch_size ? num_blocks[b] : 0;
+    const int32_t ctx = b < batch_size ? context_lens[b] : 0;
+    // runs of the request: the blocks its new positions [ctx - q, ctx) touch
+    const int32_t nr = (q > 0 && ctx >= q) ? (ctx - 1) / page_size - (ctx - q) / page_size + 1 : 0;
     part_q[tid] = q;
     part_b[tid] = n;
+    part_r[tid] = nr;
     __syncthreads();
     for (int off = 1; off < kPrepThreads; off <<= 1) {
       const int32_t aq = tid >= off ? part_q[tid - off] : 0;
       const int32_t ab = tid >= off ? part_b[tid - off] : 0;
+      const int32_t ar = tid >= off ? part_r[tid - off] : 0;
       __syncthreads();
       part_q[tid] += aq;
       part_b[tid] += ab;
+      part_r[tid] += ar;
       __syncthreads();
     }
     if (b < batch_size) {
       cu_seqlens_q[b + 1] = carry[0] + part_q[tid];
       kv_indptr[b + 1] = carry[1] + part_b[tid];
-      const int32_t ctx = context_lens[b];
+      if (run_indptr) run_indptr[b + 1] = carry[2] + part_r[tid];
       kv_last_page_len[b] = ctx > 0 ? (ctx - 1) % page_size + 1 : 0;
     }
     __syncthreads();
     if (tid == kPrepThreads - 1) {
       carry[0] += part_q[tid];
       carry[1] += part_b[tid];
+      carry[2] += part_r[tid];
     }
     __syncthreads();
   }
+  if (tid == 0 && num_runs) *num_runs = (int32_t)(carry[2] < max_runs ? carry[2] : max_runs);
   // per token: find its request by bisection over the prefix sums just written
   // (visible to the whole workgroup after the barrier above); the request's new
   // tokens occupy positions [context - input, context)
   const int64_t total = cu_seqlens_q[batch_size];
   const int64_t limit = total < nnz ? total : nnz;
-  for (int64_t out = tid; out < limit; out += kPrepThreads) {
+  for (int64_t out = tid; out < nnz; out += kPrepThreads) {
+    if (out >= limit) {  // beyond this step's tokens: entries every write kernel skips
+      batch_indices[out] = -1;
+      positions[out] = -1;
+      if (slot_mapping) slot_mapping[out] = -1;
+      continue;
+    }
     int32_t lo = 0, hi = batch_size;  // invariant: cu[lo] <= out < cu[hi]
     while (hi - lo > 1) {
       const int32_t mid = (lo + hi) >> 1;
@@ -573,16 +692,102 @@ __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
     const int32_t b = lo;
     const int32_t begin = cu_seqlens_q[b];
     const int32_t n_new = cu_seqlens_q[b + 1] - begin;
-    const int32_t pos = context_lens[b] - n_new + (int32_t)(out - begin);
+    const int32_t j = (int32_t)(out - begin);
+    const int32_t pos = context_lens[b] - n_new + j;
     batch_indices[out] = b;
     positions[out] = pos;
-    if (slot_mapping) {
-      const int64_t it = (int64_t)kv_indptr[b] + pos / page_size;
-      const int64_t table_end = kv_indptr[b + 1] < num_kv_indices ? kv_indptr[b + 1] : num_kv_indices;
-      slot_mapping[out] = (pos >= 0 && it >= 0 && it < table_end)
-                              ? (int64_t)kv_indices[it] * page_size + pos % page_size
-                              : -1;
+    const int64_t it = (int64_t)kv_indptr[b] + pos / page_size;
+    const int64_t table_end = kv_indptr[b + 1] < num_kv_indices ? kv_indptr[b + 1] : num_kv_indices;
+    const bool in_table = pos >= 0 && it >= 0 && it < table_end;
+    if (slot_mapping)
+      slot_mapping[out] = in_table ? (int64_t)kv_indices[it] * page_size + pos % page_size : -1;
+    if (runs && pos >= 0 && context_lens[b] >= n_new && (j == 0 || pos % page_size == 0)) {
+      const int32_t first_pos = context_lens[b] - n_new;
+      const int64_t r = (int64_t)run_indptr[b] + (pos / page_size - first_pos / page_size);
+      if (r >= 0 && r < max_runs) {
+        int64_t count = page_size - pos % page_size;
+        if (count > n_new - j) count = n_new - j;
+        if (count > nnz - out) count = nnz - out;
+        reinterpret_cast<int4*>(runs)[r] =
+            make_int4((int32_t)out, in_table ? kv_indices[it] : -1, pos % page_size, (int32_t)count);
+      }
     }
+  }
+}
+
+// Block runs of an arbitrary slot mapping (one workgroup): token t opens a run
+// when its slot is valid and is not the successor of token t-1's slot inside
+// the same block. Same descriptors as the index build writes.
+__global__ __launch_bounds__(kPrepThreads) void slot_runs_kernel(const void* slot_mapping, int slot_bytes,
+                                                                 int64_t num_tokens, int64_t block_size,
+                                                                 int32_t* runs, int32_t* num_runs,
+                                                                 int64_t max_runs) {
+  __shared__ int32_t part[kPrepThreads];
+  __shared__ int32_t carry;
+  const int tid = threadIdx.x;
+  const auto slot_of = [&](int64_t t) -> int64_t {
+    return slot_bytes == 8 ? reinterpret_cast<const int64_t*>(slot_mapping)[t]
+                           : (int64_t) reinterpret_cast<const int32_t*>(slot_mapping)[t];
+  };
+  const auto opens = [&](int64_t t, int64_t s) {
+    if (s < 0) return false;
+    if (t == 0 || s % block_size == 0) return true;
+    return slot_of(t - 1) != s - 1;
+  };
+  if (tid == 0) carry = 0;
+  for (int64_t r = tid; r < max_runs; r += kPrepThreads)
+    reinterpret_cast<int4*>(runs)[r] = make_int4(0, -1, 0, 0);
+  __syncthreads();
+  // pass 1: the first token of a run writes its descriptor with a count of 0
+  for (int64_t base = 0; base < num_tokens; base += kPrepThreads) {
+    const int64_t t = base + tid;
+    const int64_t s = t < num_tokens ? slot_of(t) : -1;
+    const bool head = t < num_tokens && opens(t, s);
+    part[tid] = head ? 1 : 0;
+    __syncthreads();
+    for (int off = 1; off < kPrepThreads; off <<= 1) {
+      const int32_t add = tid >= off ? part[tid - off] : 0;
+      __syncthreads();
+      part[tid] += add;
+      __syncthreads();
+    }
+    if (head) {
+      const int64_t r = (int64_t)carry + part[tid] - 1;
+      if (r < max_runs)
+        reinterpret_cast<int4*>(runs)[r] =
+            make_int4((int32_t)t, (int32_t)(s / block_size), (int32_t)(s % block_size), 0);
+    }
+    __syncthreads();
+    if (tid == kPrepThreads - 1) carry += part[tid];
+    __syncthreads();
+  }
+  if (tid == 0) {
+    *num_runs = (int32_t)(carry < max_runs ? carry : max_runs);
+    carry = 0;
+  }
+  __syncthreads();
+  // pass 2: the last token of a run writes the count (descriptors of pass 1 are
+  // visible to the workgroup after the barriers above)
+  for (int64_t base = 0; base < num_tokens; base += kPrepThreads) {
+    const int64_t t = base + tid;
+    const int64_t s = t < num_tokens ? slot_of(t) : -1;
+    const bool head = t < num_tokens && opens(t, s);
+    part[tid] = head ? 1 : 0;
+    __syncthreads();
+    for (int off = 1; off < kPrepThreads; off <<= 1) {
+      const int32_t add = tid >= off ? part[tid - off] : 0;
+      __syncthreads();
+      part[tid] += add;
+      __syncthreads();
+    }
+    if (t < num_tokens && s >= 0) {
+      const bool last = t + 1 == num_tokens || opens(t + 1, slot_of(t + 1)) || slot_of(t + 1) < 0;
+      const int64_t r = (int64_t)carry + part[tid] - 1;
+      if (last && r >= 0 && r < max_runs) runs[4 * r + 3] = (int32_t)(t - runs[4 * r] + 1);
+    }
+    __syncthreads();
+    if (tid == kPrepThreads - 1) carry += part[tid];
+    __syncthreads();
   }
 }
 
@@ -922,6 +1127,90 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     KVC_HIP(hipGetLastError());
   }
   g_last = LastLaunch{KVC_KERNEL_WRITE_ROWS, vec, l.vpt, l.threads, l.grid, (l.nt ? 1 : 0) | (l.ntl ? 2 : 0), a.pipe};
+  return KVC_OK;
+}
+
+// --------------------------- run write launch -------------------------------
+template <int VEC, int UNROLL>
+void launch_runs_nt(const RunArgs& a, unsigned grid, hipStream_t s, bool nt) {
+  if (nt) hipLaunchKernelGGL((write_runs_kernel<VEC, UNROLL, true>), dim3(grid), dim3(kThreads), 0, s, a);
+  else hipLaunchKernelGGL((write_runs_kernel<VEC, UNROLL, false>), dim3(grid), dim3(kThreads), 0, s, a);
+}
+
+template <int VEC>
+void launch_runs_unroll(const RunArgs& a, int unroll, unsigned grid, hipStream_t s, bool nt) {
+  switch (unroll) {
+    case 1: launch_runs_nt<VEC, 1>(a, grid, s, nt); break;
+    case 2: launch_runs_nt<VEC, 2>(a, grid, s, nt); break;
+    default: launch_runs_nt<VEC, 4>(a, grid, s, nt); break;
+  }
+}
+
+// The K/V write of `max_runs` block runs x 2 * num_layers planes as tile copies.
+int run_write_runs(const char* fn, const void* key, const void* value, void* kc, void* vc,
+                   const int32_t* runs, const int32_t* num_runs, int64_t max_runs, const WriteGeom& g,
+                   void* stream) {
+  int rc = check_write_geom(fn, key, value, kc, vc, g);
+  if (rc != KVC_OK) return rc;
+  if (max_runs < 0) return fail(KVC_ERR_INVALID_ARG, "%s: negative max_runs", fn);
+  if (g.num_tokens == 0 || g.row_elems == 0 || g.num_layers == 0 || max_runs == 0) return KVC_OK;
+  if (!runs || !num_runs) return fail(KVC_ERR_INVALID_ARG, "%s: null run list", fn);
+  if ((uintptr_t)runs % 16) return fail(KVC_ERR_INVALID_ARG, "%s: the run list must be 16-byte aligned", fn);
+  if (g.num_tokens > 0x7fffffffll) return fail(KVC_ERR_UNSUPPORTED, "%s: %lld tokens", fn, (long long)g.num_tokens);
+  const int64_t E = g.elem_bytes;
+  const int vec = common_vec({(uint64_t)(uintptr_t)key, (uint64_t)(uintptr_t)value,
+                              (uint64_t)(uintptr_t)kc, (uint64_t)(uintptr_t)vc,
+                              (uint64_t)(g.row_elems * E), (uint64_t)(g.key_token_stride * E),
+                              (uint64_t)(g.value_token_stride * E),
+                              (uint64_t)(g.key_layer_stride * E), (uint64_t)(g.value_layer_stride * E),
+                              (uint64_t)(g.cache_block_stride * E), (uint64_t)(g.cache_slot_stride * E),
+                              (uint64_t)(g.cache_layer_stride * E)});
+  RunArgs a{};
+  a.key = (const char*)key;
+  a.value = (const char*)value;
+  a.key_cache = (char*)kc;
+  a.value_cache = (char*)vc;
+  a.runs = runs;
+  a.num_runs = num_runs;
+  a.max_runs = (uint32_t)max_runs;
+  a.num_planes = (uint32_t)(2 * g.num_layers);
+  a.vecs_per_row = (uint32_t)(g.row_elems * E / vec);
+  a.vpr_shift = log2_exact(a.vecs_per_row);
+  a.plane_major = g_tune.runs_order;
+  a.key_token_stride = g.key_token_stride * E;
+  a.value_token_stride = g.value_token_stride * E;
+  a.key_layer_stride = g.key_layer_stride * E;
+  a.value_layer_stride = g.value_layer_stride * E;
+  a.cache_block_stride = g.cache_block_stride * E;
+  a.cache_slot_stride = g.cache_slot_stride * E;
+  a.cache_layer_stride = g.cache_layer_stride * E;
+  a.num_cache_blocks = g.num_cache_blocks;
+  a.block_size = g.block_size;
+  a.num_tokens = g.num_tokens;
+  const int64_t vecs_per_run = g.block_size * (int64_t)a.vecs_per_row;  // of a full run
+  if (vecs_per_run > 0x7fffffffll)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per run exceed 2^31", fn, (long long)vecs_per_run);
+  // Vectors per lane: 2 (8 KiB per workgroup at 16-byte vectors), fewer when a
+  // full run does not fill that, as measured for the tile kernel's large launches.
+  int unroll = g_tune.runs_unroll;
+  if (unroll != 1 && unroll != 2 && unroll != 4) unroll = 2;
+  while (unroll > 1 && (int64_t)kThreads * (unroll / 2) >= vecs_per_run) unroll /= 2;
+  const int64_t per_wg = (int64_t)kThreads * unroll;
+  a.chunks_per_run = (uint32_t)((vecs_per_run + per_wg - 1) / per_wg);
+  const int64_t grid = max_runs * (int64_t)a.num_planes * a.chunks_per_run;
+  if (grid > 0x7fffffffll || max_runs > 0x7fffffffll)
+    return fail(KVC_ERR_UNSUPPORTED, "%s: %lld workgroups exceed 2^31", fn, (long long)grid);
+  const bool nt = g_tune.runs_nt != 0;
+  hipStream_t s = (hipStream_t)stream;
+  switch (vec) {
+    case 16: launch_runs_unroll<16>(a, unroll, (unsigned)grid, s, nt); break;
+    case 8: launch_runs_unroll<8>(a, unroll, (unsigned)grid, s, nt); break;
+    case 4: launch_runs_unroll<4>(a, unroll, (unsigned)grid, s, nt); break;
+    case 2: launch_runs_unroll<2>(a, unroll, (unsigned)grid, s, nt); break;
+    default: launch_runs_unroll<1>(a, unroll, (unsigned)grid, s, nt); break;
+  }
+  KVC_HIP(hipGetLastError());
+  g_last = LastLaunch{KVC_KERNEL_WRITE_RUNS, vec, unroll, kThreads, grid, nt ? 3 : 0, 0};
   return KVC_OK;
 }
 
@@ -1669,6 +1958,12 @@ int kvc_write_plan_resolve_slots(kvc_write_plan* plan, int64_t* slots, void* str
   return rc;
 }
 
+int kvc_write_plan_set_slots(kvc_write_plan* plan, const int64_t* slots) {
+  if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_write_plan_set_slots: null plan");
+  plan->slots = slots;
+  return KVC_OK;
+}
+
 int kvc_write_plan_destroy(kvc_write_plan* plan) {
   delete plan;
   return KVC_OK;
@@ -1709,9 +2004,10 @@ int kvc_build_write_index(const int32_t* input_lens, const int32_t* context_lens
                           int64_t num_kv_indices, int64_t page_size, int64_t nnz,
                           int32_t* cu_seqlens_q, int32_t* kv_indptr, int32_t* kv_last_page_len,
                           int32_t* batch_indices, int32_t* positions, int64_t* slot_mapping,
+                          int32_t* run_indptr, int32_t* runs, int32_t* num_runs, int64_t max_runs,
                           void* stream) {
   if (batch_size < 0 || nnz < 0 || num_kv_indices < 0 || page_size <= 0 ||
-      batch_size > 0x7fffffffll || page_size > 0x7fffffffll)
+      batch_size > 0x7fffffffll || page_size > 0x7fffffffll || nnz > 0x7fffffffll)
     return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: batch_size=%lld nnz=%lld page_size=%lld",
                 (long long)batch_size, (long long)nnz, (long long)page_size);
   if (!cu_seqlens_q || !kv_indptr)
@@ -1722,12 +2018,63 @@ int kvc_build_write_index(const int32_t* input_lens, const int32_t* context_lens
     return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: null per-token output");
   if (slot_mapping && num_kv_indices > 0 && !kv_indices)
     return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: null kv_indices");
+  if (runs) {
+    if (!run_indptr || !num_runs)
+      return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: runs need run_indptr and num_runs");
+    if ((uintptr_t)runs % 16)
+      return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: the run list must be 16-byte aligned");
+    // nnz tokens over batch_size requests form at most nnz / page_size + 2 * batch_size runs
+    const int64_t bound = nnz / page_size + 2 * batch_size;
+    if (max_runs < std::min(bound, nnz))
+      return fail(KVC_ERR_INVALID_ARG, "kvc_build_write_index: max_runs=%lld cannot hold the %lld runs "
+                  "%lld tokens of %lld requests may form", (long long)max_runs,
+                  (long long)std::min(bound, nnz), (long long)nnz, (long long)batch_size);
+  } else {
+    run_indptr = nullptr;
+    num_runs = nullptr;
+    max_runs = 0;
+  }
   hipLaunchKernelGGL(build_write_index_kernel, dim3(1), dim3(kPrepThreads), 0, (hipStream_t)stream,
                      input_lens, context_lens, num_blocks, kv_indices, (int32_t)batch_size,
                      num_kv_indices, (int32_t)page_size, nnz, cu_seqlens_q, kv_indptr,
-                     kv_last_page_len, batch_indices, positions, slot_mapping);
+                     kv_last_page_len, batch_indices, positions, slot_mapping, run_indptr, runs,
+                     num_runs, max_runs);
   KVC_HIP(hipGetLastError());
   return KVC_OK;
+}
+
+int kvc_slot_runs(const void* slot_mapping, int slot_bytes, int64_t num_tokens, int64_t block_size,
+                  int32_t* runs, int32_t* num_runs, int64_t max_runs, void* stream) {
+  if (num_tokens < 0 || block_size <= 0 || max_runs < 0 || num_tokens > 0x7fffffffll)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_slot_runs: num_tokens=%lld block_size=%lld max_runs=%lld",
+                (long long)num_tokens, (long long)block_size, (long long)max_runs);
+  if (slot_bytes != 4 && slot_bytes != 8)
+    return fail(KVC_ERR_UNSUPPORTED, "kvc_slot_runs: slot_bytes=%d (need 4 or 8)", slot_bytes);
+  if (!num_runs || (max_runs > 0 && !runs) || (num_tokens > 0 && !slot_mapping))
+    return fail(KVC_ERR_INVALID_ARG, "kvc_slot_runs: null pointer");
+  if ((uintptr_t)runs % 16)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_slot_runs: the run list must be 16-byte aligned");
+  if (max_runs < num_tokens)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_slot_runs: max_runs=%lld cannot hold the %lld runs that many "
+                "tokens may form", (long long)max_runs, (long long)num_tokens);
+  hipLaunchKernelGGL(slot_runs_kernel, dim3(1), dim3(kPrepThreads), 0, (hipStream_t)stream,
+                     slot_mapping, slot_bytes, num_tokens, block_size, runs, num_runs, max_runs);
+  KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+int kvc_write_runs_layers(const void* key, const void* value, void* key_cache, void* value_cache,
+                          const int32_t* runs, const int32_t* num_runs, int64_t max_runs,
+                          int64_t num_tokens, int64_t row_elems, int64_t key_token_stride,
+                          int64_t value_token_stride, int64_t block_size, int64_t cache_block_stride,
+                          int64_t cache_slot_stride, int64_t num_cache_blocks, int64_t num_layers,
+                          int64_t key_layer_stride, int64_t value_layer_stride,
+                          int64_t cache_layer_stride, int elem_bytes, void* stream) {
+  WriteGeom g{num_tokens, row_elems, key_token_stride, value_token_stride, block_size,
+              cache_block_stride, cache_slot_stride, num_cache_blocks, num_layers,
+              key_layer_stride, value_layer_stride, cache_layer_stride, elem_bytes};
+  return run_write_runs("kvc_write_runs_layers", key, value, key_cache, value_cache, runs, num_runs,
+                        max_runs, g, stream);
 }
 
 int kvc_copy_blocks(void* kv_caches, const int64_t* block_maps, int64_t num_pairs,
@@ -1855,6 +2202,17 @@ int kvc_swap_in(void* pool, const void* host_pool, const int64_t* src_ids, const
   return run_swap("kvc_swap_in", false, (char*)pool, (char*)host_pool, dst_ids, src_ids, g, staging,
                   staging_bytes, mode, false, kernel_stream, copy_stream);
 }
+
+int kvc_swap_resolve_mode(const int64_t* host_ids, int64_t n, int64_t num_layers_in_range,
+                          int64_t block_bytes, int64_t staging_bytes) {
+  if (n < 0 || num_layers_in_range < 0 || block_bytes < 0 || staging_bytes < 0)
+    return fail(KVC_ERR_INVALID_ARG, "kvc_swap_resolve_mode: negative size");
+  const SwapGeom g{n, num_layers_in_range, 0, block_bytes, 0, 0, 0, num_layers_in_range};
+  static const char some_staging = 0;   // only its presence is looked at
+  return resolve_auto_mode(host_ids, g, staging_bytes > 0 ? &some_staging : nullptr, staging_bytes);
+}
+
+int kvc_swap_last_mode(void) { return g_last_swap_mode; }
 
 int kvc_order_pairs_by_host_id(int64_t* gpu_ids, int64_t* host_ids, int64_t n) {
   if (n < 0) return fail(KVC_ERR_INVALID_ARG, "kvc_order_pairs_by_host_id: negative size");

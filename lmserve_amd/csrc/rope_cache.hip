@@ -628,6 +628,12 @@ int kvc_rotary_plan_resolve_slots(kvc_rotary_plan* plan, int64_t* slots, void* s
   return rc;
 }
 
+int kvc_rotary_plan_set_slots(kvc_rotary_plan* plan, const int64_t* slots) {
+  if (!plan) return fail(KVC_ERR_INVALID_ARG, "kvc_rotary_plan_set_slots: null plan");
+  plan->slots = slots;
+  return KVC_OK;
+}
+
 int kvc_rotary_plan_destroy(kvc_rotary_plan* plan) {
   delete plan;
   return KVC_OK;

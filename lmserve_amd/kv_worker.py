@@ -139,21 +139,6 @@ class PinnedHostPool:
             self.ptr = None
 
 
-def memmap_disk_kv_cache(kv_cache_file: str, shape: Tuple[int, ...], dtype, mode: str = "r+"):
-    """Open the disk tier's `.npy` memory map, recreating it when the stored
-    shape or dtype no longer match (kv_worker.py:48-85)."""
-    if os.path.exists(kv_cache_file):
-        try:
-            kv_cache = np.load(kv_cache_file, mmap_mode=mode)
-            if kv_cache.shape == tuple(shape) and kv_cache.dtype == np.dtype(dtype):
-                return kv_cache
-            del kv_cache
-        except Exception:
-            pass
-        os.remove(kv_cache_file)
-    return np.lib.format.open_memmap(kv_cache_file, mode="w+", dtype=dtype, shape=tuple(shape))
-
-
 @dataclass
 class PreparedSwap:
     """Id lists of one copy, already checked and resident on the device

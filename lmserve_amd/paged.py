@@ -213,7 +213,10 @@ class PagedKVWritePlan:
     small launch on the current stream, `kvc_write_plan_resolve_slots`), and every
     layer's launch addresses the cache through the resulting slot per token: its
     chain of three dependent index loads is gone. Same results; the appends must
-    run on that stream or be ordered after it.
+    run on that stream or be ordered after it. `slots=` hands over slots that
+    already exist on the device (the slot mapping of `build_write_index`)
+    instead: no launch, and a plan over fixed-capacity index buffers stays valid
+    for every later step written into them.
 
     The plan keeps references to the index tensors, so their memory stays valid
     for as long as the plan lives.
@@ -221,7 +224,7 @@ class PagedKVWritePlan:
 
     def __init__(self, batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len,
                  num_kv_heads: int, head_dim: int, page_size: int, dtype: torch.dtype,
-                 kv_layout: str = "NHD", resolve_slots: bool = False):
+                 kv_layout: str = "NHD", resolve_slots: bool = False, slots: torch.Tensor = None):
         (self.batch_indices, self.positions, self.kv_indices, self.kv_indptr,
          self.kv_last_page_len) = _paged_common(None, None, batch_indices, positions, kv_indices,
                                                 kv_indptr, kv_last_page_len, kv_layout)
@@ -240,7 +243,14 @@ class PagedKVWritePlan:
             self.elem, ctypes.byref(handle)))
         self._plan = handle.value
         self.slots = None
-        if resolve_slots and self.nnz:
+        if slots is not None:
+            # slots the caller already has (the index build's slot_mapping): nothing to launch
+            _require_gpu(slots, "slots")
+            if slots.dtype != torch.int64 or not slots.is_contiguous() or slots.numel() != self.nnz:
+                raise TypeError("slots must be contiguous int64 [nnz]")
+            self.slots = slots
+            _lib.check(lib.kvc_write_plan_set_slots(self._plan, slots.data_ptr()))
+        elif resolve_slots and self.nnz:
             self.slots = torch.empty(self.nnz, dtype=torch.int64, device=self.device)
             with _on_device_of(self.batch_indices):
                 _lib.check(lib.kvc_write_plan_resolve_slots(self._plan, self.slots.data_ptr(),
@@ -327,9 +337,32 @@ class PagedKVWritePlan:
             _lib.check(rc)
 
 
+class BlockRuns:
+    """Block-run descriptors of a step on the device: `runs` int32 `[max_runs, 4]`
+    (first token, block id, first entry, token count), `num_runs` int32 `[1]`,
+    and, when they come from the index build, `run_indptr` int32 `[B + 1]`."""
+
+    def __init__(self, runs: torch.Tensor, num_runs: torch.Tensor, run_indptr=None):
+        self.runs, self.num_runs, self.run_indptr = runs, num_runs, run_indptr
+
+    @property
+    def max_runs(self) -> int:
+        return int(self.runs.shape[0])
+
+    def tolist(self):
+        """The step's descriptors as a list of 4-tuples (synchronises)."""
+        n = int(self.num_runs.item())
+        return [tuple(r) for r in self.runs[:n].cpu().tolist()]
+
+
+def max_block_runs(nnz: int, batch_size: int, page_size: int) -> int:
+    """Upper bound of the block runs `nnz` new tokens of `batch_size` requests form."""
+    return max(1, min(int(nnz), int(nnz) // int(page_size) + 2 * int(batch_size)))
+
+
 def build_write_index(input_lens: torch.Tensor, context_lens: torch.Tensor,
                       num_blocks: torch.Tensor, kv_indices: torch.Tensor, page_size: int,
-                      nnz: int, with_slot_mapping: bool = True):
+                      nnz: int, with_slot_mapping: bool = True, with_runs: bool = False, out=None):
     """All index tensors of a step from the per-request scalars, in one launch.
 
     input_lens, context_lens, num_blocks: int32 `[B]` on the device (new tokens,
@@ -337,7 +370,13 @@ def build_write_index(input_lens: torch.Tensor, context_lens: torch.Tensor,
     kv_indices: int32 concatenation of the block tables. Returns
     `(cu_seqlens_q, kv_indptr, kv_last_page_len, batch_indices, positions, slot_mapping)`
     -- what `ModelWorker._make_inputs` builds on the host and uploads piecewise
-    (model_worker.py:346, :362-365, :399-433), plus the slot mapping.
+    (model_worker.py:346, :362-365, :399-433), plus the slot mapping; with
+    `with_runs=True` a seventh element, the step's `BlockRuns`.
+
+    `B`, `nnz` and `kv_indices.numel()` are capacities: requests with
+    `input_lens[b] == 0` pad the batch and per-token outputs beyond the step's
+    token count are -1 (skipped by every write). `out` takes the outputs of an
+    earlier call to be written again (fixed addresses, for a recorded launch).
     """
     input_lens = _i32(input_lens, "input_lens")
     context_lens = _i32(context_lens, "context_lens")
@@ -348,16 +387,84 @@ def build_write_index(input_lens: torch.Tensor, context_lens: torch.Tensor,
         raise ValueError("input_lens, context_lens and num_blocks must have one entry per request")
     dev = input_lens.device
     nnz = int(nnz)
-    cu = torch.empty(B + 1, dtype=torch.int32, device=dev)
-    indptr = torch.empty(B + 1, dtype=torch.int32, device=dev)
-    last = torch.empty(B, dtype=torch.int32, device=dev)
-    batch_indices = torch.empty(nnz, dtype=torch.int32, device=dev)
-    positions = torch.empty(nnz, dtype=torch.int32, device=dev)
-    slots = torch.empty(nnz, dtype=torch.int64, device=dev) if with_slot_mapping else None
+    if out is not None:
+        cu, indptr, last, batch_indices, positions, slots = out[:6]
+        runs = out[6] if len(out) > 6 else None
+        if cu.numel() != B + 1 or indptr.numel() != B + 1 or last.numel() != B \
+                or batch_indices.numel() != nnz or positions.numel() != nnz \
+                or (slots is not None and slots.numel() != nnz):
+            raise ValueError("`out` does not match the sizes of this call")
+    else:
+        cu = torch.empty(B + 1, dtype=torch.int32, device=dev)
+        indptr = torch.empty(B + 1, dtype=torch.int32, device=dev)
+        last = torch.empty(B, dtype=torch.int32, device=dev)
+        batch_indices = torch.empty(nnz, dtype=torch.int32, device=dev)
+        positions = torch.empty(nnz, dtype=torch.int32, device=dev)
+        slots = torch.empty(nnz, dtype=torch.int64, device=dev) if with_slot_mapping else None
+        runs = None
+        if with_runs:
+            cap = max_block_runs(nnz, B, page_size)
+            runs = BlockRuns(torch.empty(cap, 4, dtype=torch.int32, device=dev),
+                             torch.zeros(1, dtype=torch.int32, device=dev),
+                             torch.empty(B + 1, dtype=torch.int32, device=dev))
     with _on_device_of(input_lens):
         _lib.check(_lib.lib().kvc_build_write_index(
             input_lens.data_ptr(), context_lens.data_ptr(), num_blocks.data_ptr(),
             kv_indices.data_ptr(), B, kv_indices.numel(), int(page_size), nnz, cu.data_ptr(),
             indptr.data_ptr(), last.data_ptr(), batch_indices.data_ptr(), positions.data_ptr(),
-            slots.data_ptr() if slots is not None else None, _stream_of(input_lens)))
+            slots.data_ptr() if slots is not None else None,
+            runs.run_indptr.data_ptr() if runs is not None else None,
+            runs.runs.data_ptr() if runs is not None else None,
+            runs.num_runs.data_ptr() if runs is not None else None,
+            runs.max_runs if runs is not None else 0, _stream_of(input_lens)))
+    if runs is not None:
+        return cu, indptr, last, batch_indices, positions, slots, runs
     return cu, indptr, last, batch_indices, positions, slots
+
+
+def slot_block_runs(slot_mapping: torch.Tensor, block_size: int) -> BlockRuns:
+    """Block runs of any slot mapping on the device (one small launch): token t
+    opens a run when its slot is valid and is not the successor of token t-1's
+    slot inside the same block."""
+    _require_gpu(slot_mapping, "slot_mapping")
+    if slot_mapping.dtype not in (torch.int32, torch.int64) or slot_mapping.dim() != 1:
+        raise TypeError("slot_mapping must be a 1-D int32 or int64 tensor")
+    slot_mapping = slot_mapping.contiguous()
+    T = slot_mapping.numel()
+    dev = slot_mapping.device
+    runs = BlockRuns(torch.empty(max(T, 1), 4, dtype=torch.int32, device=dev),
+                     torch.zeros(1, dtype=torch.int32, device=dev))
+    with _on_device_of(slot_mapping):
+        _lib.check(_lib.lib().kvc_slot_runs(slot_mapping.data_ptr(), slot_mapping.element_size(), T,
+                                            int(block_size), runs.runs.data_ptr(), runs.num_runs.data_ptr(),
+                                            runs.max_runs, _stream_of(slot_mapping)))
+    return runs
+
+
+def write_block_runs_layers(key: torch.Tensor, value: torch.Tensor, kv_caches: torch.Tensor,
+                            runs: BlockRuns) -> None:
+    """`reshape_and_cache_layers` on the slot mapping `runs` describes, as tile
+    copies: every (run, layer, K|V) moves as one contiguous piece.
+
+    key, value: `[L, T, H, D]` contiguous; kv_caches `[L, nb, 2, bs, H, D]` contiguous.
+    """
+    for t, n in ((key, "key"), (value, "value"), (kv_caches, "kv_caches")):
+        _require_gpu(t, n)
+    if kv_caches.dim() != 6 or kv_caches.shape[2] != 2 or not kv_caches.is_contiguous():
+        raise ValueError("kv_caches must be contiguous [L, num_blocks, 2, block_size, H, D]")
+    if key.dtype != kv_caches.dtype or value.dtype != kv_caches.dtype:
+        raise TypeError("key/value and kv_caches must share one dtype")
+    L, nb, _, bs, H, D = kv_caches.shape
+    row = H * D
+    if key.dim() != 4 or key.shape != value.shape or key.shape[0] != L or key.shape[2] * key.shape[3] != row:
+        raise ValueError("key/value must be [L, T, H, D] matching the pool")
+    key, value = key.contiguous(), value.contiguous()
+    T = key.shape[1]
+    if T == 0 or row == 0 or nb == 0 or L == 0:
+        return
+    with _on_device_of(kv_caches):
+        _lib.check(_lib.lib().kvc_write_runs_layers(
+            key.data_ptr(), value.data_ptr(), kv_caches.data_ptr(),
+            kv_caches.data_ptr() + bs * row * kv_caches.element_size(), runs.runs.data_ptr(),
+            runs.num_runs.data_ptr(), runs.max_runs, T, row, row, row, bs, 2 * bs * row, row, nb, L,
+            T * row, T * row, nb * 2 * bs * row, kv_caches.element_size(), _stream_of(kv_caches)))

@@ -240,13 +240,16 @@ class PagedRotaryWritePlan:
     `resolve_slots=True` walks the page table once, at construction (one small
     launch on the current stream); the per-layer launches then read one slot per
     token. Same results; the runs must be ordered after the construction.
+    `slots=` hands over slots that already exist on the device (the slot mapping
+    of `build_write_index`) instead: no launch, and a plan over fixed-capacity
+    index buffers stays valid for every later step written into them.
 
     The plan keeps references to its tensors for as long as it lives.
     """
 
     def __init__(self, batch_indices, positions, kv_indices, kv_indptr, kv_last_page_len,
                  cos_sin_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                 page_size: int, resolve_slots: bool = False):
+                 page_size: int, resolve_slots: bool = False, slots: torch.Tensor = None):
         for t, n in ((batch_indices, "batch_indices"), (positions, "positions"),
                      (kv_indices, "kv_indices"), (kv_indptr, "kv_indptr"),
                      (kv_last_page_len, "kv_last_page_len")):
@@ -275,7 +278,14 @@ class PagedRotaryWritePlan:
             self.page_size, self.kd, ctypes.byref(handle)))
         self._plan = handle.value
         self.slots = None
-        if resolve_slots and self.nnz:
+        if slots is not None:
+            # slots the caller already has (the index build's slot_mapping): nothing to launch
+            _require_gpu(slots, "slots")
+            if slots.dtype != torch.int64 or not slots.is_contiguous() or slots.numel() != self.nnz:
+                raise TypeError("slots must be contiguous int64 [nnz]")
+            self.slots = slots
+            _lib.check(lib.kvc_rotary_plan_set_slots(self._plan, slots.data_ptr()))
+        elif resolve_slots and self.nnz:
             # the page table is walked once, here; every layer's launch reads one slot per token
             self.slots = torch.empty(self.nnz, dtype=torch.int64, device=self.device)
             with torch.cuda.device(self.device):

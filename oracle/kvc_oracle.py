@@ -16,7 +16,11 @@ All operate IN PLACE on NumPy arrays of any item size (bf16 is carried as
 uint16, as the reference's host pool does: kv_worker.py:17-22). Citations are
 paths under the reference's runtime/worker/llm_worker/. Pinning status is listed
 in the header of kvc_oracle.c; parity of the three page-table functions with
-the third-party flashinfer binary itself is UNPINNED. The two functions that
+the third-party flashinfer binary itself is UNPINNED. The block-run functions
+(`block_runs_loops`, `slot_runs_loops`, `runs_to_slots`, `write_runs_np`) are
+pinned in tests/test_oracle_pinning.py: a step written out by hand, the runs
+expanded back to slots against the independently pinned slot mapping, maximality
+of the runs, and the slice write against the pinned slot-mapped write. The two functions that
 exist only here, `build_write_index_*` and `paged_write_slots_np`, are pinned in
 tests/test_host_logic.py: a step written out by hand, NumPy against loops, the
 pinned page-table functions, and (for the slots) the property that a slot-mapped
@@ -138,6 +142,86 @@ def build_write_index_loops(input_lens, context_lens, num_blocks, kv_indices, pa
     i32 = np.int32
     return (np.asarray(cu, dtype=i32), np.asarray(indptr, dtype=i32), np.asarray(last, dtype=i32),
             np.asarray(batch, dtype=i32), np.asarray(pos, dtype=i32), np.asarray(slots, dtype=np.int64))
+
+
+def pad_write_index(index, nnz):
+    """`build_write_index_*` output with its per-token arrays padded to the
+    capacity `nnz` the way a capacity-bound launch leaves them: -1 in
+    batch_indices, positions and slot_mapping beyond the step's tokens (entries a
+    write skips: models/layers/attention.py:76-85 is never given them)."""
+    cu, indptr, last, batch, pos, slots = index
+    t = len(batch)
+    assert t <= nnz
+
+    def pad(a):
+        out = np.full(nnz, -1, dtype=a.dtype)
+        out[:t] = a
+        return out
+    return cu, indptr, last, pad(batch), pad(pos), pad(slots)
+
+
+def block_runs_loops(input_lens, context_lens, num_blocks, kv_indices, page_size):
+    """Block runs of a step, request by request: the new tokens of request b sit
+    at positions [ctx - q, ctx) (scheduler.rs:453-541) and each block they touch
+    takes one run -- consecutive tokens on the source side, consecutive entries
+    of one block on the cache side (scheduler.rs:466-512: a chunk fills whole
+    blocks). Returns (run_indptr int32 [B+1], runs int32 [n, 4]) with
+    runs[r] = (first token, block id or -1 outside the table, first entry, count)."""
+    run_indptr, runs = [0], []
+    token, table_at = 0, 0
+    for q, ctx, nblk in zip(input_lens, context_lens, num_blocks):
+        q, ctx, nblk = int(q), int(ctx), int(nblk)
+        table = [int(x) for x in kv_indices[table_at:table_at + nblk]]
+        table_at += nblk
+        pos = ctx - q
+        if q > 0 and pos >= 0:
+            while pos < ctx:
+                page, entry = pos // page_size, pos % page_size
+                count = min(page_size - entry, ctx - pos)
+                runs.append((token + pos - (ctx - q), table[page] if page < len(table) else -1, entry, count))
+                pos += count
+        token += q
+        run_indptr.append(len(runs))
+    return np.asarray(run_indptr, dtype=np.int32), np.asarray(runs, dtype=np.int32).reshape(-1, 4)
+
+
+def slot_runs_loops(slot_mapping, block_size):
+    """Block runs of any slot mapping, token by token: a token with a valid slot
+    continues the current run when its slot follows the previous token's inside
+    the same block, and opens a new one otherwise. int32 [n, 4]."""
+    runs = []
+    prev = None
+    for t, s in enumerate(int(x) for x in slot_mapping):
+        if s < 0:
+            prev = None
+            continue
+        if prev is not None and s == prev + 1 and s % block_size != 0:
+            runs[-1][3] += 1
+        else:
+            runs.append([t, s // block_size, s % block_size, 1])
+        prev = s
+    return np.asarray(runs, dtype=np.int32).reshape(-1, 4)
+
+
+def runs_to_slots(runs, num_tokens, block_size):
+    """Slot of every token the runs cover (-1 for tokens they do not cover, and
+    for runs outside the table)."""
+    slots = np.full(num_tokens, -1, dtype=np.int64)
+    for t0, blk, e, c in np.asarray(runs, dtype=np.int64).reshape(-1, 4):
+        if blk >= 0:
+            slots[t0:t0 + c] = blk * block_size + e + np.arange(c)
+    return slots
+
+
+def write_runs_np(key, value, kv_caches, runs) -> None:
+    """The write the run descriptors stand for, as slice copies: for every layer,
+    `kv_caches[l, blk, 0, e:e+c] = key[l, t0:t0+c]`, likewise value into plane 1.
+    key/value [L, T, H, D], kv_caches [L, nb, 2, bs, H, D]."""
+    nb = kv_caches.shape[1]
+    for t0, blk, e, c in np.asarray(runs, dtype=np.int64).reshape(-1, 4):
+        if 0 <= blk < nb and c > 0:
+            kv_caches[:, blk, 0, e:e + c] = key[:, t0:t0 + c]
+            kv_caches[:, blk, 1, e:e + c] = value[:, t0:t0 + c]
 
 
 def paged_write_slots_np(batch_indices, positions, kv_indices, kv_indptr, page_size) -> np.ndarray:

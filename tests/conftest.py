@@ -28,12 +28,19 @@ def gpu():
 
 
 @pytest.fixture(autouse=True)
-def default_tuning():
+def default_tuning(request):
     """Every test starts and ends with the library's launch-shape knobs at their
-    defaults, whatever an earlier test set."""
+    defaults, whatever an earlier test set. Tests that never load the library
+    (oracle pinning, host logic) run without it."""
     from lmserve_amd import _lib
 
-    L = _lib.lib()
+    try:
+        L = _lib.lib()
+    except _lib.KVCacheLibraryError:
+        if request.node.get_closest_marker("gpu") is not None:
+            raise
+        yield
+        return
     assert L.kvc_tuning_modified() == 0, "a tuning knob was left modified by an earlier test"
     yield
     _lib.reset_tuning()

@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "kvcache.h"
+#include "kvcache_experimental.h"
 
 extern "C" {
 void oracle_reshape_and_cache(const void*, const void*, void*, const int64_t*, int64_t, int64_t,
@@ -433,7 +434,7 @@ int main() {
     KVC_OK_OR_DIE(kvc_build_write_index((const int32_t*)d_il, (const int32_t*)d_cl, (const int32_t*)d_nb,
                                         (const int32_t*)d_ind, 2, 5, bs, T, (int32_t*)d_cu, (int32_t*)d_ptr2,
                                         (int32_t*)d_last2, (int32_t*)d_bi2, (int32_t*)d_pos2,
-                                        (int64_t*)d_slots2, stream));
+                                        (int64_t*)d_slots2, nullptr, nullptr, nullptr, 0, stream));
     HIP_OK(hipStreamSynchronize(stream));
     std::vector<int32_t> g_ptr(3), g_last(2), g_bi(T), g_pos(T), g_cu(3);
     std::vector<int64_t> g_slots(T);

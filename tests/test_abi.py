@@ -1,4 +1,4 @@
-"""The C-ABI library loads and exports every symbol include/kvcache.h declares.
+"""The C-ABI library loads and exports every symbol include/*.h declares.
 
 No kernel is launched here: only symbol lookup and entry points that return
 before their first HIP call (argument validation, pure host arithmetic).
@@ -14,16 +14,20 @@ from lmserve_amd import _lib
 
 REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(REPO, "include", "kvcache.h")
+EXPERIMENTAL_HEADER = os.path.join(REPO, "include", "kvcache_experimental.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+def header_text(*paths):
+    return "\n".join(re.sub(r"/\*.*?\*/", "", open(p).read(), flags=re.S) for p in paths)
+
+
+def declared_functions(*paths):
+    text = header_text(*(paths or (HEADER, EXPERIMENTAL_HEADER)))
     return sorted(set(re.findall(r"\b(kvc_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_declares_the_expected_surface():
-    names = declared_functions()
+    names = declared_functions(HEADER)     # the stable header alone
     for must in ("kvc_reshape_and_cache", "kvc_reshape_and_cache_layers",
                  "kvc_append_paged_kv_cache", "kvc_append_paged_kv_cache_layers",
                  "kvc_get_seq_lens", "kvc_get_batch_indices_positions", "kvc_copy_blocks",
@@ -31,6 +35,10 @@ def test_header_declares_the_expected_surface():
                  "kvc_host_alloc_pinned", "kvc_host_free_pinned", "kvc_last_error_string",
                  "kvc_abi_version"):
         assert must in names
+    # knobs, launch introspection and the host-side row mover are not part of the stable surface
+    for name in names:
+        assert not name.startswith(("kvc_set_tuning", "kvc_get_tuning", "kvc_last_launch_info", "kvc_row_mover")), name
+    assert "kvc_row_mover_cancel" in declared_functions(EXPERIMENTAL_HEADER)
 
 
 def test_library_exports_every_declared_symbol():
@@ -45,7 +53,7 @@ def test_python_binding_types_every_declared_symbol():
 
 
 def test_binding_arity_matches_the_header():
-    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    text = header_text(HEADER, EXPERIMENTAL_HEADER)
     for name, (_, argtypes) in _lib.SIGNATURES.items():
         m = re.search(r"\b" + name + r"\s*\(([^;]*?)\)\s*;", text, flags=re.S)
         if m is None:
@@ -149,9 +157,14 @@ def test_rope_and_index_build_validate_their_arguments():
     assert call(ko=None) == _lib.KVC_ERR_INVALID_ARG        # no cache and no key_out: nowhere to put K
     assert call(qs=100) == _lib.KVC_ERR_INVALID_ARG         # stride smaller than the row
     g = L.kvc_build_write_index
-    assert g(None, None, None, None, -1, 0, 16, 0, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
-    assert g(None, None, None, None, 2, 0, 16, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG
-    assert g(1, 1, 1, 1, 2, 4, 0, 4, 1, 1, 1, 1, 1, 1, None) == _lib.KVC_ERR_INVALID_ARG   # page_size 0
+    no_runs = (None, None, None, 0, None)
+    assert g(None, None, None, None, -1, 0, 16, 0, 1, 1, 1, 1, 1, 1, *no_runs) == _lib.KVC_ERR_INVALID_ARG
+    assert g(None, None, None, None, 2, 0, 16, 4, 1, 1, 1, 1, 1, 1, *no_runs) == _lib.KVC_ERR_INVALID_ARG
+    assert g(1, 1, 1, 1, 2, 4, 0, 4, 1, 1, 1, 1, 1, 1, *no_runs) == _lib.KVC_ERR_INVALID_ARG   # page_size 0
+    # a run list needs its prefix sums and its count, 16-byte alignment and room for every run
+    assert g(1, 1, 1, 1, 2, 4, 16, 64, 1, 1, 1, 1, 1, 1, None, 16, 1, 64, None) == _lib.KVC_ERR_INVALID_ARG
+    assert g(1, 1, 1, 1, 2, 4, 16, 64, 1, 1, 1, 1, 1, 1, 1, 24, 1, 64, None) == _lib.KVC_ERR_INVALID_ARG
+    assert g(1, 1, 1, 1, 2, 4, 16, 64, 1, 1, 1, 1, 1, 1, 1, 16, 1, 7, None) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_set_tuning(b"no_such_knob", 1) == _lib.KVC_ERR_INVALID_ARG
 
 
@@ -161,7 +174,8 @@ def test_tuning_knobs_read_back_and_reset():
     defaults = {"copy_unroll": 0, "gather_unroll": 0, "copy_nt": 1, "copy_max_wgs": 0, "copy_order": 0,
                 "write_vpt": 0, "write_nt": 1, "write_order": 0, "write_threads": 0, "write_planes": 1,
                 "write_planes_vpt": 0, "write_planes_min_bytes": 256 << 10, "write_planes_max_vpr": 256, "write_planes_threads": 0,
-                "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 1 << 20, "rope_threads": 0, "disk_bounce_mib": 4}
+                "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 1 << 20, "rope_threads": 0, "disk_bounce_mib": 4,
+                "runs_unroll": 0, "runs_order": 0, "runs_nt": 1}
     for key, value in defaults.items():
         assert _lib.get_tuning(key) == value, key
     for i, key in enumerate(defaults):

@@ -5,7 +5,7 @@ import torch
 
 import lmserve_amd as kvc
 from lmserve_amd import _lib
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 from tests.helpers import bits_of, random_pool, to_bf16
 

@@ -10,7 +10,7 @@ import torch
 
 import lmserve_amd as kvc
 from lmserve_amd import _lib
-from lmserve_amd import workloads as wl
+import workloads as wl
 
 pytestmark = pytest.mark.gpu
 

@@ -65,7 +65,7 @@ def test_one_launch_index_build_matches_the_host_construction(gpu, kind):
     """Prefix sums, last-page lengths, request indices, positions and slots from
     one device launch equal what the host-side construction (the restatement of
     the reference's list building) produces."""
-    from lmserve_amd import workloads as wl
+    import workloads as wl
     rng = np.random.default_rng(11)
     bs = 16
     if kind == "decode":

@@ -13,7 +13,7 @@ import torch
 
 import lmserve_amd as kvc
 from lmserve_amd import rotary
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 from oracle import rope_oracle as ro
 

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import lmserve_amd as kvc
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 from tests.helpers import bits_of, random_pool, sentinel_pool, to_bf16
 

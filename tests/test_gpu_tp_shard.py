@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import lmserve_amd as kvc
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 
 pytestmark = pytest.mark.gpu

@@ -20,7 +20,7 @@ import pytest
 import torch
 
 import lmserve_amd as kvc
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 from tests.helpers import bf16_bits, bits_of, random_pool, to_bf16
 

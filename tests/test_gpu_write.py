@@ -8,7 +8,7 @@ import torch
 
 import lmserve_amd as kvc
 from lmserve_amd import _lib
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 from tests.helpers import bf16_bits, bits_of, sentinel_pool, to_bf16
 

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import lmserve_amd as kvc
-from lmserve_amd import workloads as wl
+import workloads as wl
 from lmserve_amd.index_prep import InferInput, make_kv_index_inputs
 from oracle import kvc_oracle as orc
 from tests.helpers import FifoBlockIds

@@ -315,3 +315,86 @@ def test_all_formulations_agree_on_a_mid_size_case():
     orc.copy_blocks_np(p1, maps)
     orc.c_copy_blocks(p2, maps)
     assert np.array_equal(p1, p2)
+
+
+# ------------------------------------------------------------------ block runs
+def test_block_runs_of_a_step_written_out_by_hand():
+    """Two requests, page size 4. Request 0: 6 new tokens at positions 3..8 of
+    table [7, 2, 9] -> blocks 7 (entry 3, 1 token), 2 (entries 0..3), 9 (entry 0, 1
+    token). Request 1: 2 new tokens at positions 1..2 of table [5] -> one run."""
+    indptr, runs = orc.block_runs_loops([6, 2], [9, 3], [3, 1], [7, 2, 9, 5], 4)
+    assert indptr.tolist() == [0, 3, 4]
+    assert runs.tolist() == [[0, 7, 3, 1], [1, 2, 0, 4], [5, 9, 0, 1], [6, 5, 1, 2]]
+    # a request whose table is too short: the run exists, its block is -1
+    _, runs = orc.block_runs_loops([5], [8], [1], [6], 4)
+    assert runs.tolist() == [[0, 6, 3, 1], [1, -1, 0, 4]]
+    # padding requests (no new tokens) add nothing
+    indptr, runs = orc.block_runs_loops([0, 1, 0], [0, 5, 0], [0, 2, 0], [3, 4], 4)
+    assert indptr.tolist() == [0, 0, 1, 1] and runs.tolist() == [[0, 4, 0, 1]]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_block_runs_expand_to_the_pinned_slot_mapping_and_are_maximal(seed):
+    """Independent of the run construction: expanded token by token, the runs give
+    exactly the slot mapping that `build_write_index_np` derives (pinned against a
+    hand case and against the page-table write), they cover the tokens in order
+    without gaps, and no two neighbouring runs could be one."""
+    rng = np.random.default_rng(seed)
+    bs = int(rng.choice([1, 2, 4, 16]))
+    B = int(rng.integers(1, 9))
+    q = rng.integers(0, 40, size=B)
+    filled = rng.integers(0, 50, size=B)
+    ctx = np.where(q > 0, filled + q, rng.integers(0, 3, size=B))
+    nblk = (ctx + bs - 1) // bs
+    table = rng.permutation(int(nblk.sum()) + 5)[:int(nblk.sum())]
+    index = orc.build_write_index_np(q, ctx, nblk, table, bs)
+    slots = index[5]
+    indptr, runs = orc.block_runs_loops(q, ctx, nblk, table, bs)
+    T = int(q.sum())
+    assert np.array_equal(orc.runs_to_slots(runs, T, bs), slots)
+    assert int(runs[:, 3].sum()) == T and np.all(runs[:, 3] >= 1)
+    assert np.array_equal(runs[:, 0], np.concatenate([[0], np.cumsum(runs[:, 3])[:-1]]))   # in order, no gaps
+    assert np.all(runs[:, 2] + runs[:, 3] <= bs)
+    cu = index[0]
+    for r in range(1, len(runs)):
+        same_request = np.searchsorted(cu, runs[r, 0], side="right") == np.searchsorted(cu, runs[r - 1, 0], side="right")
+        if same_request:       # inside a request a new run starts at the head of a block
+            assert runs[r, 2] == 0 and runs[r - 1, 2] + runs[r - 1, 3] == bs
+    assert indptr[-1] == len(runs)
+    # the runs of an arbitrary slot mapping: the same descriptors, found token by token
+    assert np.array_equal(orc.slot_runs_loops(slots, bs), runs)
+
+
+def test_slot_runs_split_at_gaps_blocks_and_invalid_slots():
+    runs = orc.slot_runs_loops([4, 5, 6, 7, 8, 20, 19, -1, 30, 31, 33], 4)
+    assert runs.tolist() == [[0, 1, 0, 4], [4, 2, 0, 1], [5, 5, 0, 1], [6, 4, 3, 1], [8, 7, 2, 2], [10, 8, 1, 1]]
+    assert orc.slot_runs_loops([], 4).shape == (0, 4)
+    assert orc.runs_to_slots(runs, 11, 4).tolist() == [4, 5, 6, 7, 8, 20, 19, -1, 30, 31, 33]
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_run_write_equals_the_pinned_slot_mapped_write(seed):
+    rng = np.random.default_rng(seed)
+    L, nb, bs, H, D = 3, 12, 4, 2, 4
+    q = rng.integers(1, 12, size=3)
+    ctx = q + rng.integers(0, 6, size=3)
+    nblk = (ctx + bs - 1) // bs
+    table = rng.permutation(nb)[:int(nblk.sum())]
+    slots = orc.build_write_index_np(q, ctx, nblk, table, bs)[5]
+    _, runs = orc.block_runs_loops(q, ctx, nblk, table, bs)
+    T = int(q.sum())
+    key = rng.integers(0, 1 << 16, size=(L, T, H, D), dtype=np.uint16)
+    value = rng.integers(0, 1 << 16, size=(L, T, H, D), dtype=np.uint16)
+    pool = rng.integers(0, 1 << 16, size=(L, nb, 2, bs, H, D), dtype=np.uint16)
+    want = pool.copy()
+    for l in range(L):
+        orc.reshape_and_cache_np(key[l], value[l], want[l], slots)
+    orc.write_runs_np(key, value, pool, runs)
+    assert np.array_equal(pool, want)
+
+
+def test_padded_index_marks_the_entries_beyond_the_step():
+    index = orc.build_write_index_np([2, 1], [5, 9], [2, 3], [1, 2, 3, 4, 5], 4)
+    cu, indptr, last, batch, pos, slots = orc.pad_write_index(index, 6)
+    assert batch.tolist() == [0, 0, 1, -1, -1, -1] and pos.tolist() == [3, 4, 8, -1, -1, -1]
+    assert slots.tolist()[3:] == [-1, -1, -1] and slots.tolist()[:3] == index[5].tolist()

@@ -9,7 +9,7 @@ import numpy as np
 import torch
 from hypothesis import given, settings, strategies as st
 
-from lmserve_amd import workloads as wl
+import workloads as wl
 from oracle import kvc_oracle as orc
 from oracle import torch_cpu
 

@@ -5,7 +5,7 @@ pair lists and swap id lists in the shapes the reference's scheduler produces
 (runtime/src/llm_engine/scheduler.rs:453-541,
  runtime/src/llm_engine/block_manager.rs:62-140: the free list starts as
  0..nb and turns into an arbitrary order under churn, so tables are drawn from
- a seeded permutation of the pool). Used by the tests and by bench.py.
+ a seeded permutation of the pool). Used by the tests and by bench.py; not part of the lmserve_amd package.
 """
 from __future__ import annotations
 
@@ -14,7 +14,7 @@ from typing import Dict, List, Tuple
 
 import numpy as np
 
-from .index_prep import InferInput, KVIndexInputs, make_kv_index_inputs
+from lmserve_amd.index_prep import InferInput, KVIndexInputs, make_kv_index_inputs
 
 
 @dataclass(frozen=True)
