@@ -16,8 +16,8 @@ The LAST line of stdout is one compact JSON object (under 4 KiB): the headline,
 `roofline` (algorithmic bytes of one launch over the launch's mean duration,
 against 8 TB/s), `cpu_baseline` (the torch-CPU statement of the same step on the
 host cores, bounded sample) and `configs`: one short object per benchmark
-configuration and form (us, GB/s, fraction of 8 TB/s, counter traffic over
-algorithmic bytes). Every other row (variants, passes, names in prose) goes to
+configuration and form (us, GB/s, fraction of 8 TB/s, and counter traffic over
+algorithmic bytes where it has been measured). Every other row (variants, passes, names in prose) goes to
 the details file (`--details`, default gpurun_out/bench_details.json) and to
 stderr, never to stdout.
 
@@ -180,7 +180,9 @@ def config_row(cfg_id, entry_point, form, e, wall=False, **extra):
     us = e["wall_us_per_call"] if wall else e["us_per_call"]
     gbps = e["bytes_per_call"] / (us * 1e-6) / 1e9 if us > 0 else 0.0
     row = {"id": cfg_id, "entry": entry_point, "form": form, "us": round(us, 2), "gbps": round(gbps),
-           "frac": round(gbps / HBM_PEAK_GBPS, 3), "traffic_ratio": TRAFFIC_RATIO.get((cfg_id, form))}
+           "frac": round(gbps / HBM_PEAK_GBPS, 3)}
+    if (cfg_id, form) in TRAFFIC_RATIO:      # measured with counters at the default sizes; absent = not measured
+        row["traffic_ratio"] = TRAFFIC_RATIO[(cfg_id, form)]
     row.update(extra)
     return row
 
@@ -197,6 +199,7 @@ def build_line(head, configs):
     key but `configs`; if the whole does not fit, configs are dropped from the end
     (the details file has them all) and `configs_dropped` says how many."""
     dropped = 0
+    configs = [dict(c, entry=c["entry"].replace("kvc_", "")) for c in configs]   # entry points of libkvcache, prefix dropped
     while True:
         line = dict(head)
         line["configs"] = configs[:len(configs) - dropped]
@@ -310,7 +313,7 @@ def bench_swap(torch, kvc, _lib, wl, np, dev, swap_blocks, settle_seconds, arena
             e = entry(f"cfg5 {form} stage, HBM only ({n} blocks x {L5} layers x 64 KiB)", 2 * nbytes, ms_w, ms_e,
                       launch="eager")
             detail.append(e)
-            compact.append(config_row("cfg5", f"kvc_{form}_blocks", form, e, blocks=n))
+            compact.append(config_row("cfg5", f"kvc_{form}_blocks", form, e))
         del dense
         if settle_seconds > 0:
             settle_copy_engines(torch, dev, "the swap rows", settle_seconds)
@@ -334,7 +337,7 @@ def bench_swap(torch, kvc, _lib, wl, np, dev, swap_blocks, settle_seconds, arena
                 t = timed_sync(lambda: worker.copy_kv_sync(maps, src, dst), 3)
                 detail.append({"name": f"cfg5 {direction} ({mode}; {size})", "ms_per_call": round(t * 1e3, 2),
                                "pcie_gbps": round(nbytes / t / 1e9, 2), "bytes_per_call": int(nbytes)})
-                compact.append({"id": "cfg5", "entry": f"kvc_{direction}", "form": mode, "blocks": n,
+                compact.append({"id": "cfg5", "entry": f"kvc_{direction}", "form": mode,
                                 "ms": round(t * 1e3, 1), "pcie_gbps": round(nbytes / t / 1e9, 1)})
             # one call per layer, as the layer-pipelined protocol issues them: ids checked and
             # uploaded once (kvc_swap_prepare), then one call per layer
@@ -374,7 +377,7 @@ def bench_swap(torch, kvc, _lib, wl, np, dev, swap_blocks, settle_seconds, arena
                        "ms_per_call": round(t * 1e3, 2), "pcie_gbps": round(nbytes / t / 1e9, 2),
                        "pcie_gbps_note": "sum of both directions", "bytes_per_call": int(nbytes)})
         compact.append({"id": "cfg5", "entry": "kvc_swap_out+kvc_swap_in", "form": "staged, both at once",
-                        "blocks": n, "ms": round(t * 1e3, 1), "pcie_gbps": round(nbytes / t / 1e9, 1)})
+                        "ms": round(t * 1e3, 1), "pcie_gbps": round(nbytes / t / 1e9, 1)})
         # host blocks that do not neighbour each other (every second block of the host pool:
         # what an allocator hands out after churn), one layer per call
         ns = min(512, n // 2)
@@ -400,7 +403,7 @@ def bench_swap(torch, kvc, _lib, wl, np, dev, swap_blocks, settle_seconds, arena
                            "bytes_per_call": int(sbytes)})
     finally:
         worker.close()
-    return compact, detail
+    return compact, detail, n
 
 
 def main(argv=None):
@@ -428,6 +431,7 @@ def main(argv=None):
     torch.cuda.set_device(dev)
     ops = set() if args.ops == "none" else set(args.ops.split(","))
     details, configs = [], []
+    swap_blocks_run = None
     default_sizes = args.pool_blocks == 65536
 
     # ------------------------------------------------ config 2: decode-step write (headline)
@@ -484,29 +488,17 @@ def main(argv=None):
         del srcs, dsts
 
     if "write" in ops:
+        # (the page-table one-launch form, the full-argument eager call and the plan under a
+        # graph are in the details file)
         for form, prefix, launch, entry_point, wall in (
-                ("1 launch, page table", "cfg2 decode/append_paged_kv_cache_layers", "eager",
-                 "kvc_append_paged_kv_cache_layers", False),
                 ("per layer, graph", "cfg2 decode/append_paged_kv_cache (per layer", "hipGraph",
                  "kvc_append_paged_kv_cache", False),
-                ("per layer, eager wall", "cfg2 decode/append_paged_kv_cache (per layer", "eager",
-                 "kvc_append_paged_kv_cache", True),
                 ("per layer, plan, eager wall", "cfg2 decode/PagedKVWritePlan(resolve_slots).append", "eager",
-                 "kvc_write_plan_append", True),
-                ("per layer, plan, graph", "cfg2 decode/PagedKVWritePlan(resolve_slots).append", "hipGraph",
-                 "kvc_write_plan_append", False)):
+                 "kvc_write_plan_append", True)):
             e = find(entries, prefix, launch)
             if e is not None:
                 configs.append(config_row("cfg2", entry_point, form, e, wall=wall))
     log(f"[{time.perf_counter() - t_begin:.1f} s] config 2 done")
-
-    # ------------------------------------------------ a whole decode step from one hipGraph
-    if "step" in ops:
-        with optional_section("decode step graph", torch):
-            from bench_sections import bench_decode_step_graph
-            c, d = bench_decode_step_graph(torch, kvc, wl, s8, pool, L, args.pool_blocks, dev)
-            configs += c
-            details += d
 
     if "rope" in ops:
         with optional_section("rotation rows", torch):
@@ -551,10 +543,28 @@ def main(argv=None):
                                        max(ROTATE_PREFILL, args.steps // 2), max(3, args.warmup // 2),
                                        ["fused_slot:graph", "fused_paged:graph", "per_layer_paged:graph"])
             details += e3
+            with optional_section("config 3 run write", torch):
+                # the same launch as tile copies over the block runs the index build emits
+                runs3 = []
+                for w3, _, _, _ in sets3:
+                    order = sorted(range(len(w3.inputs)), key=lambda i: -w3.inputs[i].input_len)
+                    rs = [w3.inputs[i] for i in order]
+                    up = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)   # noqa: E731
+                    runs3.append(kvc.build_write_index(
+                        up([r.input_len for r in rs]), up([r.context_len for r in rs]),
+                        up([len(r.block_ids) for r in rs]), up([b for r in rs for b in r.block_ids]),
+                        sq.block_size, w3.num_tokens, with_runs=True)[6])
+                R3 = len(sets3)
+                ms_w, ms_e = time_region(
+                    lambda i: kvc.write_block_runs_layers(sets3[i % R3][1], sets3[i % R3][2], pool3, runs3[i % R3]),
+                    max(ROTATE_PREFILL, args.steps // 2), max(3, args.warmup // 2), torch, graph_of=R3)
+                e = entry(f"cfg3 chunked prefill/write_block_runs_layers (1 launch, {L3} layers, tile copies over "
+                          f"{runs3[0].max_runs} run descriptors)", sets3[0][0].algorithmic_bytes(L3), ms_w, ms_e,
+                          launch="hipGraph replay")
+                details.append(e)
+                configs.append(config_row("cfg3", "kvc_write_runs_layers", "1 launch, block runs", e))
             for form, prefix, entry_point in (
                     ("1 launch", "cfg3 chunked prefill/reshape_and_cache_layers", "kvc_reshape_and_cache_layers"),
-                    ("1 launch, page table", "cfg3 chunked prefill/append_paged_kv_cache_layers",
-                     "kvc_append_paged_kv_cache_layers"),
                     ("per layer, graph", "cfg3 chunked prefill/append_paged_kv_cache (per layer",
                      "kvc_append_paged_kv_cache")):
                 e = find(e3, prefix, "hipGraph")
@@ -572,11 +582,27 @@ def main(argv=None):
     # buffer from the same arena: nothing large has been freed before its copies run)
     if "swap" in ops:
         with optional_section("config 5 swap rows", torch):
-            c5, d5 = bench_swap(torch, kvc, _lib, wl, np, dev, args.swap_blocks, args.settle_seconds, arena)
+            c5, d5, swap_blocks_run = bench_swap(torch, kvc, _lib, wl, np, dev, args.swap_blocks,
+                                                 args.settle_seconds, arena)
             configs += c5
             details += d5
         arena.reset()
         log(f"[{time.perf_counter() - t_begin:.1f} s] config 5 done")
+
+    # ------------------------------------------------ a whole decode step from one hipGraph
+    # (after the swap rows: whether swap-out and swap-in issued together overlap on the link
+    # depends on the streams the KV worker is handed, which depends on how many streams the
+    # process has made before; this order keeps that row comparable from run to run)
+    if "step" in ops:
+        with optional_section("decode step graph", torch):
+            from bench_sections import bench_decode_step_graph
+            pool, L = arena.pool(s8, args.pool_blocks)
+            c, d = bench_decode_step_graph(torch, kvc, wl, s8, pool, L, args.pool_blocks, dev)
+            configs += c
+            details += d
+            del pool
+        arena.reset()
+        log(f"[{time.perf_counter() - t_begin:.1f} s] decode step graph done")
 
     del arena
     torch.cuda.empty_cache()
@@ -636,7 +662,8 @@ def main(argv=None):
                    "entry": "kvc_reshape_and_cache_layers",
                    "launch": "one eager launch per step",
                    "rotation": ROTATE_DECODE,
-                   "hw_queues": os.environ.get("GPU_MAX_HW_QUEUES", "runtime default")},
+                   "hw_queues": os.environ.get("GPU_MAX_HW_QUEUES", "runtime default"),
+                   "cfg5_blocks": swap_blocks_run},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_CFG2_ONE_LAUNCH if (L == 32 and default_sizes) else None,

@@ -705,6 +705,37 @@ def bench_slot_patterns(torch, kvc, wl, dev, steps):
         out.append(entry(f"cfg3 launch, slot pattern: {label}", nbytes, ms, ms, launch="eager",
                          launches_per_round=reps + 2, rounds=rounds,
                          us_per_round=[round(x * 1e3, 2) for x in per_pattern[label]]))
+    # the workload's block runs once more, moved as tile copies over run descriptors
+    # (write_runs_kernel dispatches, after all write_rows_kernel ones)
+    run_sets = []
+    for r in range(Rq):
+        wq = wl.chunked_prefill(sq, num_blocks=nbq, seed=r)
+        order = sorted(range(len(wq.inputs)), key=lambda i: -wq.inputs[i].input_len)
+        rs = [wq.inputs[i] for i in order]
+        up = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)   # noqa: E731
+        run_sets.append(kvc.build_write_index(up([x.input_len for x in rs]), up([x.context_len for x in rs]),
+                                              up([len(x.block_ids) for x in rs]),
+                                              up([b for x in rs for b in x.block_ids]), sq.block_size, Tq,
+                                              with_runs=True)[6])
+    torch.cuda.synchronize()
+    times = []
+    for rnd in range(rounds):
+        for i in range(2):
+            kvc.write_block_runs_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, run_sets[i % Rq])
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(reps):
+            kvc.write_block_runs_layers(srcs[i % Rq][0], srcs[i % Rq][1], poolq, run_sets[i % Rq])
+        end.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(end) / reps)
+        log(f"translation: round {rnd}: {reps + 2} write_runs_kernel dispatches, the workload's block runs, "
+            f"{times[-1] * 1e3:.2f} us each")
+    ms = sorted(times)[rounds // 2]
+    out.append(entry("cfg3 launch, the workload's block runs as tile copies over run descriptors (write_runs_kernel)",
+                     nbytes, ms, ms, launch="eager", launches_per_round=reps + 2, rounds=rounds,
+                     us_per_round=[round(x * 1e3, 2) for x in times]))
     del poolq, srcs
     torch.cuda.empty_cache()
     return out
@@ -756,3 +787,97 @@ def bench_tp_shard(torch, kvc, wl, dev, steps, warmup, swap_blocks, settle_secon
     del pool_s, sets_s
     torch.cuda.empty_cache()
     return out
+
+
+def bench_decode_step_graph(torch, kvc, wl, s8, pool, L, num_blocks, dev, steps=200):
+    """A whole decode step of configuration 2 (index build + one K/V write per
+    layer) replayed from ONE hipGraph for consecutive, different steps, beside
+    the eager ways of doing the same step. Times are per 32-layer step.
+    Returns (rows of the final line, detail rows)."""
+    import numpy as np
+
+    from lmserve_amd.step_graph import KVWriteStep
+
+    R, B = 4, 256
+    H, D, bs = s8.num_kv_heads, s8.head_dim, s8.block_size
+    works = [wl.decode_step(s8, num_blocks=num_blocks, batch=B, seed=100 + r) for r in range(R)]
+    packed = []
+    for w in works:
+        order = sorted(range(len(w.inputs)), key=lambda i: -w.inputs[i].input_len)
+        rs = [w.inputs[i] for i in order]
+        packed.append((np.asarray([r.input_len for r in rs], dtype=np.int32),
+                       np.asarray([r.context_len for r in rs], dtype=np.int32),
+                       np.asarray([len(r.block_ids) for r in rs], dtype=np.int32),
+                       np.asarray([b for r in rs for b in r.block_ids], dtype=np.int32)))
+    cap_ids = max(p[3].shape[0] for p in packed)
+    step = KVWriteStep(H, D, bs, torch.bfloat16, dev, max_requests=B, max_tokens=B, max_block_ids=cap_ids)
+    key = torch.randn(L, B, H, D, device=dev).to(torch.bfloat16)
+    value = torch.randn_like(key)
+    keys, values, caches = [key[l] for l in range(L)], [value[l] for l in range(L)], [pool[l] for l in range(L)]
+    step.set_arrays(*packed[0])
+    graph = step.capture(keys, values, caches)
+    bytes_step = works[0].algorithmic_bytes(L)
+
+    def timed(fn, n):
+        for i in range(8):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6, e0.elapsed_time(e1) / n * 1e3
+
+    def replay_only(i):
+        graph.replay()
+
+    def new_step_then_replay(i):
+        step.set_arrays(*packed[i % R])       # host packing + one upload: a NEW step every time
+        graph.replay()
+
+    def eager_one_launch_index_and_plan(i):
+        w = works[i % R]
+        idx = kvc.to_device_one_launch(w.inputs, bs, dev)
+        plan = kvc.PagedKVWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices, idx.kv_block_indptrs,
+                                    idx.kv_last_block_lens, H, D, bs, torch.bfloat16, slots=idx.slot_mapping)
+        for l in range(L):
+            plan.append(keys[l], values[l], caches[l])
+
+    def eager_reference_construction(i):
+        w = works[i % R]
+        idx = kvc.to_device(kvc.make_kv_index_inputs(w.inputs, bs), bs, dev, with_slot_mapping=False)
+        for l in range(L):
+            kvc.append_paged_kv_cache(keys[l], values[l], idx.batch_indices, idx.positions, caches[l],
+                                      idx.kv_block_indices, idx.kv_block_indptrs, idx.kv_last_block_lens)
+
+    def eager_writes_only(i):
+        for l in range(L):
+            step.append(keys[l], values[l], caches[l])
+
+    compact, detail = [], []
+    # `us` of these rows is WALL time per 32-layer step (what the serving loop pays)
+    for fn, n, form, short, what in (
+            (replay_only, steps, "step wall, graph", "graph{index+32 writes}",
+             "one hipGraph replay = index build + 32 per-layer writes (the step's scalars already uploaded)"),
+            (new_step_then_replay, steps, "step wall, new step: pack+upload+graph", "set_arrays+graph",
+             "a NEW step each time: host packs 3 x 256 scalars + the block tables, one upload, one replay"),
+            (eager_writes_only, steps, "step wall, 32 eager plan calls", None,
+             "the 32 per-layer writes alone, eager, through the same plan (no index work)"),
+            (eager_one_launch_index_and_plan, max(20, steps // 8), "step wall, eager index+plan", None,
+             "eager: host packing from request objects, 2 uploads, one-launch index, 32 plan calls"),
+            (eager_reference_construction, max(10, steps // 16), "step wall, eager reference way",
+             "host lists+32 append calls",
+             "eager: the reference's host list building and six uploads, then 32 full-argument calls")):
+        wall_us, dev_us = timed(fn, n)
+        detail.append({"name": f"cfg2 decode step ({L} layers, {B} requests): {what}", "wall_us_per_step": round(wall_us, 1),
+                       "device_us_per_step": round(dev_us, 1), "bytes_per_step": int(bytes_step),
+                       "note": "K/V sources of all steps are one 64 MiB set (per-layer launches of 2 MiB are bound by "
+                               "launch latency, not by where their lines come from)"})
+        if short is not None:
+            compact.append({"id": "cfg2", "entry": short, "form": form, "us": round(wall_us, 1),
+                            "gbps": round(bytes_step / wall_us / 1e3),
+                            "frac": round(bytes_step / wall_us / 1e3 / HBM_PEAK_GBPS, 3)})
+    return compact, detail

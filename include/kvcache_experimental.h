@@ -83,8 +83,9 @@ int64_t kvc_last_launch_info(int what);
  * kvc_slot_runs derives the descriptors from any slot mapping on the device
  * (one small launch): token t opens a run when slot[t] >= 0 and slot[t] is not
  * slot[t-1] + 1 inside the same block; max_runs >= num_tokens (checked).
- * Tuning keys: "runs_unroll" (vectors per lane: 1, 2, 4; 0 = default 2),
- * "runs_order" (1 = all runs of a plane are neighbours in the grid), "runs_nt".
+ * Tuning keys: "runs_unroll" (vectors per lane: 1, 2, 4; 0 = by launch size),
+ * "runs_order" (1 = all runs of a plane are neighbours in the grid, the default;
+ * 0 = all planes of a run), "runs_nt".
  * ------------------------------------------------------------------------- */
 int kvc_slot_runs(const void* slot_mapping, int slot_bytes, int64_t num_tokens,
                   int64_t block_size, int32_t* runs, int32_t* num_runs, int64_t max_runs,

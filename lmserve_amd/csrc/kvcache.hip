@@ -90,7 +90,7 @@ struct Tuning {
                             // both directions at once want 96 or more each (91-92 against 87 GB/s
                             // in sum); the rest of the GPU stays free for the model
   int runs_unroll = 0;       // write_runs: 16-byte vectors per lane (1, 2, 4), 0 = by size
-  int runs_order = 0;        // write_runs: 1 = all runs of a plane are neighbours in the grid
+  int runs_order = 1;        // write_runs: 1 = all runs of a plane are neighbours in the grid, 0 = all planes of a run
   int runs_nt = 1;           // write_runs: non-temporal loads and stores
   int auto_min_extent_bytes = 1 << 20;  // KVC_SWAP_AUTO: mean bytes per PCIe copy from which a call
                                         // goes through the copy engines. A copy costs about 10 us
@@ -129,7 +129,7 @@ Knob* knobs(int* count) {
       {"direct_max_wgs", &g_tune.direct_max_wgs, 96},
       {"auto_min_extent_bytes", &g_tune.auto_min_extent_bytes, 1 << 20},
       {"runs_unroll", &g_tune.runs_unroll, 0},
-      {"runs_order", &g_tune.runs_order, 0},
+      {"runs_order", &g_tune.runs_order, 1},
       {"runs_nt", &g_tune.runs_nt, 1},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
@@ -1176,7 +1176,7 @@ int run_write_runs(const char* fn, const void* key, const void* value, void* kc,
   a.num_planes = (uint32_t)(2 * g.num_layers);
   a.vecs_per_row = (uint32_t)(g.row_elems * E / vec);
   a.vpr_shift = log2_exact(a.vecs_per_row);
-  a.plane_major = g_tune.runs_order;
+  a.plane_major = g_tune.runs_order != 0;
   a.key_token_stride = g.key_token_stride * E;
   a.value_token_stride = g.value_token_stride * E;
   a.key_layer_stride = g.key_layer_stride * E;
@@ -1190,10 +1190,15 @@ int run_write_runs(const char* fn, const void* key, const void* value, void* kc,
   const int64_t vecs_per_run = g.block_size * (int64_t)a.vecs_per_row;  // of a full run
   if (vecs_per_run > 0x7fffffffll)
     return fail(KVC_ERR_UNSUPPORTED, "%s: %lld vectors per run exceed 2^31", fn, (long long)vecs_per_run);
-  // Vectors per lane: 2 (8 KiB per workgroup at 16-byte vectors), fewer when a
-  // full run does not fill that, as measured for the tile kernel's large launches.
+  // One vector per lane (4 KiB per workgroup at 16-byte vectors) and all runs of a
+  // plane next to each other in the grid measured best at the 2048-token chunk of
+  // 28 layers (43.1 us; 2 and 4 vectors per lane 45.5-46.9, run-major order 43.3,
+  // an XCD-aware order 44.2-45.2; the token kernel 44.1-44.4). One layer per
+  // launch prefers 2 (4.05 against 4.49 us), where the grid is a quarter of a
+  // resident set.
   int unroll = g_tune.runs_unroll;
-  if (unroll != 1 && unroll != 2 && unroll != 4) unroll = 2;
+  if (unroll != 1 && unroll != 2 && unroll != 4)
+    unroll = max_runs * (int64_t)a.num_planes * ((vecs_per_run + kThreads - 1) / kThreads) <= resident_workgroups() ? 2 : 1;
   while (unroll > 1 && (int64_t)kThreads * (unroll / 2) >= vecs_per_run) unroll /= 2;
   const int64_t per_wg = (int64_t)kThreads * unroll;
   a.chunks_per_run = (uint32_t)((vecs_per_run + per_wg - 1) / per_wg);

@@ -75,6 +75,7 @@ class KVWorkerHandle:
     model_queue: Any = field(default_factory=queue.Queue)
     kv_queue: Any = field(default_factory=queue.Queue)
     sync: str = "events"
+    host_wait_timeout: Optional[float] = 30.0    # seconds a notifier thread waits for one event; None = forever
     _notifier: Any = field(default=None, repr=False, compare=False)
 
     @classmethod
@@ -99,9 +100,11 @@ class KVWorkerHandle:
 
     def ring_when_done(self, event, doorbell) -> None:
         """sync="host": put a token on `doorbell` once `event` has completed, in
-        the order of the calls (one notifier thread per handle and process)."""
+        the order of the calls (one notifier thread per handle and process).
+        Raises `TimeoutError` once an earlier event was given up after
+        `host_wait_timeout` seconds."""
         if self._notifier is None:
-            self._notifier = _Notifier()
+            self._notifier = _Notifier(self.host_wait_timeout)
         self._notifier.submit(event, doorbell)
 
     def close(self) -> None:
@@ -112,16 +115,34 @@ class KVWorkerHandle:
 
 class _Notifier:
     """A thread that waits for events in submission order and rings a doorbell
-    after each (host-signalled layer protocol)."""
+    after each (host-signalled layer protocol). No wait is unbounded: an event
+    that has not completed after `timeout` seconds is given up (its doorbell is
+    NOT rung, so the other side's own timeout fires rather than a false "done"),
+    the jobs queued behind it are dropped the same way, and `failed` says so.
+    `stop()` abandons whatever is still waiting."""
 
-    def __init__(self):
+    def __init__(self, timeout: Optional[float] = 30.0, poll: float = 2e-5):
         import threading
         self.jobs: "queue.Queue" = queue.Queue()
+        self.timeout, self.poll = timeout, poll
+        self.failed: Optional[str] = None
+        self._stopping = threading.Event()
         self.thread = threading.Thread(target=self._run, name="kvc-layer-doorbell", daemon=True)
         self.thread.start()
 
     def submit(self, event, doorbell) -> None:
+        if self.failed is not None:
+            raise TimeoutError(self.failed)
         self.jobs.put((event, doorbell))
+
+    def _wait(self, event) -> bool:
+        import time
+        deadline = None if self.timeout is None else time.monotonic() + self.timeout
+        while not event.query():
+            if self._stopping.is_set() or (deadline is not None and time.monotonic() > deadline):
+                return False
+            time.sleep(self.poll)
+        return True
 
     def _run(self) -> None:
         while True:
@@ -129,10 +150,15 @@ class _Notifier:
             if job is None:
                 return
             event, doorbell = job
-            event.synchronize()
-            doorbell.put(b"")
+            if self.failed is not None or self._stopping.is_set():
+                continue                      # drained, not rung
+            if self._wait(event):
+                doorbell.put(b"")
+            elif not self._stopping.is_set():
+                self.failed = f"an event of the layer protocol was not reached within {self.timeout} s"
 
     def stop(self) -> None:
+        self._stopping.set()
         self.jobs.put(None)
         self.thread.join(timeout=10)
 
@@ -196,6 +222,35 @@ class KVWorkerParams:
     sync: str = "events"   # "host": no event handles travel (see KVWorkerHandle)
 
 
+IPC_SEGMENT_LIMIT = 2 << 30
+
+
+def allocator_segment_bytes(tensor: torch.Tensor, snapshot=None) -> Optional[int]:
+    """Size of the caching-allocator segment that holds `tensor`'s storage, or None
+    when the snapshot does not list it. An IPC handle of a tensor covers its whole
+    segment, not just the tensor."""
+    address = tensor.untyped_storage().data_ptr()
+    for segment in (snapshot if snapshot is not None else torch.cuda.memory_snapshot()):
+        if segment["address"] <= address < segment["address"] + segment["total_size"]:
+            return int(segment["total_size"])
+    return None
+
+
+def check_ipc_segment(kv_caches: torch.Tensor, snapshot=None, limit: int = IPC_SEGMENT_LIMIT) -> None:
+    """Refuse to export a pool whose allocator segment is `limit` bytes or more:
+    opening such a handle in another process does not return on this platform.
+    Pools of that size are served by a `KVWorker` in the model's own process."""
+    size = allocator_segment_bytes(kv_caches, snapshot)
+    if size is None:
+        size = kv_caches.untyped_storage().nbytes()
+    if size >= limit:
+        raise ValueError(
+            f"the pool sits in an allocator segment of {size} bytes; a shared allocation must stay under "
+            f"{limit} bytes on this platform. Give the pool a segment of its own below that size "
+            "(torch.cuda.empty_cache() before allocating it), or run the KV worker in this process "
+            "(KVWorker(kv_caches, ...)) instead of exporting the pool")
+
+
 def make_kv_worker_params(kv_caches: torch.Tensor, handle: KVWorkerHandle, num_host_blocks: int,
                           num_disk_blocks: int = 0, disk_kv_cache_file: str = "") -> KVWorkerParams:
     """Export the pool and the handle's events for another process on the same GPU
@@ -207,6 +262,7 @@ def make_kv_worker_params(kv_caches: torch.Tensor, handle: KVWorkerHandle, num_h
     if kv_caches.storage_offset() != 0 or \
             kv_caches.untyped_storage().nbytes() != kv_caches.numel() * kv_caches.element_size():
         raise ValueError("kv_caches must own its storage (the other process maps the whole storage)")
+    check_ipc_segment(kv_caches)
     return KVWorkerParams(
         kv_cache_metadata=kv_caches.untyped_storage()._share_cuda_(),
         num_layers=kv_caches.shape[0], num_gpu_blocks=kv_caches.shape[1],

@@ -37,6 +37,8 @@ import asyncio
 import ctypes
 import enum
 import os
+import time
+import warnings
 import weakref
 from dataclasses import dataclass, field
 from typing import Iterable, List, Optional, Sequence, Tuple
@@ -117,6 +119,33 @@ def order_by_host_id(gpu_ids: np.ndarray, host_ids: np.ndarray) -> Tuple[np.ndar
     return gpu_ids, host_ids
 
 
+_warned_about_queues = False
+
+
+def warn_if_few_hardware_queues(environ=os.environ) -> bool:
+    """One warning per process when a KV worker is set up to copy beside a forward
+    pass while the HIP runtime runs with its default of 4 hardware queues: the
+    model's stream and the worker's stream can then share a queue and wait for
+    each other (a forward pass of 15.6 ms took 33-36 ms beside a write-through
+    on MI355X). `GPU_MAX_HW_QUEUES=8` in the environment, set before the process
+    first touches the GPU, gives every stream involved a queue of its own. The
+    reference runs the KV worker as a second process, which has its own queues.
+    Returns whether it warned."""
+    global _warned_about_queues
+    try:
+        queues = int(environ.get("GPU_MAX_HW_QUEUES", "4"))
+    except ValueError:
+        queues = 4
+    if queues >= 8 or _warned_about_queues:
+        return False
+    _warned_about_queues = True
+    warnings.warn("KVWorker with a layer-sync handle in a process with GPU_MAX_HW_QUEUES="
+                  f"{environ.get('GPU_MAX_HW_QUEUES', 'unset (4)')}: copies beside a forward pass may share a "
+                  "hardware queue with the model's stream and double its time; export GPU_MAX_HW_QUEUES=8 before "
+                  "the process starts, or run the KV worker as its own process", RuntimeWarning, stacklevel=3)
+    return True
+
+
 class PinnedHostPool:
     """`[num_host_blocks, L, block_elems]` page-locked, device-addressable host
     memory (replaces pycuda's `pagelocked_empty`, kv_worker.py:123-127)."""
@@ -166,10 +195,11 @@ class HostBounce:
         self.slot_bytes = 0
         self.mover = None     # kvc_row_mover: its thread moves the rows of the regions
 
-    def row_mover(self, threads: int):
+    def row_mover(self, threads: int, timeout: Optional[float] = None):
         if self.mover is None:
             mover = ctypes.c_void_p()
             _lib.check(_lib.lib().kvc_row_mover_create(int(threads), ctypes.byref(mover)))
+            _lib.check(_lib.lib().kvc_row_mover_set_timeout_ms(mover, -1 if timeout is None else int(timeout * 1e3)))
             self.mover = mover
         return self.mover
 
@@ -179,8 +209,10 @@ class HostBounce:
     def slot_ptr(self, layer_idx: int) -> int:
         return self.ptr + (layer_idx % self.slots) * self.slot_bytes
 
-    def close(self) -> None:
+    def close(self, cancel: bool = False) -> None:
         if self.mover is not None:
+            if cancel:   # jobs that still wait for an event give up now instead of at their deadline
+                _lib.check(_lib.lib().kvc_row_mover_cancel(self.mover))
             _lib.check(_lib.lib().kvc_row_mover_destroy(self.mover))   # after its queued jobs
             self.mover = None
         if self.ptr:
@@ -234,6 +266,10 @@ class KVWorker:
       while those are in their good state, and unaffected by the state they
       fall into for some seconds after the process has freed device memory
       (48 against 38 GB/s there).
+    host_wait_timeout: seconds after which a host-side wait of the layer protocol
+      gives up (`TimeoutError`): the doorbell of the model's next layer, the event
+      a queued row copy waits for. `close()` returns within it whatever the other
+      side does. None = no limit (the reference's behaviour).
     validate: check on the host that no block is the destination of two pairs of
       one GPU<->Host call (`ValueError`). The reference copies the pairs one
       after the other, so the later pair wins there (kv_worker.py:197-227);
@@ -258,6 +294,7 @@ class KVWorker:
         host_copy_threads: int = 4,
         host_bounce_regions: int = 4,
         host_bounce_always: bool = False,
+        host_wait_timeout: Optional[float] = 30.0,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -286,8 +323,10 @@ class KVWorker:
         self.host_copy_threads = int(host_copy_threads)
         self.host_bounce_regions = max(2, int(host_bounce_regions))
         self.host_bounce_always = bool(host_bounce_always)
+        self.host_wait_timeout = None if host_wait_timeout is None else float(host_wait_timeout)
         self._bounce = {"out": None, "in": None}
         self.last_copy_went_through_host_bounce = False
+        self.last_copy_swap_mode = -1    # KVC_SWAP_* the last layer-by-layer copy's calls ran in
 
         self._host_pool = PinnedHostPool((self.num_host_blocks, num_layers, block_elems), np_dtype)
         self.host_kv_caches = self._host_pool.array
@@ -312,6 +351,8 @@ class KVWorker:
             self.htod_stream = torch.cuda.Stream()
         self._staging = {}   # (direction, stream handle) -> [workspace, weak reference to its PreparedSwap]
         self.kv_worker_handle = kv_worker_handle
+        if kv_worker_handle is not None:
+            warn_if_few_hardware_queues()
 
         self.COPY_KV_OP_MAP = {
             (Device.GPU, Device.Host): self._copy_kv_gpu_to_host,
@@ -497,7 +538,8 @@ class KVWorker:
         blocks (the mover's thread waits for `after` first); returns the ticket."""
         with torch.cuda.device(self.device):
             ticket = _lib.lib().kvc_row_mover_submit(
-                bounce.row_mover(self.host_copy_threads), after.cuda_event if after is not None else None,
+                bounce.row_mover(self.host_copy_threads, self.host_wait_timeout),
+                after.cuda_event if after is not None else None,
                 self._host_pool.ptr, self.num_host_blocks, self.num_layers * self.block_stride,
                 layer_idx * self.block_stride, bounce.slot_ptr(layer_idx), prepared.host_ids.ctypes.data,
                 prepared.n, self.block_stride, 1 if to_pool else 0)
@@ -513,6 +555,17 @@ class KVWorker:
         else:
             _lib.check(await asyncio.to_thread(lib.kvc_row_mover_wait, bounce.mover, ticket))
 
+    async def _doorbell(self, doorbell, layer_idx: int) -> None:
+        """Take one token from `doorbell` (kv_worker.py:279-281 of the reference polls
+        the queue the same way), giving up after `host_wait_timeout`."""
+        deadline = None if self.host_wait_timeout is None else time.monotonic() + self.host_wait_timeout
+        while doorbell.empty():
+            if deadline is not None and time.monotonic() > deadline:
+                raise TimeoutError(f"no doorbell for layer {layer_idx} within {self.host_wait_timeout} s: "
+                                   "the model side has stopped posting layers")
+            await asyncio.sleep(1e-5)
+        doorbell.get()
+
     async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
                                      stream: torch.cuda.Stream) -> None:
         """GPU->Host (kv_worker.py:272-295). With a handle: per layer, wait for the
@@ -526,18 +579,19 @@ class KVWorker:
             prepared = self.prepare_swap("out", block_mappings, stream)
             bounce = self._bounce_for(prepared)
             self.last_copy_went_through_host_bounce = bounce is not None
+            if bounce is not None:
+                self.last_copy_swap_mode = _lib.KVC_SWAP_STAGED     # one dense copy per layer
             tickets: List[int] = []                 # per layer: its rows' job in the mover
             landed: List[torch.cuda.Event] = []     # per layer: the layer sits in its bounce region
             try:
                 for layer_idx in range(self.num_layers):
-                    while handle.kv_queue.empty():
-                        await asyncio.sleep(1e-5)
-                    handle.kv_queue.get()
+                    await self._doorbell(handle.kv_queue, layer_idx)
                     if handle.sync == "events":
                         stream.wait_event(handle.post_events[layer_idx])
                     # sync == "host": the token was sent after the layer's write had completed
                     if bounce is None:
                         self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
+                        self.last_copy_swap_mode = _lib.last_swap_mode()
                     else:
                         if layer_idx >= bounce.slots:       # the region's earlier rows must have left it
                             await self._host_rows_done(bounce, tickets[layer_idx - bounce.slots])
@@ -567,6 +621,8 @@ class KVWorker:
             prepared = self.prepare_swap("in", block_mappings, stream)
             bounce = self._bounce_for(prepared)
             self.last_copy_went_through_host_bounce = bounce is not None
+            if bounce is not None:
+                self.last_copy_swap_mode = _lib.KVC_SWAP_STAGED
             tickets: List[int] = []                    # per layer: the job that fills its bounce region
             region_read: List[torch.cuda.Event] = []   # per layer: the GPU has taken the region's rows
             try:
@@ -578,6 +634,7 @@ class KVWorker:
                 for layer_idx in range(self.num_layers):
                     if bounce is None:
                         self.swap_prepared_layers(prepared, layer_idx, layer_idx + 1)
+                        self.last_copy_swap_mode = _lib.last_swap_mode()
                     else:
                         await self._host_rows_done(bounce, tickets[layer_idx])
                         self._swap_layer_through_bounce(prepared, layer_idx, bounce.slot_ptr(layer_idx))
@@ -670,7 +727,7 @@ class KVWorker:
             self.disk_tier = None
         for direction, bounce in self._bounce.items():   # first: its mover still writes into the pool
             if bounce is not None:
-                bounce.close()
+                bounce.close(cancel=True)     # a job still waiting for an event is given up, not waited for
                 self._bounce[direction] = None
         self._host_pool.close()
         self._staging = {}

@@ -175,7 +175,7 @@ def test_tuning_knobs_read_back_and_reset():
                 "write_vpt": 0, "write_nt": 1, "write_order": 0, "write_threads": 0, "write_planes": 1,
                 "write_planes_vpt": 0, "write_planes_min_bytes": 256 << 10, "write_planes_max_vpr": 256, "write_planes_threads": 0,
                 "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 1 << 20, "rope_threads": 0, "disk_bounce_mib": 4,
-                "runs_unroll": 0, "runs_order": 0, "runs_nt": 1}
+                "runs_unroll": 0, "runs_order": 1, "runs_nt": 1}
     for key, value in defaults.items():
         assert _lib.get_tuning(key) == value, key
     for i, key in enumerate(defaults):
@@ -428,3 +428,118 @@ def test_operators_fail_loudly_without_the_library(monkeypatch, tmp_path):
         kvc.reshape_and_cache(torch.zeros(1, 1, 4, dtype=torch.bfloat16),
                               torch.zeros(1, 1, 4, dtype=torch.bfloat16), pool[0],
                               torch.zeros(1, dtype=torch.int64))
+
+
+# ------------------------------------------------------------------ no host-side wait is unbounded
+def _mover_fixture(n=6, row=64, layers=2, nhb=8):
+    rng = np.random.default_rng(3)
+    pool = np.zeros((nhb, layers, row), dtype=np.uint8)
+    dense = rng.integers(0, 255, size=(n, row), dtype=np.uint8)
+    ids = rng.permutation(nhb)[:n].astype(np.int64)
+    return pool, dense, ids
+
+
+def test_row_mover_job_starts_when_its_host_flag_is_set():
+    import threading
+    import time
+    L = _lib.lib()
+    mover = ctypes.c_void_p()
+    assert L.kvc_row_mover_create(2, ctypes.byref(mover)) == 0
+    pool, dense, ids = _mover_fixture()
+    flag = np.zeros(1, dtype=np.int32)
+    try:
+        t = L.kvc_row_mover_submit_after_flag(mover, flag.ctypes.data, pool.ctypes.data, 8, 2 * 64, 64,
+                                              dense.ctypes.data, ids.ctypes.data, 6, 64, 1)
+        assert t == 0
+        time.sleep(0.05)
+        assert L.kvc_row_mover_done(mover, t) == 0 and not pool.any()       # still waiting, nothing moved
+        threading.Timer(0.05, lambda: flag.__setitem__(0, 1)).start()
+        assert L.kvc_row_mover_wait(mover, t) == 0
+        assert np.array_equal(pool[ids, 1], dense)
+    finally:
+        assert L.kvc_row_mover_destroy(mover) == 0
+
+
+def test_row_mover_gives_up_at_its_deadline_and_drains_what_was_queued_behind():
+    """A job whose flag is never set (the stand-in for an event that never
+    completes) fails with KVC_ERR_TIMEOUT after the mover's deadline, the jobs
+    already queued behind it complete at once without copying, a job submitted
+    afterwards runs normally, and destroy returns."""
+    import time
+    L = _lib.lib()
+    mover = ctypes.c_void_p()
+    assert L.kvc_row_mover_create(2, ctypes.byref(mover)) == 0
+    assert L.kvc_row_mover_set_timeout_ms(mover, 150) == 0
+    pool, dense, ids = _mover_fixture()
+    never = np.zeros(1, dtype=np.int32)
+    t0 = time.monotonic()
+    stuck = L.kvc_row_mover_submit_after_flag(mover, never.ctypes.data, pool.ctypes.data, 8, 2 * 64, 0,
+                                              dense.ctypes.data, ids.ctypes.data, 6, 64, 1)
+    behind = [L.kvc_row_mover_submit(mover, None, pool.ctypes.data, 8, 2 * 64, 64, dense.ctypes.data,
+                                     ids.ctypes.data, 6, 64, 1) for _ in range(3)]
+    assert stuck == 0 and behind == [1, 2, 3]
+    assert L.kvc_row_mover_wait(mover, behind[-1]) == _lib.KVC_ERR_TIMEOUT
+    waited = time.monotonic() - t0
+    assert 0.14 <= waited < 2.0, waited
+    assert "not reached" in _lib.last_error()
+    assert not pool.any()                                   # neither the stuck job nor the ones behind it copied
+    assert L.kvc_row_mover_done(mover, behind[-1]) == 1
+    # the error has been collected: the mover works again
+    later = L.kvc_row_mover_submit(mover, None, pool.ctypes.data, 8, 2 * 64, 64, dense.ctypes.data,
+                                   ids.ctypes.data, 6, 64, 1)
+    assert later == 4 and L.kvc_row_mover_wait(mover, later) == 0
+    assert np.array_equal(pool[ids, 1], dense)
+    assert L.kvc_row_mover_destroy(mover) == 0
+
+
+def test_row_mover_cancel_and_destroy_do_not_wait_for_a_stuck_job():
+    import time
+    L = _lib.lib()
+    mover = ctypes.c_void_p()
+    assert L.kvc_row_mover_create(1, ctypes.byref(mover)) == 0
+    assert L.kvc_row_mover_set_timeout_ms(mover, -1) == 0           # no deadline at all
+    pool, dense, ids = _mover_fixture()
+    never = np.zeros(1, dtype=np.int32)
+    stuck = L.kvc_row_mover_submit_after_flag(mover, never.ctypes.data, pool.ctypes.data, 8, 2 * 64, 0,
+                                              dense.ctypes.data, ids.ctypes.data, 6, 64, 1)
+    behind = L.kvc_row_mover_submit(mover, None, pool.ctypes.data, 8, 2 * 64, 0, dense.ctypes.data,
+                                    ids.ctypes.data, 6, 64, 1)
+    time.sleep(0.05)
+    assert L.kvc_row_mover_done(mover, stuck) == 0
+    t0 = time.monotonic()
+    assert L.kvc_row_mover_cancel(mover) == 0
+    assert L.kvc_row_mover_wait(mover, behind) == _lib.KVC_ERR_CANCELLED
+    assert not pool.any()
+    assert L.kvc_row_mover_destroy(mover) == 0
+    assert time.monotonic() - t0 < 1.0
+    # destroy alone, with a deadline: returns within one deadline of the call
+    mover = ctypes.c_void_p()
+    assert L.kvc_row_mover_create(1, ctypes.byref(mover)) == 0
+    assert L.kvc_row_mover_set_timeout_ms(mover, 100) == 0
+    for _ in range(4):
+        L.kvc_row_mover_submit_after_flag(mover, never.ctypes.data, pool.ctypes.data, 8, 2 * 64, 0,
+                                          dense.ctypes.data, ids.ctypes.data, 6, 64, 1)
+    t0 = time.monotonic()
+    assert L.kvc_row_mover_destroy(mover) == 0
+    assert time.monotonic() - t0 < 1.0                      # one deadline, not four
+    assert L.kvc_row_mover_cancel(None) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_row_mover_set_timeout_ms(None, 5) == _lib.KVC_ERR_INVALID_ARG
+
+
+def test_swap_mode_can_be_asked_before_the_call():
+    L = _lib.lib()
+    MiB = 1 << 20
+    consecutive = np.arange(64, dtype=np.int64)
+    scattered = np.arange(0, 128, 2, dtype=np.int64)
+    big = L.kvc_swap_staging_bytes(64, 1, 64 << 10, _lib.KVC_SWAP_STAGED, 0)
+    # one layer of 64 consecutive 64 KiB blocks is one 4 MiB extent: the copy engines
+    assert L.kvc_swap_resolve_mode(consecutive.ctypes.data, 64, 1, 64 << 10, big) == _lib.KVC_SWAP_STAGED
+    # every second host block: 64 KiB extents, the direct kernel
+    assert L.kvc_swap_resolve_mode(scattered.ctypes.data, 64, 1, 64 << 10, big) == _lib.KVC_SWAP_DIRECT
+    # all 80 layers of a scattered block travel as one 5 MiB extent
+    assert L.kvc_swap_resolve_mode(scattered.ctypes.data, 64, 80, 64 << 10, 64 * MiB) == _lib.KVC_SWAP_STAGED
+    # no ring in the staging buffer: only the direct kernel can run
+    assert L.kvc_swap_resolve_mode(consecutive.ctypes.data, 64, 1, 64 << 10, 1024) == _lib.KVC_SWAP_DIRECT
+    assert L.kvc_swap_resolve_mode(None, 64, 1, 64 << 10, big) == _lib.KVC_SWAP_DIRECT
+    assert L.kvc_swap_resolve_mode(consecutive.ctypes.data, -1, 1, 64 << 10, big) == _lib.KVC_ERR_INVALID_ARG
+    assert L.kvc_swap_last_mode() in (-1, _lib.KVC_SWAP_STAGED, _lib.KVC_SWAP_DIRECT)

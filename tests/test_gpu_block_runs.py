@@ -48,7 +48,8 @@ def test_prefill_chunk_block_runs_every_launch_shape(gpu, unroll, order):
     runs = _run_case(gpu, L, nb, s.block_size, s.num_kv_heads, s.head_dim, w.index.slot_mapping, 30)
     ran = _lib.last_launch()
     assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_RUNS and ran["vec_bytes"] == 16
-    assert ran["per_lane"] == (unroll or 2)
+    # by default one vector per lane: 512 descriptors x 10 planes x 4 chunks exceed a resident set
+    assert ran["per_lane"] == (unroll or 1)
     assert len(runs) >= 4 * (512 // 16 // 4)
 
 
@@ -105,6 +106,30 @@ def test_runs_outside_the_pool_or_the_tokens_are_skipped(gpu):
     kvc.write_block_runs_layers(to_bf16(key, gpu), to_bf16(value, gpu), dpool, druns)
     torch.cuda.synchronize()
     assert np.array_equal(bits_of(dpool), want)
+
+
+def test_launch_rule_of_the_run_write(gpu):
+    """Two vectors per lane while the grid fits one resident set of workgroups (one
+    layer of a chunk), one beyond it (all layers)."""
+    s = wl.QWEN_2_5_7B
+    nb, T = 2048, 2048
+    w = wl.chunked_prefill(s, num_blocks=nb, min_context=16, max_context=4000, seed=1)
+    order = sorted(range(len(w.inputs)), key=lambda i: -w.inputs[i].input_len)
+    rs = [w.inputs[i] for i in order]
+    up = lambda a: torch.tensor(a, dtype=torch.int32, device=gpu)
+    out = kvc.build_write_index(up([r.input_len for r in rs]), up([r.context_len for r in rs]),
+                                up([len(r.block_ids) for r in rs]), up([b for r in rs for b in r.block_ids]),
+                                s.block_size, T, with_runs=True)
+    runs = out[6]
+    assert runs.max_runs == T // s.block_size + 2 * len(rs)
+    for L, want in ((1, 2), (28, 1)):
+        pool = torch.zeros(L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16, device=gpu)
+        k = torch.zeros(L, T, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16, device=gpu)
+        kvc.write_block_runs_layers(k, k, pool, runs)
+        ran = _lib.last_launch()
+        assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_RUNS and ran["per_lane"] == want
+        assert ran["grid"] == runs.max_runs * 2 * L * (4 // want)
+    torch.cuda.synchronize()
 
 
 def test_index_build_emits_the_oracles_runs(gpu):

@@ -218,3 +218,83 @@ def test_config5_swap_layer_by_layer_with_ids_uploaded_once(gpu):
     holder = torch.arange(nb, device=gpu)
     holder[torch.from_numpy(new).to(gpu)] = torch.from_numpy(old).to(gpu)
     _check_pattern(pool3, holder, blk_term, elem_term, "layer-by-layer swap round trip")
+
+
+def _protocol_round_trip(gpu, worker, handle, pool3, blk_term, elem_term, old, host_ids, new, L):
+    """Write-through then fetch through the layer protocol, the model side played by
+    `LayerSyncHooks` on a stream of its own; returns what the worker recorded per leg."""
+    import asyncio
+    import threading
+
+    hooks = kvc.LayerSyncHooks(handle)
+    hooks.timeout = 120
+    model_stream = torch.cuda.Stream()
+    taken = []
+
+    def leg(maps, src, dst, saving):
+        errors = []
+
+        def run():
+            try:
+                asyncio.run(worker.copy_kv(maps, src, dst))
+            except Exception as exc:      # surfaces in the main thread below
+                errors.append(exc)
+        th = threading.Thread(target=run)
+        hooks.enable_record_after_execute = saving
+        hooks.enable_wait_before_execute = not saving
+        th.start()
+        with torch.cuda.stream(model_stream):
+            for l in range(L):
+                hooks.pre(l)
+                hooks.post(l)
+        th.join(timeout=300)
+        hooks.enable_record_after_execute = hooks.enable_wait_before_execute = False
+        assert not th.is_alive(), "the copy did not finish"
+        assert not errors, errors
+        torch.cuda.synchronize()
+        taken.append((worker.last_copy_went_through_host_bounce, worker.last_copy_swap_mode))
+
+    leg([kvc.BlockMapping.from_pairs(zip(old.tolist(), host_ids.tolist()))], kvc.Device.GPU, kvc.Device.Host, True)
+    host = worker.host_kv_caches.view(np.int16)
+    elem_np, blk_np = elem_term.cpu().numpy(), blk_term.cpu().numpy()
+    n = len(old)
+    for i in list(range(0, n, max(1, n // 48))) + [n - 1]:
+        for l in (0, L // 2, L - 1):
+            want = (blk_np[old[i]] + elem_np + np.int16(257 * l)).astype(np.int16)
+            assert np.array_equal(host[host_ids[i], l], want), f"host block {host_ids[i]}, layer {l}"
+    leg([kvc.BlockMapping.from_pairs(zip(host_ids.tolist(), new.tolist()))], kvc.Device.Host, kvc.Device.GPU, False)
+    return taken
+
+
+@pytest.mark.parametrize("bounce_bytes,through_bounce", [(1 << 30, True), (256 << 20, False)])
+def test_config5_layer_protocol_with_scattered_host_blocks_full(gpu, bounce_bytes, through_bounce):
+    """The path the layer protocol takes once an allocator has churned: Llama-3.1-70B
+    shape, 4096 blocks whose host blocks are every second block of an 8192-block
+    (40 GiB) pinned pool, written through and fetched back layer by layer behind the
+    model's hooks. With the default 1 GiB of dense pinned buffer every layer travels
+    as one copy and host threads place its 64 KiB rows (asserted); with a buffer too
+    small for two regions the worker falls back to the direct kernel (asserted).
+    Either way the payload arrives bit-exact and nothing else changes."""
+    s = wl.LLAMA_3_1_70B
+    nb, L, n = 16384, s.num_layers, SWAP_BLOCKS // 2
+    nhb = 2 * n
+    pool = torch.empty(L, nb, 2, s.block_size, s.num_kv_heads, s.head_dim, dtype=torch.bfloat16, device=gpu)
+    pool3 = pool.view(torch.int16).view(L, nb, -1)
+    blk_term, elem_term = _pattern_terms(nb, pool3.shape[2], gpu)
+    _fill_pattern(pool3, blk_term, elem_term)
+    old, _, new = wl.swap_round_trip(nb, n, seed=2)
+    host_ids = np.arange(0, nhb, 2, dtype=np.int64)
+    handle = kvc.KVWorkerHandle.create(L)
+    worker = kvc.KVWorker(pool, nhb, kv_worker_handle=handle, host_bounce_bytes=bounce_bytes)
+    try:
+        worker.host_kv_caches[1::2] = 0x5A5A            # the host blocks in between must stay as they are
+        taken = _protocol_round_trip(gpu, worker, handle, pool3, blk_term, elem_term, old, host_ids, new, L)
+        assert np.all(worker.host_kv_caches[1:256:2] == 0x5A5A) and np.all(worker.host_kv_caches[-1] == 0x5A5A)
+    finally:
+        worker.close()
+        handle.close()
+    want_mode = _lib.KVC_SWAP_STAGED if through_bounce else _lib.KVC_SWAP_DIRECT
+    assert taken == [(through_bounce, want_mode)] * 2, taken
+    holder = torch.arange(nb, device=gpu)
+    holder[torch.from_numpy(new).to(gpu)] = torch.from_numpy(old).to(gpu)
+    _check_pattern(pool3, holder, blk_term, elem_term, "layer protocol, scattered host blocks")

@@ -315,3 +315,106 @@ def test_plan_cache_matches_the_configured_pools():
         (32768, 65536, 8192, 0)
     p = kvc.plan_cache(80 << 30, 40 << 30, 1 << 30, 80, 8, 128, 16, torch.float16)
     assert (p.num_gpu_blocks, p.num_host_blocks, p.num_disk_blocks) == (16384, 8192, 204)
+
+
+# ------------------------------------------------------------------ waits of the layer protocol give up
+class _NeverDone:
+    """Stand-in for a GPU event whose work never completes (handled on the host only)."""
+    def query(self):
+        return False
+
+
+class _Done:
+    def query(self):
+        return True
+
+
+def test_notifier_rings_in_order_gives_up_at_its_deadline_and_stops():
+    import queue
+    import time
+    from lmserve_amd.kv_pool import KVWorkerHandle, _Notifier
+    bell = queue.Queue()
+    n = _Notifier(timeout=0.15)
+    n.submit(_Done(), bell)
+    n.submit(_Done(), bell)
+    assert bell.get(timeout=2) == b"" and bell.get(timeout=2) == b""
+    t0 = time.monotonic()
+    n.submit(_NeverDone(), bell)
+    n.submit(_Done(), bell)              # queued behind the stuck one: dropped with it, never rung
+    while n.failed is None and time.monotonic() - t0 < 3:
+        time.sleep(0.01)
+    assert n.failed is not None and 0.14 <= time.monotonic() - t0 < 2.0
+    time.sleep(0.05)
+    assert bell.empty()
+    with pytest.raises(TimeoutError):
+        n.submit(_Done(), bell)
+    t0 = time.monotonic()
+    n.stop()
+    assert not n.thread.is_alive() and time.monotonic() - t0 < 1.0
+    # without a deadline, stop() still ends a wait that would never finish
+    n = _Notifier(timeout=None)
+    n.submit(_NeverDone(), bell)
+    time.sleep(0.05)
+    t0 = time.monotonic()
+    n.stop()
+    assert not n.thread.is_alive() and time.monotonic() - t0 < 1.0 and bell.empty()
+    # the handle passes its own deadline on
+    h = KVWorkerHandle([], [], host_wait_timeout=0.1, sync="host")
+    h.ring_when_done(_NeverDone(), bell)
+    assert h._notifier.timeout == 0.1
+    h.close()
+
+
+def test_save_loop_gives_up_when_the_model_stops_posting_layers():
+    """`KVWorker._doorbell` (the poll of kv_worker.py:279-281 with a deadline) on a
+    queue nobody rings: TimeoutError after `host_wait_timeout`, not a hang."""
+    import asyncio
+    import queue
+    import time
+    from lmserve_amd.kv_worker import KVWorker
+
+    class Stub:
+        host_wait_timeout = 0.1
+    bell = queue.Queue()
+    t0 = time.monotonic()
+    with pytest.raises(TimeoutError):
+        asyncio.run(KVWorker._doorbell(Stub(), bell, 3))
+    assert 0.09 <= time.monotonic() - t0 < 2.0
+    bell.put(b"")
+    asyncio.run(KVWorker._doorbell(Stub(), bell, 3))       # a token that is there is taken at once
+    assert bell.empty()
+
+
+def test_few_hardware_queues_are_warned_about_once():
+    import warnings
+    from lmserve_amd import kv_worker
+    kv_worker._warned_about_queues = False
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        assert kv_worker.warn_if_few_hardware_queues({"GPU_MAX_HW_QUEUES": "8"}) is False
+        assert kv_worker.warn_if_few_hardware_queues({"GPU_MAX_HW_QUEUES": "4"}) is True
+        assert kv_worker.warn_if_few_hardware_queues({}) is False          # once per process
+    assert len(caught) == 1 and "GPU_MAX_HW_QUEUES" in str(caught[0].message)
+    kv_worker._warned_about_queues = False
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        assert kv_worker.warn_if_few_hardware_queues({}) is True           # unset = the runtime's 4
+    kv_worker._warned_about_queues = False
+
+
+def test_pool_in_a_segment_of_two_gib_or_more_is_not_exported():
+    """The IPC handle of a tensor covers its whole allocator segment; segments of
+    2 GiB or more must never be shared between processes here."""
+    import torch
+    from lmserve_amd import kv_pool
+    t = torch.zeros(16, dtype=torch.bfloat16)
+    base = t.untyped_storage().data_ptr()
+    small = [{"address": base - 4096, "total_size": 1 << 30}]
+    large = [{"address": base - 4096, "total_size": 2 << 30}]
+    elsewhere = [{"address": base + (1 << 40), "total_size": 4 << 30}]
+    assert kv_pool.allocator_segment_bytes(t, small) == 1 << 30
+    assert kv_pool.allocator_segment_bytes(t, elsewhere) is None
+    kv_pool.check_ipc_segment(t, small)
+    kv_pool.check_ipc_segment(t, elsewhere)          # not listed: judged by the storage's own size
+    with pytest.raises(ValueError, match="segment"):
+        kv_pool.check_ipc_segment(t, large)

@@ -167,3 +167,52 @@ def test_noalloc_swap_at_its_maximum_size(gpu):
     finally:
         torch.cuda.synchronize()
         host.close()
+
+
+def test_noalloc_swap_leaves_device_memory_alone_and_replays_from_a_graph(gpu):
+    """After one warm-up call (which looks up the static array's address), further
+    calls change neither the free device memory nor torch's allocator; a call
+    recorded into a hipGraph replays bit-exactly, twice, with eager work and a
+    synchronisation between the replays."""
+    pool, dpool_new, dpool_ref, host_new, host_ref = _setup(gpu, 21)
+    staging = torch.empty(1 << 16, dtype=torch.uint8, device=gpu)
+    try:
+        rng = np.random.default_rng(22)
+        one = np.zeros(1, dtype=np.int64)
+        assert _noalloc(1, dpool_new, host_new, one, one) == _lib.KVC_OK          # warm-up, outside any capture
+        assert _existing(1, dpool_ref, host_ref, one, one, staging) == _lib.KVC_OK
+        torch.cuda.synchronize()
+        free_before, _ = torch.cuda.mem_get_info()
+        reserved_before = torch.cuda.memory_reserved()
+        for n in (700, 3, 1200):
+            gpu_ids = rng.permutation(NB)[:n].astype(np.int64)
+            host_ids = rng.permutation(NHB)[:n].astype(np.int64)
+            assert _noalloc(1, dpool_new, host_new, gpu_ids, host_ids) == _lib.KVC_OK
+            assert _noalloc(0, dpool_new, host_new, rng.permutation(NB)[:n].astype(np.int64), host_ids) == _lib.KVC_OK
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.memory_reserved() == reserved_before
+
+        # recorded into a graph: the ids travel as kernel arguments, so a replay moves the same blocks again
+        dpool_new.copy_(dpool_ref)
+        host_new.array[...] = host_ref.array
+        n = 600
+        gpu_ids = rng.permutation(NB)[:n].astype(np.int64)
+        host_ids = rng.permutation(NHB)[:n].astype(np.int64)
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            assert _noalloc(1, dpool_new, host_new, gpu_ids, host_ids, stream=side.cuda_stream) == _lib.KVC_OK
+        for rep in range(2):
+            fresh = to_bf16(random_pool((L, NB) + BLOCK_SHAPE, 30 + rep), gpu)
+            dpool_new.copy_(fresh)                                      # eager work between the replays
+            dpool_ref.copy_(fresh)
+            torch.cuda.synchronize()
+            graph.replay()
+            assert _existing(1, dpool_ref, host_ref, gpu_ids, host_ids, staging) == _lib.KVC_OK
+            torch.cuda.synchronize()
+            assert np.array_equal(host_new.array, host_ref.array), f"replay {rep}"
+    finally:
+        torch.cuda.synchronize()
+        host_new.close()
+        host_ref.close()
