@@ -612,6 +612,33 @@ __global__ void batch_indices_positions_kernel(const int32_t* append_indptr,
 // token count. The first token of every run writes it.
 constexpr int kPrepThreads = 1024;
 
+// Inclusive scan of three values over the workgroup's 1024 lanes: shuffles inside
+// each wavefront, then the 16 wavefront totals through LDS (two barriers).
+__device__ __forceinline__ void scan3(int32_t& q, int32_t& n, int32_t& r, int32_t (*wave_sums)[3]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int32_t uq = __shfl_up(q, off, 64), un = __shfl_up(n, off, 64), ur = __shfl_up(r, off, 64);
+    if (lane >= off) {
+      q += uq;
+      n += un;
+      r += ur;
+    }
+  }
+  __syncthreads();  // the previous round's readers are done with wave_sums
+  if (lane == 63) {
+    wave_sums[wave][0] = q;
+    wave_sums[wave][1] = n;
+    wave_sums[wave][2] = r;
+  }
+  __syncthreads();
+  for (int w = 0; w < wave; ++w) {
+    q += wave_sums[w][0];
+    n += wave_sums[w][1];
+    r += wave_sums[w][2];
+  }
+}
+
 __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
     const int32_t* input_lens, const int32_t* context_lens, const int32_t* num_blocks,
     const int32_t* kv_indices, int32_t batch_size, int64_t num_kv_indices, int32_t page_size,
@@ -619,54 +646,50 @@ __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
     int32_t* batch_indices, int32_t* positions, int64_t* slot_mapping, int32_t* run_indptr,
     int32_t* runs, int32_t* num_runs, int64_t max_runs) {
   __shared__ int32_t carry[3];
-  __shared__ int32_t part_q[kPrepThreads];
-  __shared__ int32_t part_b[kPrepThreads];
-  __shared__ int32_t part_r[kPrepThreads];
+  __shared__ int32_t wave_sums[kPrepThreads / 64][3];
+  // prefix sums of a batch that fits one chunk stay in LDS for the per-token part
+  __shared__ int32_t lds_cu[kPrepThreads + 1], lds_indptr[kPrepThreads + 1], lds_runptr[kPrepThreads + 1];
   const int tid = threadIdx.x;
+  const bool in_lds = batch_size <= kPrepThreads;
   if (tid == 0) {
     carry[0] = carry[1] = carry[2] = 0;
     cu_seqlens_q[0] = 0;
     kv_indptr[0] = 0;
     if (run_indptr) run_indptr[0] = 0;
+    lds_cu[0] = lds_indptr[0] = lds_runptr[0] = 0;
   }
   // every descriptor starts out empty: a run whose first token lies beyond `nnz` is never written
   if (runs)
     for (int64_t r = tid; r < max_runs; r += kPrepThreads)
       reinterpret_cast<int4*>(runs)[r] = make_int4(0, -1, 0, 0);
   __syncthreads();
-  // chunked inclusive scan (Hillis-Steele inside a chunk of kPrepThreads requests)
   for (int32_t base = 0; base < batch_size; base += kPrepThreads) {
     const int32_t b = base + tid;
-    const int32_t q = b < batch_size ? input_lens[b] : 0;
-    const int32_t n = b < batch_size ? num_blocks[b] : 0;
+    int32_t q = b < batch_size ? input_lens[b] : 0;
+    int32_t n = b < batch_size ? num_blocks[b] : 0;
     const int32_t ctx = b < batch_size ? context_lens[b] : 0;
     // runs of the request: the blocks its new positions [ctx - q, ctx) touch
-    const int32_t nr = (q > 0 && ctx >= q) ? (ctx - 1) / page_size - (ctx - q) / page_size + 1 : 0;
-    part_q[tid] = q;
-    part_b[tid] = n;
-    part_r[tid] = nr;
-    __syncthreads();
-    for (int off = 1; off < kPrepThreads; off <<= 1) {
-      const int32_t aq = tid >= off ? part_q[tid - off] : 0;
-      const int32_t ab = tid >= off ? part_b[tid - off] : 0;
-      const int32_t ar = tid >= off ? part_r[tid - off] : 0;
-      __syncthreads();
-      part_q[tid] += aq;
-      part_b[tid] += ab;
-      part_r[tid] += ar;
-      __syncthreads();
-    }
+    int32_t nr = (q > 0 && ctx >= q) ? (ctx - 1) / page_size - (ctx - q) / page_size + 1 : 0;
+    scan3(q, n, nr, wave_sums);
+    q += carry[0];
+    n += carry[1];
+    nr += carry[2];
     if (b < batch_size) {
-      cu_seqlens_q[b + 1] = carry[0] + part_q[tid];
-      kv_indptr[b + 1] = carry[1] + part_b[tid];
-      if (run_indptr) run_indptr[b + 1] = carry[2] + part_r[tid];
+      cu_seqlens_q[b + 1] = q;
+      kv_indptr[b + 1] = n;
+      if (run_indptr) run_indptr[b + 1] = nr;
       kv_last_page_len[b] = ctx > 0 ? (ctx - 1) % page_size + 1 : 0;
+      if (in_lds) {
+        lds_cu[b + 1] = q;
+        lds_indptr[b + 1] = n;
+        lds_runptr[b + 1] = nr;
+      }
     }
-    __syncthreads();
+    __syncthreads();  // everyone has read the carry
     if (tid == kPrepThreads - 1) {
-      carry[0] += part_q[tid];
-      carry[1] += part_b[tid];
-      carry[2] += part_r[tid];
+      carry[0] = q;
+      carry[1] = n;
+      carry[2] = nr;
     }
     __syncthreads();
   }
@@ -674,7 +697,10 @@ __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
   // per token: find its request by bisection over the prefix sums just written
   // (visible to the whole workgroup after the barrier above); the request's new
   // tokens occupy positions [context - input, context)
-  const int64_t total = cu_seqlens_q[batch_size];
+  const int32_t* cu = in_lds ? lds_cu : cu_seqlens_q;
+  const int32_t* indptr = in_lds ? lds_indptr : kv_indptr;
+  const int32_t* runptr = in_lds ? lds_runptr : run_indptr;
+  const int64_t total = carry[0];
   const int64_t limit = total < nnz ? total : nnz;
   for (int64_t out = tid; out < nnz; out += kPrepThreads) {
     if (out >= limit) {  // beyond this step's tokens: entries every write kernel skips
@@ -686,30 +712,30 @@ __global__ __launch_bounds__(kPrepThreads) void build_write_index_kernel(
     int32_t lo = 0, hi = batch_size;  // invariant: cu[lo] <= out < cu[hi]
     while (hi - lo > 1) {
       const int32_t mid = (lo + hi) >> 1;
-      if (cu_seqlens_q[mid] <= out) lo = mid;
+      if (cu[mid] <= out) lo = mid;
       else hi = mid;
     }
     const int32_t b = lo;
-    const int32_t begin = cu_seqlens_q[b];
-    const int32_t n_new = cu_seqlens_q[b + 1] - begin;
+    const int32_t begin = cu[b];
+    const int32_t n_new = cu[b + 1] - begin;
     const int32_t j = (int32_t)(out - begin);
-    const int32_t pos = context_lens[b] - n_new + j;
+    const int32_t ctx = context_lens[b];
+    const int32_t pos = ctx - n_new + j;
     batch_indices[out] = b;
     positions[out] = pos;
-    const int64_t it = (int64_t)kv_indptr[b] + pos / page_size;
-    const int64_t table_end = kv_indptr[b + 1] < num_kv_indices ? kv_indptr[b + 1] : num_kv_indices;
+    const int64_t it = (int64_t)indptr[b] + pos / page_size;
+    const int64_t table_end = indptr[b + 1] < num_kv_indices ? indptr[b + 1] : num_kv_indices;
     const bool in_table = pos >= 0 && it >= 0 && it < table_end;
-    if (slot_mapping)
-      slot_mapping[out] = in_table ? (int64_t)kv_indices[it] * page_size + pos % page_size : -1;
-    if (runs && pos >= 0 && context_lens[b] >= n_new && (j == 0 || pos % page_size == 0)) {
-      const int32_t first_pos = context_lens[b] - n_new;
-      const int64_t r = (int64_t)run_indptr[b] + (pos / page_size - first_pos / page_size);
+    const int32_t block = in_table ? kv_indices[it] : -1;
+    if (slot_mapping) slot_mapping[out] = in_table ? (int64_t)block * page_size + pos % page_size : -1;
+    if (runs && pos >= 0 && ctx >= n_new && (j == 0 || pos % page_size == 0)) {
+      const int32_t first_pos = ctx - n_new;
+      const int64_t r = (int64_t)runptr[b] + (pos / page_size - first_pos / page_size);
       if (r >= 0 && r < max_runs) {
         int64_t count = page_size - pos % page_size;
         if (count > n_new - j) count = n_new - j;
         if (count > nnz - out) count = nnz - out;
-        reinterpret_cast<int4*>(runs)[r] =
-            make_int4((int32_t)out, in_table ? kv_indices[it] : -1, pos % page_size, (int32_t)count);
+        reinterpret_cast<int4*>(runs)[r] = make_int4((int32_t)out, block, pos % page_size, (int32_t)count);
       }
     }
   }
