@@ -18,7 +18,7 @@ against 8 TB/s), `cpu_baseline` (the torch-CPU statement of the same step on the
 host cores, bounded sample) and `configs`: one short object per benchmark
 configuration and form (us, GB/s, fraction of 8 TB/s, and counter traffic over
 algorithmic bytes where it has been measured). Every other row (variants, passes, names in prose) goes to
-the details file (`--details`, default gpurun_out/bench_details.json) and to
+the details file (`--details`, default bench_out/bench_details.json) and to
 stderr, never to stdout.
 
 Sections beyond the operations the benchmark names are opt-in
@@ -72,7 +72,7 @@ def parse_args(argv=None):
                         "decode step, index build included, replayed from one hipGraph). Opt-in: rope, shard, "
                         "index, overlap, twoproc, disk, sweep, calib, translation. 'none' = headline only")
     p.add_argument("--details", default=None,
-                   help="file for every row beyond the final line (default gpurun_out/bench_details.json; "
+                   help="file for every row beyond the final line (default bench_out/bench_details.json; "
                         "'-' = stderr only)")
     p.add_argument("--settle-seconds", type=float, default=0.0,
                    help="quiet time before sections that use the copy engines after the bench has freed a "
@@ -220,7 +220,7 @@ def write_details(path, details):
     if path == "-":
         return None
     if path is None:
-        path = os.path.join(REPO_ROOT, "gpurun_out", "bench_details.json")
+        path = os.path.join(REPO_ROOT, "bench_out", "bench_details.json")
     try:
         os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
         with open(path, "w") as f:

@@ -24,7 +24,8 @@ extern "C" {
  *   "direct_max_wgs"                  grid cap of the direct swap kernel
  *   "write_vpt"                       vectors per lane in the write kernel (0 = by size, 1, 2, 4, 8)
  *   "write_threads"                   lanes per workgroup in the write kernel (0 = by size, 64, 128, 256)
- *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads
+ *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads (applied to rows
+ *                                     of 1 KiB or more); default 3
  *   "write_order"                     1 = a token's workgroups are neighbours in the grid
  *   "write_planes"                    the plane kernel (lanes of a workgroup run over consecutive
  *                                     tokens of one (layer, K|V) plane): 0 = never, 1 = by row

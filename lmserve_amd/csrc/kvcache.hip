@@ -73,7 +73,10 @@ struct Tuning {
   int copy_max_wgs = 0;     // 0 = one workgroup per chunk, else grid cap
   int copy_order = 0;       // copy_tiles: 1 = walk all blocks of a layer before the next layer
   int write_vpt = 0;        // vectors per lane in write_rows, 0 = by size
-  int write_nt = 1;         // write_rows: bit 0 non-temporal stores, bit 1 non-temporal loads
+  int write_nt = 3;         // write kernels: bit 0 non-temporal stores, bit 1 non-temporal loads (rows of
+                            // 1 KiB or more only: narrower rows measured 4 % slower with them). Loads:
+                            // -6 % at the 64 MiB decode step, -7 to -17 % at one layer of a 2048-token
+                            // chunk, -2 to -3 % at 224-256 MiB, neutral at 2 and 32 MiB
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
   int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
   int write_planes = 1;     // the plane kernel (lanes of a workgroup run over consecutive tokens of
@@ -117,7 +120,7 @@ Knob* knobs(int* count) {
       {"copy_max_wgs", &g_tune.copy_max_wgs, 0},
       {"copy_order", &g_tune.copy_order, 0},
       {"write_vpt", &g_tune.write_vpt, 0},
-      {"write_nt", &g_tune.write_nt, 1},
+      {"write_nt", &g_tune.write_nt, 3},
       {"write_order", &g_tune.write_order, 0},
       {"write_threads", &g_tune.write_threads, 0},
       {"write_planes", &g_tune.write_planes, 1},
@@ -325,7 +328,7 @@ __global__ __launch_bounds__(kThreads) void write_rows_kernel(WriteArgs a) {
 //     several loads in flight per lane.
 // 16-byte vectors and a power-of-two number of them per row (up to 256) only;
 // blockIdx.x = plane_group * num_token_groups + token_group.
-template <int VPT, bool PAGED, bool NT>
+template <int VPT, bool PAGED, bool NT, bool NTL>
 __global__ __launch_bounds__(1024) void write_planes_kernel(WriteArgs a) {
   using V = u32x4;
   const uint32_t pg = blockIdx.x / a.num_token_groups;
@@ -345,7 +348,7 @@ __global__ __launch_bounds__(1024) void write_planes_kernel(WriteArgs a) {
     const int64_t layer = plane >> 1;
     const char* src = (plane & 1u) ? value_row + layer * a.value_layer_stride
                                    : key_row + layer * a.key_layer_stride;
-    return *reinterpret_cast<const V*>(src);
+    return ld<NTL>(reinterpret_cast<const V*>(src));
   };
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
@@ -887,8 +890,10 @@ void launch_write(const WriteArgs& a, int vec, const WriteLaunch& l, hipStream_t
 template <int VPT, bool PAGED>
 void launch_planes_nt(const WriteArgs& a, const WriteLaunch& l, hipStream_t s) {
   const dim3 grid(l.grid), block(l.threads);
-  if (l.nt) hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, true>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, false>), grid, block, 0, s, a);
+  if (l.nt && l.ntl) hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, true, true>), grid, block, 0, s, a);
+  else if (l.nt) hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, true, false>), grid, block, 0, s, a);
+  else if (l.ntl) hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, false, true>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((write_planes_kernel<VPT, PAGED, false, false>), grid, block, 0, s, a);
 }
 
 template <bool PAGED>
@@ -1068,6 +1073,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
     a.tokens_per_wg = l.threads / a.vecs_per_row;
     a.num_planes = (uint32_t)num_planes;
     l.nt = (g_tune.write_nt & 1) != 0;
+    l.ntl = (g_tune.write_nt & 2) != 0 && !narrow;
     const int64_t plane_groups = (a.num_planes + l.vpt - 1) / l.vpt;
     const int64_t max_groups = std::max<int64_t>(1, 0x7fffffffll / plane_groups);
     const int64_t max_tokens = max_groups * a.tokens_per_wg;
@@ -1088,7 +1094,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
       }
       KVC_HIP(hipGetLastError());
     }
-    g_last = LastLaunch{KVC_KERNEL_WRITE_PLANES, 16, l.vpt, l.threads, l.grid, l.nt, a.pipe};
+    g_last = LastLaunch{KVC_KERNEL_WRITE_PLANES, 16, l.vpt, l.threads, l.grid, (l.nt ? 1 : 0) | (l.ntl ? 2 : 0), a.pipe};
     return KVC_OK;
   }
 
@@ -1127,7 +1133,7 @@ int run_write(const char* fn, const void* key, const void* value, void* kc, void
   const int64_t lanes = (items64 + l.vpt - 1) / l.vpt;
   l.threads = (unsigned)std::min<int64_t>(wg, (lanes + 63) / 64 * 64);
   l.nt = (g_tune.write_nt & 1) != 0;
-  l.ntl = (g_tune.write_nt & 2) != 0;
+  l.ntl = (g_tune.write_nt & 2) != 0 && g.row_elems * E >= 1024;
   a.pipe = g_tune.write_pipe >= 0 ? g_tune.write_pipe : (l.vpt > 1 ? 1 : 0);
   const int64_t groups = (items64 + (int64_t)l.vpt * l.threads - 1) / ((int64_t)l.vpt * l.threads);
 

@@ -172,7 +172,7 @@ def test_tuning_knobs_read_back_and_reset():
     L = _lib.lib()
     assert L.kvc_tuning_modified() == 0
     defaults = {"copy_unroll": 0, "gather_unroll": 0, "copy_nt": 1, "copy_max_wgs": 0, "copy_order": 0,
-                "write_vpt": 0, "write_nt": 1, "write_order": 0, "write_threads": 0, "write_planes": 1,
+                "write_vpt": 0, "write_nt": 3, "write_order": 0, "write_threads": 0, "write_planes": 1,
                 "write_planes_vpt": 0, "write_planes_min_bytes": 256 << 10, "write_planes_max_vpr": 256, "write_planes_threads": 0,
                 "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 1 << 20, "rope_threads": 0, "disk_bounce_mib": 4,
                 "runs_unroll": 0, "runs_order": 1, "runs_nt": 1}

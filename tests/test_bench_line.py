@@ -21,7 +21,7 @@ def _head():
                              "sample": "6097 decode-step writes (T=256, 32 layers) via oracle/torch_cpu.py, pool 2048 "
                                        "blocks/layer, 10.0 s",
                              "others_gbps": {"cfg3": 98.62, "cfg4": 8.92, "cfg5_out": 8.48, "cfg5_in": 32.07}},
-            "details": "gpurun_out/bench_details.json"}
+            "details": "bench_out/bench_details.json"}
 
 
 def _row(i):

@@ -144,6 +144,8 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
     # workgroup size and load order vary over the cases (both are by rule otherwise)
     _lib.set_tuning("write_planes_threads", (0, 256, 512, 1024)[(T + L) % 4])
     _lib.set_tuning("write_pipe", (-1, 0, 1)[(T + vpt) % 3])
+    nt = (3, 1, 2, 0)[(T + vpt + L + int(paged)) % 4]       # every load/store kind over the cases
+    _lib.set_tuning("write_nt", nt)
     if paged:
         # requests of up to three tokens, each token on a page of its own:
         # page = slot // bs at table entry j, position = j * bs + slot % bs
@@ -165,6 +167,8 @@ def test_narrow_rows_take_the_plane_kernel_and_match_the_oracle(gpu, T, H, D, L,
     torch.cuda.synchronize()
     ran = _lib.last_launch()
     assert ran["kernel"] == _lib.KVC_KERNEL_WRITE_PLANES and ran["vec_bytes"] == 16
+    # non-temporal loads are taken for rows of 1 KiB or more only
+    assert ran["non_temporal"] == ((nt & 1) | (nt & 2 if H * D * 2 >= 1024 else 0))
     if vpt:
         assert ran["per_lane"] == min(vpt, 1 << (2 * L - 1).bit_length())
     assert np.array_equal(bits_of(dpool), want)
