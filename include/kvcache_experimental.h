@@ -39,6 +39,7 @@ extern "C" {
  *   "runs_unroll", "runs_order", "runs_nt"   the run-descriptor write below
  *   "auto_min_extent_bytes"           KVC_SWAP_AUTO: mean bytes per PCIe copy from which a call is staged
  *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
+ *   "rope_nt"                         non-temporal loads in that kernel: bit 0 the K and V rows, bit 1 the Q rows
  *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier
  * Unknown key: KVC_ERR_INVALID_ARG. kvc_reset_tuning puts every knob back to its
  * default; kvc_tuning_modified counts the knobs that are not at their default. */

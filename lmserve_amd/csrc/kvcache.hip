@@ -135,6 +135,7 @@ Knob* knobs(int* count) {
       {"runs_order", &g_tune.runs_order, 1},
       {"runs_nt", &g_tune.runs_nt, 1},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
+      {"rope_nt", &kvc::g_rope_tune.nt, 3},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
   };
   *count = (int)(sizeof(table) / sizeof(table[0]));

@@ -140,7 +140,14 @@ struct RopeArgs {
 // consecutive vectors): all of the lane's global loads are issued first, the
 // cos/sin row is staged in LDS while they are in flight, then the lane computes
 // and stores.
-template <typename T, bool VECTOR, int IPL>
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const char* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  else return *reinterpret_cast<const u32x4*>(p);
+}
+
+// NTL: non-temporal loads, bit 0 for the K and V rows, bit 1 for the Q rows.
+template <typename T, bool VECTOR, int IPL, int NTL>
 __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
   using VT = Vec<T>;
   constexpr int EV = VECTOR ? VT::kElems : 1;
@@ -189,8 +196,13 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
       const char* in = (is_k[j] ? a.key + (int64_t)t * a.k_token_stride
                                 : a.query + (int64_t)t * a.q_token_stride) + in_off[j];
       if constexpr (VECTOR) {
-        rx[j] = *reinterpret_cast<const u32x4*>(in + (int64_t)e0[j] * E);
-        ry[j] = *reinterpret_cast<const u32x4*>(in + (int64_t)(half + e0[j]) * E);
+        if (is_k[j]) {
+          rx[j] = ld16<(NTL & 1) != 0>(in + (int64_t)e0[j] * E);
+          ry[j] = ld16<(NTL & 1) != 0>(in + (int64_t)(half + e0[j]) * E);
+        } else {
+          rx[j] = ld16<(NTL & 2) != 0>(in + (int64_t)e0[j] * E);
+          ry[j] = ld16<(NTL & 2) != 0>(in + (int64_t)(half + e0[j]) * E);
+        }
       } else {
         sx[j] = VT::load1(in + (int64_t)e0[j] * E);
         sy[j] = VT::load1(in + (int64_t)(half + e0[j]) * E);
@@ -205,13 +217,13 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
       in_off[j] = ((int64_t)hh * D + e0[j]) * E;
       const char* in = (is_k[j] ? a.key + (int64_t)t * a.k_token_stride
                                 : a.query + (int64_t)t * a.q_token_stride) + in_off[j];
-      if constexpr (VECTOR) rx[j] = *reinterpret_cast<const u32x4*>(in);
+      if constexpr (VECTOR) rx[j] = is_k[j] ? ld16<(NTL & 1) != 0>(in) : ld16<(NTL & 2) != 0>(in);
       else sx[j] = VT::load1(in);
     } else if (item < rot_items + tail_items + v_items) {
       kind[j] = kValue;
       in_off[j] = (int64_t)(item - rot_items - tail_items) * EV * E;
       const char* in = a.value + (int64_t)t * a.v_token_stride + in_off[j];
-      if constexpr (VECTOR) rx[j] = *reinterpret_cast<const u32x4*>(in);
+      if constexpr (VECTOR) rx[j] = ld16<(NTL & 1) != 0>(in);
       else sx[j] = VT::load1(in);
     }
   }
@@ -330,7 +342,16 @@ __global__ __launch_bounds__(kThreads) void rope_cache_kernel(RopeArgs a) {
 // or already has enough workgroups in flight).
 template <typename T, bool VECTOR>
 void launch_rope_ipl(const RopeArgs& a, dim3 grid, dim3 block, hipStream_t s) {
-  hipLaunchKernelGGL((rope_cache_kernel<T, VECTOR, 1>), grid, block, 0, s, a);
+  if constexpr (VECTOR) {
+    switch (kvc::g_rope_tune.nt & 3) {
+      case 1: hipLaunchKernelGGL((rope_cache_kernel<T, true, 1, 1>), grid, block, 0, s, a); break;
+      case 2: hipLaunchKernelGGL((rope_cache_kernel<T, true, 1, 2>), grid, block, 0, s, a); break;
+      case 3: hipLaunchKernelGGL((rope_cache_kernel<T, true, 1, 3>), grid, block, 0, s, a); break;
+      default: hipLaunchKernelGGL((rope_cache_kernel<T, true, 1, 0>), grid, block, 0, s, a); break;
+    }
+  } else {
+    hipLaunchKernelGGL((rope_cache_kernel<T, false, 1, 0>), grid, block, 0, s, a);
+  }
 }
 
 template <typename T>

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 import lmserve_amd as kvc
-from lmserve_amd import rotary
+from lmserve_amd import _lib, rotary
 import workloads as wl
 from oracle import kvc_oracle as orc
 from oracle import rope_oracle as ro
@@ -132,6 +132,37 @@ def test_fused_slot_mapped_write_places_the_rotated_key_bit_exactly(gpu, dtype, 
     q2, none = kvc.rotary_pos_emb_and_cache(q.to(gpu), k.to(gpu), v.to(gpu), pos.to(gpu), cs.to(gpu),
                                             D, pool2, torch.from_numpy(slots).to(gpu), return_key=False)
     assert none is None and torch.equal(q2, plain_q) and torch.equal(pool2, pool)
+
+
+@pytest.mark.parametrize("dtype,D,rd", [(torch.bfloat16, 128, 128), (torch.float16, 64, 32), (torch.float32, 32, 32)])
+def test_every_load_policy_of_the_rotation_kernel_gives_the_same_bits(gpu, dtype, D, rd):
+    """`rope_nt` selects one of four instantiations per storage type (plain or
+    non-temporal loads of K/V and of Q); results may not depend on it, in place
+    or out of place, with and without a cache."""
+    T, Hq, Hkv, nb, bs = 133, 8, 2, 16, 16
+    q, k, v, pos, cs = _case(gpu, T, Hq, Hkv, D, rd, dtype, seed=11)
+    slots = torch.from_numpy(np.random.default_rng(12).permutation(nb * bs)[:T].astype(np.int64)).to(gpu)
+    q, k, v, pos, cs = q.to(gpu), k.to(gpu), v.to(gpu), pos.to(gpu), cs.to(gpu)
+    results = []
+    for nt in (0, 1, 2, 3):
+        _lib.set_tuning("rope_nt", nt)
+        pool = torch.zeros(nb, 2, bs, Hkv, D, dtype=dtype, device=gpu)
+        q_out, k_out = kvc.rotary_pos_emb_and_cache(q, k, v, pos, cs, D, pool, slots)
+        plain_q, plain_k = kvc.rotary_pos_emb(q, k, pos, cs, D)
+        q_in, k_in = q.clone(), k.clone()
+        rc = _lib.lib().kvc_rotary_pos_emb(q_in.data_ptr(), k_in.data_ptr(), pos.data_ptr(), pos.element_size(),
+                                           cs.data_ptr(), cs.shape[0], T, Hq, Hkv, D, rd, Hq * D, Hkv * D,
+                                           q_in.data_ptr(), k_in.data_ptr(), Hq * D, Hkv * D,
+                                           rotary._DTYPES[dtype], torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert torch.equal(q_in, plain_q) and torch.equal(k_in, plain_k)
+        assert torch.equal(q_out, plain_q) and torch.equal(k_out, plain_k)
+        results.append((q_out, k_out, pool))
+    for r in results[1:]:
+        for a, b in zip(results[0], r):
+            assert torch.equal(a, b)
+    _check_rotation(results[0][0].cpu(), q.cpu(), pos.cpu(), cs.cpu(), D, dtype, "query")
 
 
 def test_fused_paged_write_equals_rotation_then_append(gpu):
