@@ -22,13 +22,15 @@ inline int log2_exact(int64_t x) {
 
 // Launch shape of the rotation kernel, set through kvc_set_tuning
 // ("rope_threads": 64/128/256 lanes per workgroup, 0 = by size; "rope_nt":
-// non-temporal loads, bit 0 the K and V rows, bit 1 the Q rows: the kernel reads
-// each of them once. Both on measured 4.06 against 4.46 us per layer at a
-// 256-token decode step and 9.05 against 9.70 us at a 2048-token chunk; either
-// bit alone gains a third of that or nothing).
+// non-temporal loads, bit 0 the K and V rows, bit 1 the Q rows). Off by default:
+// with both bits a launch whose Q/K/V come from HBM gains 7-9 % (9.25 against
+// 9.94 us per layer at a 2048-token chunk over 28 distinct source sets), but
+// a forward pass hands the kernel rows its projection has just written, and
+// with sources that are still in cache the same launch is 10 % slower (8.77
+// against 7.95 us) and a 256-token decode launch is unchanged.
 struct RopeTuning {
   int threads = 0;
-  int nt = 3;
+  int nt = 0;
 };
 extern RopeTuning g_rope_tune;
 

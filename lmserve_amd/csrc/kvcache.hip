@@ -75,8 +75,9 @@ struct Tuning {
   int write_vpt = 0;        // vectors per lane in write_rows, 0 = by size
   int write_nt = 3;         // write kernels: bit 0 non-temporal stores, bit 1 non-temporal loads (rows of
                             // 1 KiB or more only: narrower rows measured 4 % slower with them). Loads:
-                            // -6 % at the 64 MiB decode step, -7 to -17 % at one layer of a 2048-token
-                            // chunk, -2 to -3 % at 224-256 MiB, neutral at 2 and 32 MiB
+                            // -3 % at the 64 MiB decode step, -2 to -3 % at 224-256 MiB, -10 to -15 %
+                            // for one layer per launch when the K/V rows come from HBM, neutral when
+                            // they are still in cache (one source set, or a producer kernel in front)
   int write_order = 0;      // write_rows: 1 = a token's workgroups are neighbours in the grid
   int write_threads = 0;    // write_rows: lanes per workgroup (64, 128, 256), 0 = by size
   int write_planes = 1;     // the plane kernel (lanes of a workgroup run over consecutive tokens of
@@ -135,7 +136,7 @@ Knob* knobs(int* count) {
       {"runs_order", &g_tune.runs_order, 1},
       {"runs_nt", &g_tune.runs_nt, 1},
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
-      {"rope_nt", &kvc::g_rope_tune.nt, 3},
+      {"rope_nt", &kvc::g_rope_tune.nt, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
   };
   *count = (int)(sizeof(table) / sizeof(table[0]));
