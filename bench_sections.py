@@ -881,3 +881,58 @@ def bench_decode_step_graph(torch, kvc, wl, s8, pool, L, num_blocks, dev, steps=
                             "gbps": round(bytes_step / wall_us / 1e3),
                             "frac": round(bytes_step / wall_us / 1e3 / HBM_PEAK_GBPS, 3)})
     return compact, detail
+
+
+def bench_load_policy(torch, kvc, wl, dev):
+    """A/B of plain against non-temporal loads of the source rows, per layer, in one
+    process: the per-layer write (`write_nt` 1 against 3) and the fused rotation
+    (`rope_nt` 0 against 3), with the layers of a replayed step cycling through
+    `sets` distinct source sets (1 = rows still in cache, as after the projection
+    of a forward pass; one set per layer = rows from HBM or the last-level cache).
+    Two rounds, interleaved; microseconds per layer from a hipGraph replay."""
+    from lmserve_amd import _lib
+    out = []
+    nb = 16384
+    for label, shape, Hq, T, decode in (("cfg2 decode batch", wl.LLAMA_3_8B, 32, 256, True),
+                                        ("cfg3 prefill chunk", wl.QWEN_2_5_7B, 28, 2048, False)):
+        L, Hkv, D = shape.num_layers, shape.num_kv_heads, shape.head_dim
+        pool, _ = alloc_pool(torch, shape, nb, dev)
+        w = wl.decode_step(shape, num_blocks=nb, batch=T, max_context=100, seed=1) if decode \
+            else wl.chunked_prefill(shape, num_blocks=nb, seed=1)
+        idx = kvc.to_device(w.index, shape.block_size, dev)
+        cs = kvc.make_cos_sin_cache(D, 40000, 500000.0, dtype=torch.bfloat16).to(dev)
+        q = torch.randn(L, T, Hq * D, device=dev).to(torch.bfloat16)
+        k = torch.randn(L, T, Hkv, D, device=dev).to(torch.bfloat16)
+        v = torch.randn(L, T, Hkv, D, device=dev).to(torch.bfloat16)
+        qo = torch.empty(T, Hq * D, dtype=torch.bfloat16, device=dev)
+        wplan = kvc.PagedKVWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices, idx.kv_block_indptrs,
+                                     idx.kv_last_block_lens, Hkv, D, shape.block_size, torch.bfloat16)
+        rplan = kvc.PagedRotaryWritePlan(idx.batch_indices, idx.positions, idx.kv_block_indices,
+                                         idx.kv_block_indptrs, idx.kv_last_block_lens, cs, Hq, Hkv, D,
+                                         shape.block_size, resolve_slots=True)
+        for sets in (1, 4, L):
+            def write(i):
+                for l in range(L):
+                    wplan.append(k[l % sets], v[l % sets], pool[l])
+
+            def rotate(i):
+                for l in range(L):
+                    rplan.run(q[l % sets], k[l % sets].view(T, Hkv * D), v[l % sets].view(T, Hkv * D), pool[l],
+                              query_out=qo)
+
+            for fn, knob, values, what in ((write, "write_nt", (1, 3), "PagedKVWritePlan.append"),
+                                           (rotate, "rope_nt", (0, 3), "PagedRotaryWritePlan.run")):
+                us = {val: [] for val in values}
+                for _ in range(2):
+                    for val in values:
+                        _lib.reset_tuning()
+                        _lib.set_tuning(knob, val)
+                        _, ms_e = time_region(fn, 32, 4, torch, graph_of=1)
+                        us[val].append(round(ms_e * 1e3 / L, 3))
+                _lib.reset_tuning()
+                out.append({"name": f"load policy/{label}, {what} per layer, {sets} source set(s)", "knob": knob,
+                            "us_per_layer": {f"{knob}={val}": us[val] for val in values}})
+                log(f"  {out[-1]['name']}: {out[-1]['us_per_layer']}")
+        del pool, q, k, v
+        torch.cuda.empty_cache()
+    return out
