@@ -857,9 +857,28 @@ def bench_decode_step_graph(torch, kvc, wl, s8, pool, L, num_blocks, dev, steps=
         for l in range(L):
             step.append(keys[l], values[l], caches[l])
 
+    # the same step with the rotation of Q and K fused into each layer's write
+    Hq = 32
+    cs = kvc.make_cos_sin_cache(D, 8192, 500000.0, dtype=torch.bfloat16).to(dev)
+    rstep = KVWriteStep(H, D, bs, torch.bfloat16, dev, max_requests=B, max_tokens=B, max_block_ids=cap_ids,
+                        cos_sin_cache=cs, num_heads=Hq)
+    query = torch.randn(B, Hq * D, device=dev).to(torch.bfloat16)
+    q_out = torch.empty_like(query)
+    rstep.set_arrays(*packed[0])
+    rgraph = rstep.capture([k.view(B, H * D) for k in keys], [v.view(B, H * D) for v in values], caches,
+                           queries=[query] * L, query_outs=[q_out] * L)
+
+    def rotary_replay_only(i):
+        rgraph.replay()
+
+    write_bytes_step = bytes_step
+    rotary_bytes_step = L * B * (2 * Hq * D * 2 + 4 * H * D * 2 + 2 * D * 2 + 12)
+
     compact, detail = [], []
     # `us` of these rows is WALL time per 32-layer step (what the serving loop pays)
     for fn, n, form, short, what in (
+            (rotary_replay_only, steps, "step wall, graph, rotation fused", "graph{index+32 rotate+write}",
+             "one hipGraph replay = index build + 32 x (rotation of Q and K + K/V write) in one launch per layer"),
             (replay_only, steps, "step wall, graph", "graph{index+32 writes}",
              "one hipGraph replay = index build + 32 per-layer writes (the step's scalars already uploaded)"),
             (new_step_then_replay, steps, "step wall, new step: pack+upload+graph", "set_arrays+graph",
@@ -872,6 +891,8 @@ def bench_decode_step_graph(torch, kvc, wl, s8, pool, L, num_blocks, dev, steps=
              "host lists+32 append calls",
              "eager: the reference's host list building and six uploads, then 32 full-argument calls")):
         wall_us, dev_us = timed(fn, n)
+        # the fused rows also read and write Q and read the cos/sin rows
+        bytes_step = rotary_bytes_step if fn is rotary_replay_only else write_bytes_step
         detail.append({"name": f"cfg2 decode step ({L} layers, {B} requests): {what}", "wall_us_per_step": round(wall_us, 1),
                        "device_us_per_step": round(dev_us, 1), "bytes_per_step": int(bytes_step),
                        "note": "K/V sources of all steps are one 64 MiB set (per-layer launches of 2 MiB are bound by "
