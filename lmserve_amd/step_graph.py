@@ -184,6 +184,8 @@ class KVWriteStep:
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            # thread-local capture: a KV worker's threads (row mover, notifier) may
+            # query events and enqueue copies on their own streams meanwhile
+            with torch.cuda.graph(graph, capture_error_mode="thread_local"):
                 body()
         return graph

@@ -241,3 +241,69 @@ def test_a_step_beyond_the_capacities_is_refused_before_any_upload(gpu):
     step.build_index()
     torch.cuda.synchronize()
     assert step.slot_mapping.cpu().tolist() == [1 * 4 + 0, 1 * 4 + 1, -1, -1, -1, -1, -1, -1]
+
+
+def test_a_step_is_recorded_while_another_thread_works_on_its_own_stream(gpu):
+    """The recording is thread-local: a second thread (what a KV worker's mover and
+    notifier threads are in a serving process) keeps launching copies, recording
+    and querying events on its own stream while the step is captured; the capture
+    succeeds and its replay is bit-exact."""
+    import threading
+
+    s = wl.LLAMA_3_8B
+    L, nb, bs, B = 4, 256, s.block_size, 32
+    H, D = s.num_kv_heads, s.head_dim
+    rng = np.random.default_rng(21)
+    ids = FifoBlockIds(nb)
+    reqs = []
+    for i in range(B):
+        ctx = int(rng.integers(1, 50))
+        reqs.append(kvc.InferInput(i, [0], 1, ctx, ctx + 1, ids.take((ctx + 1 + bs - 1) // bs)))
+    rs, index, padded = _oracle_index(reqs, bs, B)
+    pool_np = sentinel_pool((L, nb, 2, bs, H, D), 5)
+    dpool = to_bf16(pool_np, gpu)
+    other_pool = torch.zeros(2, 64, 2, bs, H, D, dtype=torch.bfloat16, device=gpu)
+    key, value = bf16_bits((L, B, H, D), 31), bf16_bits((L, B, H, D), 32)
+    dk, dv = to_bf16(key, gpu), to_bf16(value, gpu)
+    step = KVWriteStep(H, D, bs, torch.bfloat16, gpu, max_requests=B, max_tokens=B, max_block_ids=B * 8)
+    step.set_requests(reqs)
+    stop, failures, rounds = threading.Event(), [], [0]
+
+    def busy():
+        try:
+            torch.cuda.set_device(gpu)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                while not stop.is_set():
+                    kvc.copy_blocks(other_pool, {0: [1, 2], 3: [4]})
+                    done = torch.cuda.Event()
+                    done.record(stream)
+                    while not done.query():
+                        pass
+                    rounds[0] += 1
+        except Exception as exc:      # noqa: BLE001 - reported by the assertion below
+            failures.append(repr(exc))
+
+    worker = threading.Thread(target=busy)
+    worker.start()
+    try:
+        while rounds[0] < 3 and worker.is_alive():
+            pass
+        graph = step.capture([dk[l] for l in range(L)], [dv[l] for l in range(L)], [dpool[l] for l in range(L)])
+        before = rounds[0]
+        dpool.copy_(to_bf16(pool_np, gpu))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        while rounds[0] < before + 3 and worker.is_alive():
+            pass
+    finally:
+        stop.set()
+        worker.join(30)
+    assert not failures and not worker.is_alive(), failures
+    want = pool_np.copy()
+    for l in range(L):
+        orc.c_append_paged_kv_cache(key[l], value[l], index[3], index[4], want[l],
+                                    [b for r in rs for b in r.block_ids], index[1])
+    assert np.array_equal(bits_of(dpool), want)
+    _check_index(step, rs, index, padded)
