@@ -182,7 +182,8 @@ def bench_write_through_overlap(torch, kvc, wl, dev, scattered=False):
     for mode, bounce_bytes, always, label in variants:
         handle = kvc.KVWorkerHandle.create(L)
         worker = kvc.KVWorker(pool, num_host_blocks=nhb, swap_mode=mode, kv_worker_handle=handle,
-                              host_bounce_bytes=bounce_bytes, host_bounce_always=always)
+                              host_bounce_bytes=bounce_bytes, host_bounce_always=always,
+                              model_streams=[model_stream, torch.cuda.current_stream()])
         scattered_timing = scattered or always      # measured through the protocol, not through prepared calls
         hooks = kvc.LayerSyncHooks(handle)
 
@@ -351,7 +352,8 @@ def bench_small_write_through(torch, kvc, wl, dev):
                "bytes_per_call": int(n * L * s8.block_bytes)}
         for mode in ("staged", "direct"):
             handle = kvc.KVWorkerHandle.create(L)
-            worker = kvc.KVWorker(pool, num_host_blocks=n, swap_mode=mode, kv_worker_handle=handle)
+            worker = kvc.KVWorker(pool, num_host_blocks=n, swap_mode=mode, kv_worker_handle=handle,
+                                  model_streams=[model_stream, torch.cuda.current_stream()])
             hooks = kvc.LayerSyncHooks(handle)
             try:
                 def timed_forward():

@@ -105,6 +105,25 @@ int kvc_write_runs_layers(const void* key, const void* value,
                           int elem_bytes, void* stream);
 
 /*
+ * Do two streams feed the same hardware queue? The runtime maps every stream of
+ * a process onto a few hardware queues (4 unless GPU_MAX_HW_QUEUES says
+ * otherwise). Kernels of streams that share one run one after the other, and a
+ * wait that one of them queues (a kernel behind a copy-engine transfer, an
+ * event of another stream) holds back the other as well: swap-out and swap-in
+ * issued together then take turns instead of overlapping (55 against 94 GB/s
+ * in sum), and a forward pass beside a write-through takes twice its time.
+ * The call finds out by doing it: stream_x is kept busy for 200 us by a kernel
+ * that watches the clock, an empty kernel is launched on stream_y, and the host
+ * sees which finishes first (up to three rounds; both streams are synchronised
+ * before it returns; about 0.3 ms). *shared = 1 when y's kernel never finished
+ * before x's, 0 otherwise; the same handle twice gives 1 without a launch.
+ * Not under stream capture (KVC_ERR_INVALID_ARG). No counterpart in the
+ * reference, whose two streams (kv_worker.py:159-160) live in a process of
+ * their own; KVWorker uses it to choose its streams.
+ */
+int kvc_streams_share_hw_queue(void* stream_x, void* stream_y, int* shared);
+
+/*
  * Host side of a one-layer swap to or from scattered host blocks, on host threads.
  * Serves
  *   _save_layer_kv_blocks_to_host     (runtime/worker/llm_worker/kv_worker.py:213-227)

@@ -104,6 +104,7 @@ SIGNATURES = {
     "kvc_build_write_index": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P,
                                       _P, _P, _P, _I64, _P]),
     "kvc_slot_runs": (c_int, [_P, c_int, _I64, _I64, _P, _P, _I64, _P]),
+    "kvc_streams_share_hw_queue": (c_int, [_P, _P, _P]),
     "kvc_write_runs_layers": (c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                       _I64, _I64, _I64, _I64, _I64, _I64, c_int, _P]),
     "kvc_write_plan_set_slots": (c_int, [_P, _P]),
@@ -245,6 +246,14 @@ def get_tuning(key: str) -> int:
 
 def reset_tuning() -> None:
     check(lib().kvc_reset_tuning())
+
+
+def streams_share_hw_queue(stream_x: int, stream_y: int) -> bool:
+    """Whether two streams (raw handles) feed the same hardware queue, found out
+    by holding one for 200 us and watching an empty kernel on the other."""
+    out = ctypes.c_int(1)
+    check(lib().kvc_streams_share_hw_queue(stream_x, stream_y, ctypes.byref(out)))
+    return bool(out.value)
 
 
 def last_swap_mode() -> int:

@@ -822,6 +822,19 @@ __global__ __launch_bounds__(kPrepThreads) void slot_runs_kernel(const void* slo
   }
 }
 
+// Two kernels for kvc_streams_share_hw_queue: one keeps its hardware queue busy
+// for `ticks` of the 100 MHz wall clock (one wavefront that sleeps between
+// looks at the clock; `max_iters` bounds the loop whatever the clock reads),
+// the other does nothing.
+__global__ void hold_queue_kernel(uint64_t ticks, uint32_t max_iters) {
+  const uint64_t begin = wall_clock64();
+  for (uint32_t i = 0; i < max_iters; ++i) {
+    if (wall_clock64() - begin >= ticks) break;
+    __builtin_amdgcn_s_sleep(32);
+  }
+}
+__global__ void touch_queue_kernel() {}
+
 // ---------------------------------------------------------------------------
 // host helpers
 // ---------------------------------------------------------------------------
@@ -2079,6 +2092,72 @@ int kvc_build_write_index(const int32_t* input_lens, const int32_t* context_lens
                      kv_last_page_len, batch_indices, positions, slot_mapping, run_indptr, runs,
                      num_runs, max_runs);
   KVC_HIP(hipGetLastError());
+  return KVC_OK;
+}
+
+int kvc_streams_share_hw_queue(void* stream_x, void* stream_y, int* shared) {
+  const char* fn = "kvc_streams_share_hw_queue";
+  if (!shared) return fail(KVC_ERR_INVALID_ARG, "%s: null result pointer", fn);
+  *shared = 1;
+  hipStream_t x = (hipStream_t)stream_x, y = (hipStream_t)stream_y;
+  if (x == y) return KVC_OK;
+  for (hipStream_t s : {x, y}) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    KVC_HIP(hipStreamIsCapturing(s, &capturing));
+    if (capturing != hipStreamCaptureStatusNone)
+      return fail(KVC_ERR_INVALID_ARG, "%s: a stream is being captured", fn);
+  }
+  // first use of a stream creates or attaches its hardware queue: keep that out of the timing
+  hipLaunchKernelGGL(touch_queue_kernel, dim3(1), dim3(64), 0, x);
+  hipLaunchKernelGGL(touch_queue_kernel, dim3(1), dim3(64), 0, y);
+  KVC_HIP(hipGetLastError());
+  KVC_HIP(hipStreamSynchronize(x));
+  KVC_HIP(hipStreamSynchronize(y));
+  hipEvent_t ex = nullptr, ey = nullptr;
+  KVC_HIP(hipEventCreateWithFlags(&ex, hipEventDisableTiming));
+  if (hipEventCreateWithFlags(&ey, hipEventDisableTiming) != hipSuccess) {
+    (void)hipEventDestroy(ex);
+    return fail(KVC_ERR_HIP, "%s: hipEventCreateWithFlags failed", fn);
+  }
+  // x is held for 200 us; y's empty kernel takes about 10 us from launch to done unless
+  // it sits behind x's in the same hardware queue. A host thread that loses the
+  // processor for the whole hold would see both done at once: three rounds, and the
+  // streams count as sharing only if every round says so.
+  int rc = KVC_OK;
+  int blocked_rounds = 0;
+  constexpr int kRounds = 3;
+  for (int round = 0; round < kRounds && rc == KVC_OK; ++round) {
+    hipLaunchKernelGGL(hold_queue_kernel, dim3(1), dim3(64), 0, x, (uint64_t)20000, (uint32_t)4000);
+    hipError_t e = hipEventRecord(ex, x);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(touch_queue_kernel, dim3(1), dim3(64), 0, y);
+      e = hipEventRecord(ey, y);
+    }
+    bool blocked = false;
+    if (e == hipSuccess) {
+      for (;;) {
+        const hipError_t qx = hipEventQuery(ex);   // x first: "y done, x not" proves y was not held up
+        const hipError_t qy = hipEventQuery(ey);
+        if ((qx != hipSuccess && qx != hipErrorNotReady) || (qy != hipSuccess && qy != hipErrorNotReady)) {
+          e = qx != hipSuccess && qx != hipErrorNotReady ? qx : qy;
+          break;
+        }
+        if (qy == hipSuccess) {
+          blocked = qx == hipSuccess;
+          break;
+        }
+      }
+    }
+    const hipError_t sx = hipStreamSynchronize(x), sy = hipStreamSynchronize(y);
+    if (e == hipSuccess) e = sx != hipSuccess ? sx : sy;
+    if (e != hipSuccess) rc = fail(KVC_ERR_HIP, "%s: %s", fn, hipGetErrorString(e));
+    if (!blocked) break;
+    ++blocked_rounds;
+  }
+  (void)hipEventDestroy(ex);
+  (void)hipEventDestroy(ey);
+  if (rc != KVC_OK) return rc;
+  *shared = blocked_rounds == kRounds ? 1 : 0;
   return KVC_OK;
 }
 

@@ -41,7 +41,7 @@ import time
 import warnings
 import weakref
 from dataclasses import dataclass, field
-from typing import Iterable, List, Optional, Sequence, Tuple
+from typing import Callable, Iterable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -143,6 +143,47 @@ def warn_if_few_hardware_queues(environ=os.environ) -> bool:
                   f"{environ.get('GPU_MAX_HW_QUEUES', 'unset (4)')}: copies beside a forward pass may share a "
                   "hardware queue with the model's stream and double its time; export GPU_MAX_HW_QUEUES=8 before "
                   "the process starts, or run the KV worker as its own process", RuntimeWarning, stacklevel=3)
+    return True
+
+
+def pick_streams_apart(count: int, avoid: Sequence, make_stream: Callable, share: Callable,
+                       tries: int = 24) -> Tuple[list, bool]:
+    """`count` streams of which none shares a hardware queue with another or with a
+    stream of `avoid`, drawn with `make_stream()` and tested with
+    `share(a, b) -> bool`. The runtime maps all streams of a process onto a few
+    hardware queues and says nothing about which; streams that share one take
+    turns, and a wait queued by one holds back the other. Returns
+    `(streams, apart)`; after `tries` draws without success the remaining
+    streams are taken as they come and `apart` is False."""
+    chosen: list = []
+    drawn = 0
+    while len(chosen) < count and drawn < tries:
+        s = make_stream()
+        drawn += 1
+        if any(share(s, o) for o in list(avoid) + chosen):
+            continue
+        chosen.append(s)
+    apart = len(chosen) == count
+    while len(chosen) < count:
+        chosen.append(make_stream())
+    return chosen, apart
+
+
+_warned_about_shared_queue = False
+
+
+def warn_streams_share_a_queue(environ=os.environ) -> bool:
+    """One warning per process when a KV worker could not be given streams with
+    hardware queues of their own. Returns whether it warned."""
+    global _warned_about_shared_queue
+    if _warned_about_shared_queue:
+        return False
+    _warned_about_shared_queue = True
+    warnings.warn("KVWorker: no pair of streams with hardware queues of their own was found "
+                  f"(GPU_MAX_HW_QUEUES={environ.get('GPU_MAX_HW_QUEUES', 'unset (4)')}): swap-out and swap-in issued "
+                  "together will take turns (about 55 instead of 94 GB/s in sum) and copies beside a forward pass "
+                  "may hold it back; export GPU_MAX_HW_QUEUES=8 before the process starts",
+                  RuntimeWarning, stacklevel=3)
     return True
 
 
@@ -270,6 +311,13 @@ class KVWorker:
       gives up (`TimeoutError`): the doorbell of the model's next layer, the event
       a queued row copy waits for. `close()` returns within it whatever the other
       side does. None = no limit (the reference's behaviour).
+    model_streams: the stream(s) the model's forward pass runs on, when that is not
+      the stream that is current where the worker is made. The worker takes two
+      streams that share a hardware queue neither with each other nor with these
+      (`kvc_streams_share_hw_queue`; about 1 ms at construction). Whether it
+      found them is `streams_have_own_queues`; if not it warns once: with the
+      runtime's default of 4 hardware queues a process that already runs many
+      streams may have none left, `GPU_MAX_HW_QUEUES=8` helps.
     validate: check on the host that no block is the destination of two pairs of
       one GPU<->Host call (`ValueError`). The reference copies the pairs one
       after the other, so the later pair wins there (kv_worker.py:197-227);
@@ -295,6 +343,7 @@ class KVWorker:
         host_bounce_regions: int = 4,
         host_bounce_always: bool = False,
         host_wait_timeout: Optional[float] = 30.0,
+        model_streams: Optional[Sequence[torch.cuda.Stream]] = None,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -346,13 +395,23 @@ class KVWorker:
             self.disk_tier = None
             self.disk_kv_caches = None
 
+        # Two streams as in the reference (kv_worker.py:159-160), chosen so that they share
+        # a hardware queue neither with each other nor with the stream(s) the model runs
+        # on (by default the stream that is current here): every swap call starts by
+        # waiting for the caller's current stream, and a wait in a shared queue holds
+        # back the other direction and the model's kernels as well.
         with torch.cuda.device(self.device):
-            self.dtoh_stream = torch.cuda.Stream()
-            self.htod_stream = torch.cuda.Stream()
+            if model_streams is None:
+                model_streams = [torch.cuda.current_stream(self.device)]
+            (self.dtoh_stream, self.htod_stream), self.streams_have_own_queues = pick_streams_apart(
+                2, list(model_streams), torch.cuda.Stream,
+                lambda a, b: _lib.streams_share_hw_queue(a.cuda_stream, b.cuda_stream))
         self._staging = {}   # (direction, stream handle) -> [workspace, weak reference to its PreparedSwap]
         self.kv_worker_handle = kv_worker_handle
-        if kv_worker_handle is not None:
-            warn_if_few_hardware_queues()
+        if not self.streams_have_own_queues:
+            warn_streams_share_a_queue()
+            if kv_worker_handle is not None:
+                warn_if_few_hardware_queues()
 
         self.COPY_KV_OP_MAP = {
             (Device.GPU, Device.Host): self._copy_kv_gpu_to_host,

@@ -545,3 +545,13 @@ def test_swap_mode_can_be_asked_before_the_call():
     assert L.kvc_swap_resolve_mode(None, 64, 1, 64 << 10, big) == _lib.KVC_SWAP_DIRECT
     assert L.kvc_swap_resolve_mode(consecutive.ctypes.data, -1, 1, 64 << 10, big) == _lib.KVC_ERR_INVALID_ARG
     assert L.kvc_swap_last_mode() in (-1, _lib.KVC_SWAP_STAGED, _lib.KVC_SWAP_DIRECT)
+
+
+def test_queue_sharing_query_without_a_launch():
+    """The same stream twice shares its queue with itself: answered without
+    touching the GPU; a null result pointer is refused."""
+    L = _lib.lib()
+    out = ctypes.c_int(0)
+    assert L.kvc_streams_share_hw_queue(None, None, ctypes.byref(out)) == _lib.KVC_OK and out.value == 1
+    assert L.kvc_streams_share_hw_queue(None, None, None) == _lib.KVC_ERR_INVALID_ARG
+    assert _lib.streams_share_hw_queue(0, 0) is True

@@ -402,6 +402,45 @@ def test_few_hardware_queues_are_warned_about_once():
     kv_worker._warned_about_queues = False
 
 
+def test_streams_are_picked_apart_by_hardware_queue():
+    """Stand-in streams are integers and their queue is the integer modulo the
+    number of queues, which is what the picker cannot see and has to find out."""
+    import warnings
+    from lmserve_amd import kv_worker
+
+    def world(queues, first=0):
+        counter = [first]
+
+        def make():
+            counter[0] += 1
+            return counter[0]
+        return make, (lambda a, b: a % queues == b % queues), counter
+
+    # 4 queues, the model on stream 1: 2 shares nothing, 3 shares nothing, done after two draws
+    make, share, counter = world(4, first=1)
+    got, apart = kv_worker.pick_streams_apart(2, [1], make, share)
+    assert (got, apart) == ([2, 3], True) and counter[0] == 3
+    # the model's queue and the first pick's queue are skipped
+    make, share, counter = world(4, first=4)
+    got, apart = kv_worker.pick_streams_apart(2, [5, 2], make, share)      # queues 1 and 2 are taken
+    assert apart and [g % 4 for g in got] == [3, 0] and got == [7, 8]
+    # two queues, one of them the model's: one stream fits, the second cannot; the picker gives up and says so
+    make, share, counter = world(2)
+    got, apart = kv_worker.pick_streams_apart(2, [0], make, share, tries=10)
+    assert not apart and len(got) == 2 and got[0] % 2 == 1 and counter[0] == 11
+    # nothing to avoid, one queue
+    make, share, _ = world(1)
+    got, apart = kv_worker.pick_streams_apart(2, [], make, share, tries=5)
+    assert not apart and len(got) == 2
+    kv_worker._warned_about_shared_queue = False
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        assert kv_worker.warn_streams_share_a_queue({"GPU_MAX_HW_QUEUES": "2"}) is True
+        assert kv_worker.warn_streams_share_a_queue({}) is False
+    assert len(caught) == 1 and "GPU_MAX_HW_QUEUES=2" in str(caught[0].message)
+    kv_worker._warned_about_shared_queue = False
+
+
 def test_pool_in_a_segment_of_two_gib_or_more_is_not_exported():
     """The IPC handle of a tensor covers its whole allocator segment; segments of
     2 GiB or more must never be shared between processes here."""
