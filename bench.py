@@ -22,7 +22,7 @@ the details file (`--details`, default bench_out/bench_details.json) and to
 stderr, never to stdout.
 
 Sections beyond the operations the benchmark names are opt-in
-(`--ops ...,rope,shard,index,overlap,twoproc,disk,sweep,calib,translation,loads`) and
+(`--ops ...,rope,shard,index,overlap,twoproc,disk,sweep,calib,translation,loads,duplex`) and
 live in bench_sections.py.
 """
 from __future__ import annotations
@@ -70,7 +70,7 @@ def parse_args(argv=None):
                    help="comma list of sections beside the headline. Default: write (per-layer / page-table "
                         "forms of config 2), prefill (config 3), copy (config 4), swap (config 5), step (a whole "
                         "decode step, index build included, replayed from one hipGraph). Opt-in: rope, shard, "
-                        "index, overlap, twoproc, disk, sweep, calib, translation, loads. 'none' = headline only")
+                        "index, overlap, twoproc, disk, sweep, calib, translation, loads, duplex. 'none' = headline only")
     p.add_argument("--details", default=None,
                    help="file for every row beyond the final line (default bench_out/bench_details.json; "
                         "'-' = stderr only)")
@@ -615,6 +615,10 @@ def main(argv=None):
         with optional_section("load policy rows", torch):
             from bench_sections import bench_load_policy
             details += bench_load_policy(torch, kvc, wl, dev)
+    if "duplex" in ops:
+        with optional_section("both swap directions by stream choice", torch):
+            from bench_sections import bench_duplex_streams
+            details += bench_duplex_streams(torch, kvc, wl, dev)
     if "overlap" in ops:
         with optional_section("write-through overlap", torch):
             from bench_sections import bench_small_write_through, bench_write_through_overlap

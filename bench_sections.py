@@ -959,3 +959,67 @@ def bench_load_policy(torch, kvc, wl, dev):
         del pool, q, k, v
         torch.cuda.empty_cache()
     return out
+
+
+def bench_duplex_streams(torch, kvc, wl, dev, workers=6):
+    """Swap-out beside swap-in for KV workers made one after another once a
+    recorded step graph has run, with the two streams taken as they come and
+    with streams chosen apart by hardware queue; for each worker, which of its
+    streams share a queue (with each other, with the current stream) and the
+    rate of each direction alone and of both together."""
+    from lmserve_amd import _lib
+    from lmserve_amd.step_graph import KVWriteStep
+
+    s8, s70 = wl.LLAMA_3_8B, wl.LLAMA_3_1_70B
+    L8, B, nb8 = 8, 256, 2048
+    pool8 = torch.empty(L8, nb8, 2, 16, 8, 128, dtype=torch.bfloat16, device=dev)
+    w = wl.decode_step(s8, num_blocks=nb8, batch=B, max_context=200, seed=1)
+    step = KVWriteStep(8, 128, 16, torch.bfloat16, dev, max_requests=B, max_tokens=B, max_block_ids=B * 16)
+    step.set_requests(w.inputs)
+    k = torch.zeros(L8, B, 8, 128, dtype=torch.bfloat16, device=dev)
+    graph = step.capture([k[l] for l in range(L8)], [k[l] for l in range(L8)], [pool8[l] for l in range(L8)])
+    for _ in range(50):
+        graph.replay()
+    torch.cuda.synchronize()
+    nb, n = 4096, 2048                                   # 5 GiB each way
+    pool = torch.empty(s70.num_layers, nb, 2, 16, 8, 128, dtype=torch.bfloat16, device=dev)
+    old, _, new = wl.swap_round_trip(nb, n, seed=0)
+    out_maps = [kvc.BlockMapping.from_pairs(zip(old[:n // 2].tolist(), range(n // 2)))]
+    in_maps = [kvc.BlockMapping.from_pairs(zip(range(n // 2, n), new[n // 2:].tolist()))]
+    half = n // 2 * s70.num_layers * s70.block_bytes
+    cur = torch.cuda.current_stream()
+    rows = []
+    for own in (False, True):
+        for number in range(1, workers + 1):
+            worker = kvc.KVWorker(pool, n, swap_mode="staged", own_queues=own)
+            a, b = worker.dtoh_stream, worker.htod_stream
+            try:
+                shares = {"out/in": _lib.streams_share_hw_queue(a.cuda_stream, b.cuda_stream),
+                          "current/out": _lib.streams_share_hw_queue(cur.cuda_stream, a.cuda_stream),
+                          "current/in": _lib.streams_share_hw_queue(cur.cuda_stream, b.cuda_stream)}
+
+                def run(do_out, do_in):
+                    if do_out:
+                        worker.save_kv_blocks_to_host_nowait(out_maps)
+                    if do_in:
+                        worker.load_kv_blocks_from_host_nowait(in_maps)
+                    a.synchronize()
+                    b.synchronize()
+
+                rates = {}
+                for label, do_out, do_in in (("out", True, False), ("in", False, True), ("both", True, True)):
+                    run(do_out, do_in)
+                    ts = []
+                    for _ in range(3):
+                        torch.cuda.synchronize()
+                        t0 = time.perf_counter()
+                        run(do_out, do_in)
+                        ts.append(time.perf_counter() - t0)
+                    rates[label] = round(half * (int(do_out) + int(do_in)) / sorted(ts)[1] / 1e9, 1)
+            finally:
+                worker.close()
+            rows.append({"name": f"duplex/worker {number} after a recorded step ran, streams "
+                                 f"{'chosen apart by hardware queue' if own else 'as they come'}",
+                         "share_a_queue": shares, "pcie_gbps": rates})
+            log(f"  {rows[-1]['name']}: share {shares}; GB/s {rates}")
+    return rows

@@ -318,6 +318,8 @@ class KVWorker:
       found them is `streams_have_own_queues`; if not it warns once: with the
       runtime's default of 4 hardware queues a process that already runs many
       streams may have none left, `GPU_MAX_HW_QUEUES=8` helps.
+    own_queues: False takes the two streams as torch hands them out, as the
+      reference does, without looking at their queues (for measurements).
     validate: check on the host that no block is the destination of two pairs of
       one GPU<->Host call (`ValueError`). The reference copies the pairs one
       after the other, so the later pair wins there (kv_worker.py:197-227);
@@ -344,6 +346,7 @@ class KVWorker:
         host_bounce_always: bool = False,
         host_wait_timeout: Optional[float] = 30.0,
         model_streams: Optional[Sequence[torch.cuda.Stream]] = None,
+        own_queues: bool = True,
     ):
         if not gpu_kv_caches.is_cuda:
             raise ValueError("gpu_kv_caches must live on the GPU")
@@ -403,9 +406,13 @@ class KVWorker:
         with torch.cuda.device(self.device):
             if model_streams is None:
                 model_streams = [torch.cuda.current_stream(self.device)]
-            (self.dtoh_stream, self.htod_stream), self.streams_have_own_queues = pick_streams_apart(
-                2, list(model_streams), torch.cuda.Stream,
-                lambda a, b: _lib.streams_share_hw_queue(a.cuda_stream, b.cuda_stream))
+            if own_queues:
+                (self.dtoh_stream, self.htod_stream), self.streams_have_own_queues = pick_streams_apart(
+                    2, list(model_streams), torch.cuda.Stream,
+                    lambda a, b: _lib.streams_share_hw_queue(a.cuda_stream, b.cuda_stream))
+            else:
+                self.dtoh_stream, self.htod_stream = torch.cuda.Stream(), torch.cuda.Stream()
+                self.streams_have_own_queues = True    # not looked at: nothing to warn about
         self._staging = {}   # (direction, stream handle) -> [workspace, weak reference to its PreparedSwap]
         self.kv_worker_handle = kv_worker_handle
         if not self.streams_have_own_queues:
