@@ -117,6 +117,8 @@ int kvc_write_runs_layers(const void* key, const void* value,
  * sees which finishes first (up to three rounds; both streams are synchronised
  * before it returns; about 0.3 ms). *shared = 1 when y's kernel never finished
  * before x's, 0 otherwise; the same handle twice gives 1 without a launch.
+ * Ask while both streams are idle: work already queued on stream_y delays its
+ * empty kernel as a shared queue would (the answer then errs towards 1).
  * Not under stream capture (KVC_ERR_INVALID_ARG). No counterpart in the
  * reference, whose two streams (kv_worker.py:159-160) live in a process of
  * their own; KVWorker uses it to choose its streams.
