@@ -41,6 +41,7 @@ extern "C" {
  *   "rope_threads"                    lanes per workgroup in the rotation kernel (0 = default, 64, 128, 256)
  *   "rope_nt"                         non-temporal loads in that kernel: bit 0 the K and V rows, bit 1 the Q rows
  *   "disk_bounce_mib"                 MiB of aligned staging per thread in the disk tier
+ *   "host_rows_nt"                    row copies on host threads: 1 = stores that go past the cache (default)
  * Unknown key: KVC_ERR_INVALID_ARG. kvc_reset_tuning puts every knob back to its
  * default; kvc_tuning_modified counts the knobs that are not at their default. */
 int kvc_set_tuning(const char* key, int value);

@@ -44,6 +44,9 @@ int launch_resolve_slots(const char* fn, const int32_t* batch_indices, const int
 // MiB of aligned staging per thread in the disk tier ("disk_bounce_mib").
 extern int g_disk_bounce_mib;
 
+// Row copies on host threads ("host_rows_nt"): 1 = stores that go past the cache.
+extern int g_host_rows_nt;
+
 }  // namespace kvc
 
 #define KVC_HIP(call)                                                          \

@@ -8,10 +8,12 @@
 // holds back the kernels of every other stream while it runs. Here the PCIe leg
 // of a layer is ONE copy between the GPU and a dense pinned buffer, and the rows
 // go between that buffer and their places in the pool on a few host threads
-// (one thread moves about 23 GB/s of 64 KiB rows, four match the link).
+// (into the pool one thread moves about 50 GB/s of 64 KiB rows and four 130-150,
+// into the dense buffer 26 and 77; the link carries 55).
 //
 // No GPU work in this file.
 
+#include <emmintrin.h>
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -32,6 +34,7 @@
 
 namespace kvc {
 int fail(int code, const char* fmt, ...);
+int g_host_rows_nt = 1;
 }
 
 namespace {
@@ -63,28 +66,58 @@ int check_rows(const char* fn, const void* host_pool, int64_t num_host_blocks, i
   return KVC_OK;
 }
 
-// the rows of one call on `threads` host threads (this thread is one of them); false = out of memory
-bool copy_rows(const RowCopy& c, int threads) {
-  // rows are handed out in runs of 8 so that a thread stays on neighbouring dense rows
-  constexpr int64_t kRun = 8;
-  std::atomic<int64_t> next{0};
-  const auto work = [&]() {
-    for (;;) {
-      const int64_t first = next.fetch_add(kRun, std::memory_order_relaxed);
-      if (first >= c.n) return;
-      const int64_t last = std::min(c.n, first + kRun);
-      for (int64_t i = first; i < last; ++i) {
-        char* p = c.pool + c.host_ids[i] * c.pool_block_bytes;
-        char* d = c.dense + i * c.row_bytes;
-        if (c.to_pool) std::memcpy(p, d, (size_t)c.row_bytes);
-        else std::memcpy(d, p, (size_t)c.row_bytes);
-      }
+// One row. A row is written once and read next by a copy engine, a disk write
+// or another process, never by this thread: when both ends are 64-byte aligned the
+// stores go past the cache (16-byte non-temporal stores, a cache line at a time),
+// which saves the read of the destination line a cached store starts with.
+inline void copy_row(char* dst, const char* src, int64_t bytes, bool stream) {
+  if (!stream || (((uintptr_t)dst | (uintptr_t)src | (uint64_t)bytes) & 63u) != 0) {
+    std::memcpy(dst, src, (size_t)bytes);
+    return;
+  }
+  const __m128i* s = reinterpret_cast<const __m128i*>(src);
+  __m128i* d = reinterpret_cast<__m128i*>(dst);
+  for (int64_t i = 0; i < bytes / 16; i += 4) {
+    const __m128i a = _mm_load_si128(s + i), b = _mm_load_si128(s + i + 1);
+    const __m128i c = _mm_load_si128(s + i + 2), e = _mm_load_si128(s + i + 3);
+    _mm_stream_si128(d + i, a);
+    _mm_stream_si128(d + i + 1, b);
+    _mm_stream_si128(d + i + 2, c);
+    _mm_stream_si128(d + i + 3, e);
+  }
+}
+
+// Rows are handed out in runs of 8 so that a thread stays on neighbouring dense rows.
+constexpr int64_t kRun = 8;
+inline void copy_rows_share(const RowCopy& c, std::atomic<int64_t>& next, bool stream) {
+  for (;;) {
+    const int64_t first = next.fetch_add(kRun, std::memory_order_relaxed);
+    if (first >= c.n) break;
+    const int64_t last = std::min(c.n, first + kRun);
+    for (int64_t i = first; i < last; ++i) {
+      char* p = c.pool + c.host_ids[i] * c.pool_block_bytes;
+      char* d = c.dense + i * c.row_bytes;
+      if (c.to_pool) copy_row(p, d, c.row_bytes, stream);
+      else copy_row(d, p, c.row_bytes, stream);
     }
-  };
-  // a thread per MiB at most: small calls are not worth starting threads for
+  }
+  // non-temporal stores are ordered by nothing else before the rows are handed on
+  if (stream) _mm_sfence();
+}
+
+// threads worth starting for a call: one per MiB at most, one per run of rows at most
+inline int64_t useful_threads(const RowCopy& c, int threads) {
   int64_t nthreads = threads > 0 ? threads : 4;
   nthreads = std::min<int64_t>(nthreads, std::max<int64_t>(1, c.n * c.row_bytes >> 20));
-  nthreads = std::min<int64_t>(nthreads, (c.n + kRun - 1) / kRun);
+  return std::min<int64_t>(nthreads, std::max<int64_t>(1, (c.n + kRun - 1) / kRun));
+}
+
+// the rows of one call on `threads` host threads (this thread is one of them); false = out of memory
+bool copy_rows(const RowCopy& c, int threads) {
+  std::atomic<int64_t> next{0};
+  const bool stream = kvc::g_host_rows_nt != 0;
+  const auto work = [&]() { copy_rows_share(c, next, stream); };
+  const int64_t nthreads = useful_threads(c, threads);
   if (nthreads <= 1) {
     work();
     return true;
@@ -134,6 +167,83 @@ struct kvc_row_mover {
   std::atomic<bool> cancel{false};
   int64_t skip_below = 0;
   std::thread dispatcher;
+
+  // Helper threads that live as long as the mover (a job of one layer lasts a few
+  // hundred microseconds: starting threads for each would cost a fifth of that).
+  // The dispatcher publishes a job under `team_mu`, takes a share of the rows
+  // itself and waits until the helpers it asked for have finished theirs.
+  std::mutex team_mu;
+  std::condition_variable team_start, team_finished;
+  std::vector<std::thread> helpers;
+  const RowCopy* team_job = nullptr;
+  std::atomic<int64_t> team_next{0};
+  bool team_stream = false;
+  uint64_t team_generation = 0;
+  int team_wanted = 0, team_running = 0;
+  bool team_stop = false;
+
+  void helper_main(int index) {
+    uint64_t seen = 0;
+    for (;;) {
+      const RowCopy* job;
+      bool stream;
+      {
+        std::unique_lock<std::mutex> lock(team_mu);
+        team_start.wait(lock, [&] { return team_stop || team_generation != seen; });
+        if (team_stop) return;
+        seen = team_generation;
+        if (index >= team_wanted) continue;   // a small job: not every helper is asked
+        job = team_job;
+        stream = team_stream;
+      }
+      copy_rows_share(*job, team_next, stream);
+      {
+        std::lock_guard<std::mutex> lock(team_mu);
+        --team_running;
+      }
+      team_finished.notify_one();
+    }
+  }
+
+  void start_helpers() {
+    try {
+      for (int i = 0; i + 1 < threads; ++i) helpers.emplace_back([this, i] { helper_main(i); });
+    } catch (...) {
+      // fewer helpers than asked for: the jobs run on those that started
+    }
+  }
+
+  void stop_helpers() {
+    {
+      std::lock_guard<std::mutex> lock(team_mu);
+      team_stop = true;
+    }
+    team_start.notify_all();
+    for (auto& t : helpers) t.join();
+    helpers.clear();
+  }
+
+  // the rows of one job on the dispatcher and as many helpers as the job is worth
+  void team_copy(const RowCopy& c) {
+    const bool stream = kvc::g_host_rows_nt != 0;
+    const int wanted = (int)std::min<int64_t>(useful_threads(c, threads) - 1, (int64_t)helpers.size());
+    team_next.store(0, std::memory_order_relaxed);
+    if (wanted > 0) {
+      {
+        std::lock_guard<std::mutex> lock(team_mu);
+        team_job = &c;
+        team_stream = stream;
+        team_wanted = team_running = wanted;
+        ++team_generation;
+      }
+      team_start.notify_all();
+    }
+    copy_rows_share(c, team_next, stream);
+    if (wanted > 0) {
+      std::unique_lock<std::mutex> lock(team_mu);
+      team_finished.wait(lock, [&] { return team_running == 0; });
+    }
+  }
 
   // KVC_OK once the job's condition holds; the caller's thread sleeps in 20 us steps
   // (hipEventSynchronize would spin on a core for an event made without the
@@ -202,10 +312,7 @@ struct kvc_row_mover {
       }
       if (rc == KVC_OK) {
         job.copy.host_ids = job.ids.data();
-        if (!copy_rows(job.copy, threads)) {
-          rc = KVC_ERR_HIP;
-          std::snprintf(text, sizeof text, "kvc_row_mover: out of host memory");
-        }
+        team_copy(job.copy);
       }
       {
         std::lock_guard<std::mutex> lock(mu);
@@ -229,9 +336,11 @@ int kvc_row_mover_create(int threads, kvc_row_mover** out) {
   kvc_row_mover* m = new (std::nothrow) kvc_row_mover;
   if (!m) return fail(KVC_ERR_HIP, "kvc_row_mover_create: out of host memory");
   m->threads = threads > 0 ? threads : 4;
+  m->start_helpers();
   try {
     m->dispatcher = std::thread([m] { m->run(); });
   } catch (...) {
+    m->stop_helpers();
     delete m;
     return fail(KVC_ERR_HIP, "kvc_row_mover_create: cannot start a thread");
   }
@@ -335,6 +444,7 @@ int kvc_row_mover_destroy(kvc_row_mover* mover) {
   }
   mover->has_jobs.notify_all();
   if (mover->dispatcher.joinable()) mover->dispatcher.join();   // after the jobs still queued
+  mover->stop_helpers();
   delete mover;
   return KVC_OK;
 }

@@ -138,6 +138,7 @@ Knob* knobs(int* count) {
       {"rope_threads", &kvc::g_rope_tune.threads, 0},
       {"rope_nt", &kvc::g_rope_tune.nt, 0},
       {"disk_bounce_mib", &kvc::g_disk_bounce_mib, 4},
+      {"host_rows_nt", &kvc::g_host_rows_nt, 1},
   };
   *count = (int)(sizeof(table) / sizeof(table[0]));
   return table;
