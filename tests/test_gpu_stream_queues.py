@@ -10,6 +10,7 @@ with what the process has done before (a recorded graph shifts it), so the
 worker finds out at construction (`kvc_streams_share_hw_queue`) and draws
 streams until two are apart from each other and from the model's stream.
 """
+import os
 import time
 
 import numpy as np
@@ -23,6 +24,8 @@ from lmserve_amd.step_graph import KVWriteStep
 
 pytestmark = pytest.mark.gpu
 
+HW_QUEUES = int(os.environ.get("GPU_MAX_HW_QUEUES", "4") or 4)      # the runtime's default is 4
+
 
 def test_a_stream_shares_its_queue_with_itself_and_the_answer_is_stable(gpu):
     a, b = torch.cuda.Stream(), torch.cuda.Stream()
@@ -34,7 +37,10 @@ def test_a_stream_shares_its_queue_with_itself_and_the_answer_is_stable(gpu):
     # among the streams torch hands out, some pair shares a queue (there are more streams than queues)
     streams = [torch.cuda.Stream() for _ in range(12)]
     shares = [_lib.streams_share_hw_queue(streams[0].cuda_stream, s.cuda_stream) for s in streams[1:]]
-    assert any(shares) and not all(shares)
+    if HW_QUEUES < 12:
+        assert any(shares)
+    if HW_QUEUES > 1:
+        assert not all(shares)
     # not while a stream is being captured
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g, stream=a):
@@ -48,6 +54,8 @@ def test_both_swap_directions_overlap_for_every_worker_made_after_a_graph_ran(gp
     state in which a worker's streams used to land in one queue every other
     time): each has streams apart from each other and from the current stream,
     and swap-out beside swap-in takes clearly less than the two in turn."""
+    if HW_QUEUES < 3:
+        pytest.skip("needs three hardware queues: the caller's and one per direction")
     s8 = wl.LLAMA_3_8B
     L8, B, nb8 = 4, 64, 512
     pool8 = torch.zeros(L8, nb8, 2, 16, 8, 128, dtype=torch.bfloat16, device=gpu)
