@@ -58,3 +58,20 @@ def test_default_sections_are_the_benchmarks_operations():
     args = bench.parse_args([])
     assert args.gpus == 1 and set(args.ops.split(",")) == {"write", "prefill", "copy", "swap", "step"}
     assert args.hw_queues == 0 and args.settle_seconds == 0.0
+
+
+def test_every_section_module_imports_without_a_gpu():
+    """The opt-in sections are imported lazily on the GPU box; a mistake in them must
+    show here first. Every section the parser advertises has its function."""
+    import bench
+    import bench_sections
+    import bench_util
+    for name in ("bench_size_sweep", "bench_disk_tier", "bench_write_through_overlap", "bench_small_write_through",
+                 "bench_two_process_swap", "bench_rope_decode", "bench_rope_prefill", "bench_index_prep",
+                 "bench_calibration", "bench_slot_patterns", "bench_tp_shard", "bench_decode_step_graph",
+                 "bench_load_policy", "bench_duplex_streams"):
+        assert callable(getattr(bench_sections, name)), name
+    assert callable(bench_util.time_region) and callable(bench.main)
+    help_text = bench.parse_args(["--ops", "none"]) and bench.__doc__
+    for op in ("rope", "shard", "index", "overlap", "twoproc", "disk", "sweep", "calib", "translation", "loads", "duplex"):
+        assert op in help_text, op
