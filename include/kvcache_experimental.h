@@ -22,6 +22,7 @@ extern "C" {
  *   "copy_order"                      1 = walk all blocks of a layer before the next layer
  *   "copy_max_wgs"                    grid cap of the tile kernel (0 = one workgroup per chunk)
  *   "direct_max_wgs"                  grid cap of the direct swap kernel
+ *   "direct_max_wgs_in"               the same for Host->GPU (0 = direct_max_wgs)
  *   "write_vpt"                       vectors per lane in the write kernel (0 = by size, 1, 2, 4, 8)
  *   "write_threads"                   lanes per workgroup in the write kernel (0 = by size, 64, 128, 256)
  *   "write_nt"                        bit 0: non-temporal stores, bit 1: non-temporal loads (applied to rows

@@ -93,6 +93,14 @@ struct Tuning {
                             // with 48-64 workgroups (more cost a 16 MiB one-layer launch 2-4 %),
                             // both directions at once want 96 or more each (91-92 against 87 GB/s
                             // in sum); the rest of the GPU stays free for the model
+  int direct_max_wgs_in = 16;  // the same cap for Host->GPU (0 = direct_max_wgs). Reads over PCIe hold back
+                               // the kernels of other streams in proportion to what is in flight: 16
+                               // workgroups keep the link rate (57.1 against 57.3 GB/s) and let a forward
+                               // pass that waits for each fetched layer through after 22.8 ms instead of
+                               // 31.5 (13.8 alone, fetch alone 19.5); 8-12 are through after 22.1-22.3 but
+                               // lose the rate on large calls (36-52 GB/s). The price: beside a direct
+                               // swap-out the fetch gets less of the link (54 against 91 GB/s in sum).
+                               // Stores over PCIe hold others back whatever the cap (4 workgroups: +110 %)
   int runs_unroll = 0;       // write_runs: 16-byte vectors per lane (1, 2, 4), 0 = by size
   int runs_order = 1;        // write_runs: 1 = all runs of a plane are neighbours in the grid, 0 = all planes of a run
   int runs_nt = 1;           // write_runs: non-temporal loads and stores
@@ -131,6 +139,7 @@ Knob* knobs(int* count) {
       {"write_planes_threads", &g_tune.write_planes_threads, 0},
       {"write_pipe", &g_tune.write_pipe, -1},
       {"direct_max_wgs", &g_tune.direct_max_wgs, 96},
+      {"direct_max_wgs_in", &g_tune.direct_max_wgs_in, 16},
       {"auto_min_extent_bytes", &g_tune.auto_min_extent_bytes, 1 << 20},
       {"runs_unroll", &g_tune.runs_unroll, 0},
       {"runs_order", &g_tune.runs_order, 1},
@@ -143,6 +152,11 @@ Knob* knobs(int* count) {
   *count = (int)(sizeof(table) / sizeof(table[0]));
   return table;
 }
+// grid cap of the direct swap kernel for one direction
+inline int direct_wgs(bool to_host) {
+  return (!to_host && g_tune.direct_max_wgs_in > 0) ? g_tune.direct_max_wgs_in : g_tune.direct_max_wgs;
+}
+
 Knob* find_knob(const char* key) {
   int n = 0;
   Knob* t = knobs(&n);
@@ -1668,7 +1682,7 @@ int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_
   if (mode == KVC_SWAP_DIRECT && prepared) {
     // nothing but the launch: no events, no upload
     const TileArgs t = direct_swap_tiles(out, pool, host_pool, d_gpu_ids, d_host_ids, g);
-    return launch_tiles(t, g.n, g_tune.direct_max_wgs, ks);
+    return launch_tiles(t, g.n, direct_wgs(out), ks);
   }
   rc = swap_ctx_prepare();
   if (rc != KVC_OK) return rc;
@@ -1684,7 +1698,7 @@ int run_swap(const char* fn, bool out, char* pool, char* host_pool, const int64_
   if (mode == KVC_SWAP_DIRECT) {
     // pool <-> mapped host pool in a single kernel
     const TileArgs t = direct_swap_tiles(out, pool, host_pool, d_gpu_ids, d_host_ids, g);
-    return launch_tiles(t, g.n, g_tune.direct_max_wgs, ks);
+    return launch_tiles(t, g.n, direct_wgs(out), ks);
   }
 
   TileArgs t{};
@@ -2429,7 +2443,7 @@ int kvc_swap_noalloc(int to_host, void* pool, void* host_pool, const int64_t* gp
   const SwapGeom g{n, num_layers, layer_stride_bytes, block_bytes, num_gpu_blocks, num_host_blocks,
                    layer_begin, layer_end};
   const TileArgs t = direct_swap_tiles(to_host != 0, (char*)pool, (char*)host_pool, ids, ids + n, g);
-  return launch_tiles(t, n, g_tune.direct_max_wgs, s);
+  return launch_tiles(t, n, direct_wgs(to_host != 0), s);
 }
 
 void* kvc_host_alloc_pinned(size_t bytes) {

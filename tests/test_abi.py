@@ -175,7 +175,7 @@ def test_tuning_knobs_read_back_and_reset():
                 "write_vpt": 0, "write_nt": 3, "write_order": 0, "write_threads": 0, "write_planes": 1,
                 "write_planes_vpt": 0, "write_planes_min_bytes": 256 << 10, "write_planes_max_vpr": 256, "write_planes_threads": 0,
                 "write_pipe": -1, "direct_max_wgs": 96, "auto_min_extent_bytes": 1 << 20, "rope_threads": 0, "disk_bounce_mib": 4,
-                "runs_unroll": 0, "runs_order": 1, "runs_nt": 1, "rope_nt": 0, "host_rows_nt": 1}
+                "runs_unroll": 0, "runs_order": 1, "runs_nt": 1, "rope_nt": 0, "host_rows_nt": 1, "direct_max_wgs_in": 16}
     for key, value in defaults.items():
         assert _lib.get_tuning(key) == value, key
     for i, key in enumerate(defaults):
