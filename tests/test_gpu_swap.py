@@ -8,6 +8,7 @@ import torch
 
 import lmserve_amd as kvc
 import workloads as wl
+from lmserve_amd import _lib
 from oracle import kvc_oracle as orc
 from tests.helpers import bits_of, random_pool, sentinel_pool, to_bf16
 
@@ -57,6 +58,38 @@ def test_swap_out_then_in_matches_oracle(gpu, mode, chunk):
         assert np.array_equal(w.host_kv_caches, host_np)                    # host untouched
         # round trip: payload of the old blocks now sits in the new blocks
         assert np.array_equal(gpu_np[:, new], pool.reshape(L, nb, -1)[:, old])
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("cap_out,cap_in", [(1, 1), (3, 2), (96, 16), (96, 0), (4096, 4096)])
+def test_direct_swap_under_every_grid_cap(gpu, cap_out, cap_in):
+    """The direct kernel walks its chunks grid-stride under a cap per direction
+    (`direct_max_wgs`, `direct_max_wgs_in`; 0 = the other's): one workgroup, a
+    few, the defaults and more workgroups than chunks all move the same bytes."""
+    s = wl.LLAMA_3_8B
+    L, nb, nhb, n = 3, 48, 40, 29
+    block_shape = (2, s.block_size, s.num_kv_heads, s.head_dim)
+    pool, dpool, w = _worker(gpu, L, nb, block_shape, nhb, "direct", 0, seed=31)
+    try:
+        _lib.set_tuning("direct_max_wgs", cap_out)
+        _lib.set_tuning("direct_max_wgs_in", cap_in)
+        rng = np.random.default_rng(32)
+        perm = rng.permutation(nb)
+        old, new = perm[:n].astype(np.int64), perm[n:n + 19].astype(np.int64)
+        host_ids = rng.permutation(nhb)[:n].astype(np.int64)
+        gpu_np = pool.reshape(L, nb, -1).copy()
+        host_np = w.host_kv_caches.copy()
+        orc.c_save_blocks_to_host(gpu_np, host_np, old, host_ids)
+        w.copy_kv_sync(_mappings(old, host_ids), kvc.Device.GPU, kvc.Device.Host)
+        assert _lib.last_swap_mode() == _lib.KVC_SWAP_DIRECT
+        assert np.array_equal(w.host_kv_caches, host_np)
+        orc.c_load_blocks_from_host(gpu_np, host_np, host_ids[:19], new)
+        w.copy_kv_sync(_mappings(host_ids[:19], new), kvc.Device.Host, kvc.Device.GPU)
+        ran = _lib.last_launch()
+        assert np.array_equal(bits_of(dpool).reshape(L, nb, -1), gpu_np)
+        want_cap = cap_in if cap_in > 0 else cap_out
+        assert ran["kernel"] == _lib.KVC_KERNEL_COPY_TILES and 1 <= ran["grid"] <= want_cap
     finally:
         w.close()
 
