@@ -876,7 +876,21 @@ def bench_decode_step_graph(torch, kvc, wl, s8, pool, L, num_blocks, dev, steps=
     write_bytes_step = bytes_step
     rotary_bytes_step = L * B * (2 * Hq * D * 2 + 4 * H * D * 2 + 2 * D * 2 + 12)
 
+    # the floor of a graph node on this machine: L kernels that touch one element each
+    one = torch.zeros(1, device=dev)
+    floor_graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(floor_graph):
+        for _ in range(L):
+            one.add_(1.0)
+
+    def floor_replay(i):
+        floor_graph.replay()
+
     compact, detail = [], []
+    floor_wall, floor_dev = timed(floor_replay, steps)
+    detail.append({"name": f"cfg2 decode step: {L} one-element kernels replayed from a hipGraph (what a graph node costs "
+                           f"at least)", "wall_us_per_step": round(floor_wall, 1), "device_us_per_step": round(floor_dev, 1),
+                   "us_per_node": round(floor_dev / L, 2)})
     # `us` of these rows is WALL time per 32-layer step (what the serving loop pays)
     for fn, n, form, short, what in (
             (rotary_replay_only, steps, "step wall, graph, rotation fused", "graph{index+32 rotate+write}",
