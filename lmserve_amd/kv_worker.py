@@ -37,6 +37,7 @@ import asyncio
 import ctypes
 import enum
 import os
+import queue
 import time
 import warnings
 import weakref
@@ -622,15 +623,33 @@ class KVWorker:
             _lib.check(await asyncio.to_thread(lib.kvc_row_mover_wait, bounce.mover, ticket))
 
     async def _doorbell(self, doorbell, layer_idx: int) -> None:
-        """Take one token from `doorbell` (kv_worker.py:279-281 of the reference polls
-        the queue the same way), giving up after `host_wait_timeout`."""
+        """Take one token from `doorbell`, giving up after `host_wait_timeout`. A token
+        that is there is taken at once. Otherwise the wait blocks on the queue in a
+        helper thread, in slices of 50 ms so that a closing worker is not held up:
+        the reference polls with `asyncio.sleep(1e-5)` (kv_worker.py:279-281), which
+        an event loop on epoll rounds up to a millisecond per poll."""
+        try:
+            doorbell.get_nowait()
+            return
+        except queue.Empty:
+            pass
         deadline = None if self.host_wait_timeout is None else time.monotonic() + self.host_wait_timeout
-        while doorbell.empty():
-            if deadline is not None and time.monotonic() > deadline:
-                raise TimeoutError(f"no doorbell for layer {layer_idx} within {self.host_wait_timeout} s: "
-                                   "the model side has stopped posting layers")
-            await asyncio.sleep(1e-5)
-        doorbell.get()
+
+        def take() -> bool:
+            while True:
+                left = 0.05 if deadline is None else min(0.05, deadline - time.monotonic())
+                if left <= 0:
+                    return False
+                try:
+                    doorbell.get(True, left)
+                    return True
+                except queue.Empty:
+                    if getattr(self, "_closing", False):
+                        return False
+
+        if not await asyncio.to_thread(take):
+            raise TimeoutError(f"no doorbell for layer {layer_idx} within {self.host_wait_timeout} s: "
+                               "the model side has stopped posting layers")
 
     async def save_kv_blocks_to_host(self, block_mappings: Sequence[BlockMapping],
                                      stream: torch.cuda.Stream) -> None:
@@ -783,6 +802,7 @@ class KVWorker:
             self.load_kv_blocks_from_disk_sync(block_mappings)
 
     def close(self) -> None:
+        self._closing = True      # a doorbell wait in a helper thread ends at its next slice
         with torch.cuda.device(self.device):
             torch.cuda.synchronize()
         self.host_kv_caches_tensor = None
